@@ -1,0 +1,165 @@
+"""Benchmark of the TBIK hot path on ONE MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--table]
+
+A step is one tree-ordered matmul (`matmul_tp_persistent`) over the headline batch: X[2048,12288]
+(SiLU-gated synthetic activations, bf16) times the down_proj weight W[4096,12288] (N(0,0.02), bf16,
+stored [N,K] as nn.Linear does), inputs resident in HBM before the timed region.  Prints ONE JSON line.
+`--table` additionally prints (to stderr) the other shapes of the workload family: decode-sized M,
+simulated TP shards + combine, and the batch-invariant reductions.
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+M_, K_, N_ = 2048, 12288, 4096
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+
+
+def hip_time_ms(fn, steps, warmup):
+    """Average milliseconds per call, from HIP events on the stream the kernels are launched on."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    s.record()
+    for _ in range(steps):
+        fn()
+    e.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    return s.elapsed_time(e) / steps, wall_ms / steps
+
+
+def cpu_baseline(rows=512, repeats=3):
+    """The CPU oracle (PyTorch restatement of the reference's tree order) on the first `rows` rows of the
+    same workload, all host threads, median of `repeats` after one warm-up."""
+    import torch
+    from oracle import tbik_oracle as O
+    X = O.silu_gated_bf16((rows, K_), 0)
+    W = O.gaussian_bf16((N_, K_), 0.02, 1)
+    Wt = W.t()
+    O.matmul_tree(X[:64], Wt)
+    ts = []
+    for _ in range(repeats):
+        t0 = time.perf_counter()
+        O.matmul_tree(X, Wt)
+        ts.append(time.perf_counter() - t0)
+    t = statistics.median(ts)
+    return {"value": round(2.0 * rows * N_ * K_ / t / 1e12, 4), "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"oracle matmul_tree on the first {rows} of {M_} rows of the same X and W "
+                      f"(median of {repeats}, {t:.2f} s each)"}
+
+
+def table(steps, warmup):
+    import torch
+    from oracle import tbik_oracle as O
+    from llm_reproducibility_amd.bio import batch_invariant_ops as bio
+    from llm_reproducibility_amd.tbik import choose_leaf_k, matmul_tp_persistent, tree_combine
+    dev = torch.device("cuda:0")
+    rows = []
+
+    def gemm_row(name, M, K, N, leaf):
+        X = torch.randn((M, K), device=dev).to(torch.bfloat16)
+        W = (torch.randn((N, K), device=dev) * 0.02).to(torch.bfloat16)
+        ms, _ = hip_time_ms(lambda: matmul_tp_persistent(X, W.t(), leaf_k=leaf), steps, warmup)
+        fl, by = 2.0 * M * N * K, 2.0 * (M * K + K * N + M * N)
+        rows.append((name, ms * 1e3, fl / ms / 1e9, by / ms / 1e6))
+
+    for M in (1, 16, 128, 2048):
+        gemm_row(f"down_proj 8B  M={M} K=12288 N=4096", M, 12288, 4096, 256)
+    for p in (2, 4, 8):
+        gemm_row(f"  shard TP={p}  M=2048 K={12288 // p} N=4096", 2048, 12288 // p, 4096, 256)
+    for M in (1, 64, 512, 4096):
+        gemm_row(f"o_proj 32B    M={M} K=8192 N=5120", M, 8192, 5120, 256)
+    for M in (1, 64, 512, 4096):
+        gemm_row(f"down_proj 32B M={M} K=25600 N=5120 leaf128", M, 25600, 5120, choose_leaf_k(25600))
+    for p in (2, 4, 8):
+        parts = [torch.randn((2048, 4096), device=dev).to(torch.bfloat16) for _ in range(p)]
+        ms, _ = hip_time_ms(lambda: tree_combine(parts), steps, warmup)
+        rows.append((f"tree_combine p={p} [2048,4096]", ms * 1e3, 0.0, (p + 1) * 2048 * 4096 * 2 / ms / 1e6))
+    w = torch.ones(4096, device=dev, dtype=torch.bfloat16)
+    for r in (1, 7, 256, 4096):
+        x = torch.randn((r, 4096), device=dev).to(torch.bfloat16)
+        ms, _ = hip_time_ms(lambda: bio.rms_norm(x, w, 1e-6), steps, warmup)
+        rows.append((f"rmsnorm rows={r} hidden=4096", ms * 1e3, 0.0, (r * 4096 * 4 + 8192) / ms / 1e6))
+    for r in (1, 7, 256, 4096):
+        x = torch.randn((r, 151936), device=dev)
+        ms, _ = hip_time_ms(lambda: bio.log_softmax(x), max(steps // 4, 3), warmup)
+        rows.append((f"log_softmax rows={r} vocab=151936 (8 B/elem)", ms * 1e3, 0.0, r * 151936 * 8 / ms / 1e6))
+    for r in (1, 7, 256, 4096):
+        x = torch.randn((r, 4096), device=dev)
+        ms, _ = hip_time_ms(lambda: bio.mean_dim(x, -1), steps, warmup)
+        rows.append((f"mean rows={r} n=4096", ms * 1e3, 0.0, r * 4096 * 4 / ms / 1e6))
+    print(f"{'case':52s} {'us':>10s} {'TFLOP/s':>9s} {'%MFMA':>6s} {'GB/s':>9s} {'%HBM':>6s}", file=sys.stderr)
+    for name, us, tf, gbs in rows:
+        print(f"{name:52s} {us:10.1f} {tf:9.1f} {100 * tf / PEAK_BF16_TFLOPS:6.1f} {gbs:9.1f} {100 * gbs / PEAK_HBM_GBS:6.1f}",
+              file=sys.stderr)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--table", action="store_true", help="also print the per-shape table to stderr")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+
+    import torch
+    from llm_reproducibility_amd import _lib
+    from llm_reproducibility_amd.tbik import matmul_tp_persistent
+    from oracle import tbik_oracle as O
+
+    _lib.lib()
+    dev = torch.device("cuda:0")
+    X = O.silu_gated_bf16((M_, K_), 0).to(dev)
+    W = O.gaussian_bf16((N_, K_), 0.02, 1).to(dev)      # [N,K], K contiguous
+    Wt = W.t()
+    step = lambda: matmul_tp_persistent(X, Wt)          # noqa: E731
+    C = step()
+    # sanity inside the bench: TP invariance of what is being timed (not timed itself)
+    from llm_reproducibility_amd.tbik import tree_combine
+    parts = [matmul_tp_persistent(X[:, r * 3072:(r + 1) * 3072], W[:, r * 3072:(r + 1) * 3072].t()) for r in range(4)]
+    assert torch.equal(tree_combine(parts), C), "TP=4 result differs from TP=1"
+    del parts
+
+    ms, wall_ms = hip_time_ms(step, args.steps, args.warmup)
+    flops = 2.0 * M_ * N_ * K_
+    algo_bytes = 2.0 * (M_ * K_ + K_ * N_ + M_ * N_)
+    tflops = flops / (ms * 1e-3) / 1e12
+    out = {
+        "metric": "TBIK matmul TFLOP/s & % bf16 MFMA peak, M=2048 K=12288 N=4096",
+        "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "Qwen3-8B down_proj tree matmul X[2048,12288] x W[12288,4096] (configs[1], M=2048), leaf 256, TP=1",
+                   "M": M_, "K": K_, "N": N_, "leaf_k": 256},
+        "pct_bf16_mfma_peak": round(100 * tflops / PEAK_BF16_TFLOPS, 2),
+        "algorithmic_GBps": round(algo_bytes / (ms * 1e-3) / 1e9, 1),
+        "roofline": {"bound": "mfma", "achieved": round(tflops, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(tflops / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "kernel_avg_us": round(ms * 1e3, 2)},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline()
+    if args.table:
+        table(max(args.steps // 2, 5), max(args.warmup // 2, 2))
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,147 @@
+/*
+ * libtbik_hip.so -- C ABI of the MI355X (gfx950) tree-based invariant kernels.
+ *
+ * Every entry point
+ *   - takes plain device pointers, sizes and element strides (no torch types),
+ *   - enqueues its kernels on the caller's `stream` (a hipStream_t; NULL = the default stream),
+ *   - allocates nothing, synchronises nothing, keeps no mutable global state (re-entrant),
+ *   - validates shapes / alignment on the host BEFORE launching and returns a TBIK_* code
+ *     (0 = success); codes >= TBIK_ERR_HIP_BASE are TBIK_ERR_HIP_BASE + hipError_t.
+ *
+ * Each declaration cites the interface of the reference (nanomaoli/llm_reproducibility) that it
+ * replaces; paths are relative to the reference checkout.
+ */
+#ifndef TBIK_HIP_H
+#define TBIK_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TBIK_OK               0
+#define TBIK_ERR_INVALID      1   /* bad shape / null pointer / K not a whole number of leaves      */
+#define TBIK_ERR_ALIGNMENT    2   /* pointer or leading dimension not aligned for 16-byte accesses  */
+#define TBIK_ERR_UNSUPPORTED  3   /* layout or tree depth this build has no kernel for              */
+#define TBIK_ERR_WORKSPACE    4   /* workspace missing or too small                                 */
+#define TBIK_ERR_HIP_BASE     1000
+
+typedef void* tbik_stream_t;  /* hipStream_t */
+
+/* ABI version of this header (bumped when a signature changes). */
+int tbik_abi_version(void);
+
+/* Static text for a TBIK_* code. */
+const char* tbik_error_string(int code);
+
+/*
+ * Tree parameters of a K extent: T = K / leaf_k leaves, FLB = T with factors of two removed while
+ * even and > 2, LEVEL_K = halvings + 1.
+ * Replaces: the host arithmetic of matmul_tp_persistent, src/tbik/tree_based_matmul.py:242-249.
+ */
+int tbik_tree_params(int K, int leaf_k, int* T, int* flb, int* level_k);
+
+/*
+ * C[M,N] (bf16) = tree-ordered A[M,K] x B[K,N] (+ bias[N], added in bf16 after the tree).
+ * K is cut into leaves of leaf_k (256 = the reference's bf16 BLOCK_K; 128 is accepted for layers
+ * whose shards are not a multiple of 256).  Each leaf is accumulated in fp32 by a fixed chain of
+ * 16x16x32 bf16 MFMAs and rounded once to bf16; leaves are merged level 0 left-to-right over FLB
+ * leaves and then by an adjacent-pair binary tree, every node rounded to bf16.  The value of
+ * C[m,n] depends only on row m of A and column n of B -- not on M, N, the tile configuration or
+ * the launch.
+ *   A: element (m,k) at A[m*lda + k]                       (K contiguous)
+ *   B: element (k,n) at B[k*ldb_k + n*ldb_n]; ldb_k == 1   (the nn.Linear weight [N,K], i.e.
+ *      weight.t()) is the native layout; ldb_n == 1 (row-major [K,N]) returns
+ *      TBIK_ERR_UNSUPPORTED in this build and is repacked by the caller.
+ *   C: element (m,n) at C[m*ldc + n]
+ * Replaces: matmul_tp_persistent + matmul_kernel_tp_persistent,
+ *           src/tbik/tree_based_matmul.py:190-277 and :50-187.
+ */
+int tbik_gemm_bf16(const void* A, int64_t lda,
+                   const void* B, int64_t ldb_k, int64_t ldb_n,
+                   void* C, int64_t ldc,
+                   int M, int N, int K, int leaf_k,
+                   const void* bias_or_null,
+                   tbik_stream_t stream);
+
+/*
+ * out[i] = adjacent-pair binary tree over parts[0..nparts-1][i], bf16 adds (round to nearest even
+ * at every node); nparts in {1,2,4,8}; all buffers contiguous, numel elements, 2-byte aligned
+ * (16-byte aligned buffers take the vector path).  `out` may alias parts[0].
+ * Replaces: the local adds of tree_all_reduce_sum_native, src/tbik/tree_based_all_reduce.py:32-37,
+ *           simple_matmul.py:35-38, and packed_tree_reduce / custom_tree_all_reduce,
+ *           mini_allreduce/tbik_kernel/csrc/allreduce/custom_all_reduce.cuh:203-234, 301-312.
+ */
+int tbik_tree_combine_bf16(const void* const* parts, int nparts,
+                           void* out, int64_t numel,
+                           tbik_stream_t stream);
+
+/*
+ * C[M,N] (bf16) = A[M,K] x B[K,N] (+ bias[N] in fp32 before the single rounding), one fp32
+ * accumulator per element run strictly sequentially over K by the same MFMA chain for every M
+ * (batch invariant).  Layout rules as tbik_gemm_bf16; K only needs to be a multiple of 8.
+ * Replaces: matmul_persistent + matmul_kernel_persistent, src/bio/batch_invariant_ops.py:127-197
+ *           and :42-124 (aten::mm / aten::addmm overrides, :442-447).
+ */
+int bi_gemm_bf16(const void* A, int64_t lda,
+                 const void* B, int64_t ldb_k, int64_t ldb_n,
+                 void* C, int64_t ldc,
+                 int M, int N, int K,
+                 const void* bias_or_null,
+                 tbik_stream_t stream);
+
+/*
+ * RMSNorm over the last dimension, bf16 in/out, fp32 arithmetic, one wavefront per row in a fixed
+ * lane->element order (row i's result does not depend on `rows`):
+ *   x32 = x (+ residual);  residual_out = bf16(x32)          (only when residual != NULL)
+ *   out = bf16( bf16(x32 * rsqrt(mean(x32^2) + eps)) * weight )   (weight may be NULL)
+ * x/out/residual/residual_out have row stride ld* elements; hidden % 8 == 0.
+ * Replaces: patch_rms_norm -> vLLM RMSNorm.forward_native -> aten::mean.dim override,
+ *           src/patch/patch_batch_invariant.py:9-16, src/bio/batch_invariant_ops.py:459-472.
+ */
+int bi_rmsnorm_bf16(const void* x, int64_t ldx,
+                    const void* residual_or_null, int64_t ldr,
+                    const void* weight_or_null,
+                    void* out, int64_t ldo,
+                    void* residual_out_or_null, int64_t ldro,
+                    int64_t rows, int hidden, float eps,
+                    tbik_stream_t stream);
+
+/*
+ * Bytes of workspace bi_log_softmax_f32 needs for a [rows, cols] input.
+ */
+size_t bi_log_softmax_workspace_bytes(int64_t rows, int64_t cols);
+
+/*
+ * out[r, :] = x[r, :] - max - log(sum(exp(x[r, :] - max))), fp32, last dimension.
+ * Every row is cut into fixed 4096-element segments (a function of `cols` only); segment
+ * (max, sum) pairs go to `workspace` and are merged in segment order, so row r's result does not
+ * depend on `rows`.  `write_softmax` != 0 writes exp(log_softmax) instead.
+ * Replaces: log_softmax + _log_softmax_kernel, src/bio/batch_invariant_ops.py:263-301 and
+ *           :200-260 (aten::_log_softmax / aten::_softmax overrides, :450-456).
+ */
+int bi_log_softmax_f32(const void* x, int64_t ldx,
+                       void* out, int64_t ldo,
+                       int64_t rows, int64_t cols,
+                       void* workspace, size_t workspace_bytes,
+                       int write_softmax,
+                       tbik_stream_t stream);
+
+/*
+ * Mean over the middle dimension of a contiguous (outer, n, inner) view, fp32 accumulation in a
+ * fixed order that depends only on n and inner; dtype_code: 0 = fp32, 1 = bf16, 2 = fp16 (input
+ * and output share it).
+ * Replaces: mean_dim + mean_kernel, src/bio/batch_invariant_ops.py:352-439 and :304-349
+ *           (aten::mean.dim override, :459-472).
+ */
+int bi_mean_dim(const void* x, void* out,
+                int64_t outer, int64_t n, int64_t inner,
+                int dtype_code,
+                tbik_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TBIK_HIP_H */

@@ -1,0 +1,83 @@
+"""ctypes binding of libtbik_hip.so (declared in include/tbik_hip.h).
+
+The library is the only compute path of this package: if it is missing, loading fails with an error
+that says how to build it -- there is no eager / CPU fallback.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+_PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG_DIR, "libtbik_hip.so")
+
+TBIK_OK = 0
+TBIK_ERR_INVALID = 1
+TBIK_ERR_ALIGNMENT = 2
+TBIK_ERR_UNSUPPORTED = 3
+TBIK_ERR_WORKSPACE = 4
+
+EXPORTS = (
+    "tbik_abi_version", "tbik_error_string", "tbik_tree_params", "tbik_gemm_bf16", "tbik_tree_combine_bf16",
+    "bi_gemm_bf16", "bi_rmsnorm_bf16", "bi_log_softmax_workspace_bytes", "bi_log_softmax_f32", "bi_mean_dim",
+)
+
+_lib = None
+
+
+class TbikError(RuntimeError):
+    def __init__(self, code: int, where: str):
+        self.code = code
+        msg = lib().tbik_error_string(code).decode()
+        super().__init__(f"{where}: {msg} (code {code})")
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: the HIP kernels are the only implementation of this package. "
+            "Build them with `python -m llm_reproducibility_amd.build` (needs hipcc).")
+    L = ctypes.CDLL(LIB_PATH)
+    i32, i64, vp, sz, f32 = ctypes.c_int, ctypes.c_int64, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_float
+    pi32 = ctypes.POINTER(ctypes.c_int)
+    L.tbik_abi_version.argtypes = []
+    L.tbik_abi_version.restype = i32
+    L.tbik_error_string.argtypes = [i32]
+    L.tbik_error_string.restype = ctypes.c_char_p
+    L.tbik_tree_params.argtypes = [i32, i32, pi32, pi32, pi32]
+    L.tbik_tree_params.restype = i32
+    L.tbik_gemm_bf16.argtypes = [vp, i64, vp, i64, i64, vp, i64, i32, i32, i32, i32, vp, vp]
+    L.tbik_gemm_bf16.restype = i32
+    L.tbik_tree_combine_bf16.argtypes = [ctypes.POINTER(vp), i32, vp, i64, vp]
+    L.tbik_tree_combine_bf16.restype = i32
+    L.bi_gemm_bf16.argtypes = [vp, i64, vp, i64, i64, vp, i64, i32, i32, i32, vp, vp]
+    L.bi_gemm_bf16.restype = i32
+    L.bi_rmsnorm_bf16.argtypes = [vp, i64, vp, i64, vp, vp, i64, vp, i64, i64, i32, f32, vp]
+    L.bi_rmsnorm_bf16.restype = i32
+    L.bi_log_softmax_workspace_bytes.argtypes = [i64, i64]
+    L.bi_log_softmax_workspace_bytes.restype = sz
+    L.bi_log_softmax_f32.argtypes = [vp, i64, vp, i64, i64, i64, vp, sz, i32, vp]
+    L.bi_log_softmax_f32.restype = i32
+    L.bi_mean_dim.argtypes = [vp, vp, i64, i64, i64, i32, vp]
+    L.bi_mean_dim.restype = i32
+    if L.tbik_abi_version() != 1:
+        raise RuntimeError(f"{LIB_PATH}: ABI version {L.tbik_abi_version()} does not match this package (1)")
+    _lib = L
+    return L
+
+
+def check(code: int, where: str) -> None:
+    if code != TBIK_OK:
+        raise TbikError(code, where)
+
+
+def tree_params(K: int, leaf_k: int):
+    """(T, FLB, LEVEL_K) of a K extent; ValueError if K is not a whole number of leaves."""
+    t, f, l = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    rc = lib().tbik_tree_params(int(K), int(leaf_k), ctypes.byref(t), ctypes.byref(f), ctypes.byref(l))
+    if rc != TBIK_OK:
+        raise ValueError(f"K={K} is not a whole number of leaves of {leaf_k}")
+    return t.value, f.value, l.value

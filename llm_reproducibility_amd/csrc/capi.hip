@@ -1,0 +1,80 @@
+// extern "C" surface of libtbik_hip.so (declared in include/tbik_hip.h): argument checks live in the
+// dispatchers next to each kernel, this file only binds names.
+#include "common.h"
+
+namespace tbik {
+int gemm_dispatch(bool tree, const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C,
+                  int64_t ldc, int M, int N, int K, int leaf_k, const void* bias, hipStream_t stream);
+int tree_combine_dispatch(const void* const* parts, int nparts, void* out, int64_t numel, hipStream_t stream);
+int rmsnorm_dispatch(const void* x, int64_t ldx, const void* res, int64_t ldr, const void* w, void* out, int64_t ldo,
+                     void* res_out, int64_t ldro, int64_t rows, int hidden, float eps, hipStream_t stream);
+size_t lsm_workspace_bytes(int64_t rows, int64_t cols);
+int log_softmax_dispatch(const void* x, int64_t ldx, void* out, int64_t ldo, int64_t rows, int64_t cols, void* ws,
+                         size_t ws_bytes, int write_softmax, hipStream_t stream);
+int mean_dispatch(const void* x, void* out, int64_t outer, int64_t n, int64_t inner, int dtype_code, hipStream_t stream);
+}  // namespace tbik
+
+extern "C" {
+
+int tbik_abi_version(void) { return 1; }
+
+const char* tbik_error_string(int code) {
+  switch (code) {
+    case TBIK_OK: return "ok";
+    case TBIK_ERR_INVALID: return "invalid argument (shape, null pointer, or K not a whole number of leaves)";
+    case TBIK_ERR_ALIGNMENT: return "pointer or leading dimension not aligned for 16-byte accesses";
+    case TBIK_ERR_UNSUPPORTED: return "layout, dtype or tree depth not supported by this build";
+    case TBIK_ERR_WORKSPACE: return "workspace missing or too small";
+    default: return code >= TBIK_ERR_HIP_BASE ? hipGetErrorString((hipError_t)(code - TBIK_ERR_HIP_BASE)) : "unknown";
+  }
+}
+
+int tbik_tree_params(int K, int leaf_k, int* T, int* flb, int* level_k) {
+  if (K <= 0 || leaf_k <= 0 || K % leaf_k != 0 || !T || !flb || !level_k) return TBIK_ERR_INVALID;
+  int t = K / leaf_k, f = t, l = 1;
+  while (f > 2 && (f & 1) == 0) {
+    f >>= 1;
+    l++;
+  }
+  *T = t;
+  *flb = f;
+  *level_k = l;
+  return TBIK_OK;
+}
+
+int tbik_gemm_bf16(const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C, int64_t ldc, int M,
+                   int N, int K, int leaf_k, const void* bias_or_null, tbik_stream_t stream) {
+  return tbik::gemm_dispatch(true, A, lda, B, ldb_k, ldb_n, C, ldc, M, N, K, leaf_k, bias_or_null,
+                             static_cast<hipStream_t>(stream));
+}
+
+int tbik_tree_combine_bf16(const void* const* parts, int nparts, void* out, int64_t numel, tbik_stream_t stream) {
+  return tbik::tree_combine_dispatch(parts, nparts, out, numel, static_cast<hipStream_t>(stream));
+}
+
+int bi_gemm_bf16(const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C, int64_t ldc, int M,
+                 int N, int K, const void* bias_or_null, tbik_stream_t stream) {
+  return tbik::gemm_dispatch(false, A, lda, B, ldb_k, ldb_n, C, ldc, M, N, K, 0, bias_or_null,
+                             static_cast<hipStream_t>(stream));
+}
+
+int bi_rmsnorm_bf16(const void* x, int64_t ldx, const void* residual_or_null, int64_t ldr, const void* weight_or_null,
+                    void* out, int64_t ldo, void* residual_out_or_null, int64_t ldro, int64_t rows, int hidden, float eps,
+                    tbik_stream_t stream) {
+  return tbik::rmsnorm_dispatch(x, ldx, residual_or_null, ldr, weight_or_null, out, ldo, residual_out_or_null, ldro, rows,
+                                hidden, eps, static_cast<hipStream_t>(stream));
+}
+
+size_t bi_log_softmax_workspace_bytes(int64_t rows, int64_t cols) { return tbik::lsm_workspace_bytes(rows, cols); }
+
+int bi_log_softmax_f32(const void* x, int64_t ldx, void* out, int64_t ldo, int64_t rows, int64_t cols, void* workspace,
+                       size_t workspace_bytes, int write_softmax, tbik_stream_t stream) {
+  return tbik::log_softmax_dispatch(x, ldx, out, ldo, rows, cols, workspace, workspace_bytes, write_softmax,
+                                    static_cast<hipStream_t>(stream));
+}
+
+int bi_mean_dim(const void* x, void* out, int64_t outer, int64_t n, int64_t inner, int dtype_code, tbik_stream_t stream) {
+  return tbik::mean_dispatch(x, out, outer, n, inner, dtype_code, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,355 @@
+// Tiled bf16 MFMA GEMM for gfx950 with two accumulation disciplines:
+//
+//   TREE = true   tree-ordered (TP-invariant) GEMM.  K is cut into leaves of LS*64 elements; a leaf is
+//                 a chain of 16x16x32 bf16 MFMAs into a zeroed fp32 accumulator, rounded once to bf16;
+//                 leaves merge through a binary-counter stack of packed-bf16 partials held in registers
+//                 (level 0: left-to-right over FLB leaves, levels above: adjacent pairs), every node
+//                 rounded to bf16.  Replaces matmul_kernel_tp_persistent,
+//                 src/tbik/tree_based_matmul.py:50-187 of the reference.
+//   TREE = false  one fp32 accumulator per element run sequentially over all of K (batch-invariant mm),
+//                 replaces matmul_kernel_persistent, src/bio/batch_invariant_ops.py:42-124.
+//
+// Invariance argument: the value of C[m,n] is produced by ONE lane's accumulator registers from the
+// k-ordered MFMA chain on row m of A and row n of W; tile sizes, wave placement, padding rows and
+// the block->tile map only decide WHICH lane does it.  All tile configurations therefore give the
+// same bits, and row m never sees M.
+//
+// Operand roles: W ([N,K], K contiguous) feeds the MFMA "A" port and X ([M,K]) the "B" port, so an
+// output lane holds 4 consecutive n of one m and stores them as one 8-byte word.
+#include "common.h"
+
+namespace tbik {
+
+struct GemmArgs {
+  const uint16_t* X;   // [M,K], row stride ldx
+  const uint16_t* W;   // [N,K], row stride ldw
+  uint16_t* C;         // [M,N], row stride ldc
+  const uint16_t* bias;
+  int64_t ldx, ldw, ldc;
+  int M, N, K;
+  int T;      // leaves (TREE)
+  int flb;    // leaves summed left to right at level 0
+  int lb;     // binary levels above level 0
+  int vec_store;  // C rows allow 8-byte stores
+};
+
+constexpr int BK = 64;  // K elements per LDS stage (8 chunks of 16 bytes per row)
+
+// Element offset of 16-byte chunk `c` (0..7) of tile row `r` in an LDS tile of 64-element rows.
+// The XOR spreads the 16 rows an MFMA fragment read touches over all banks.
+__device__ __forceinline__ int lds_off(int r, int c) { return r * BK + ((c ^ (r & 7)) << 3); }
+
+template <int WAVES_M, int WAVES_N, int TM, int TN, int LS, int LBMAX, bool TREE>
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmArgs p) {
+  constexpr int NT = WAVES_M * WAVES_N * 64;
+  constexpr int BM = WAVES_M * TM * 16;
+  constexpr int BN = WAVES_N * TN * 16;
+  constexpr int XCH = (BM * 8 + NT - 1) / NT;  // 16-byte chunks of the X tile per thread
+  constexpr int WCH = (BN * 8 + NT - 1) / NT;
+
+  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+  constexpr int STAGE = (BM + BN) * BK;  // elements per LDS stage: X tile, then W tile
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave / WAVES_N;
+  const int wn = wave % WAVES_N;
+
+  // ---- block -> tile: consecutive logical ids stay on one XCD (blocks are dealt round-robin over the
+  // 8 XCDs), and walk the tile grid in bands of 8 m-tiles so an XCD's L2 sees few distinct panels.
+  const int tiles_m = (p.M + BM - 1) / BM;
+  const int tiles_n = (p.N + BN - 1) / BN;
+  int lid = blockIdx.x;
+  {
+    const int nwg = gridDim.x;
+    if ((nwg & 7) == 0) lid = (lid & 7) * (nwg >> 3) + (lid >> 3);
+  }
+  constexpr int GROUP = 8;
+  const int per_group = GROUP * tiles_n;
+  const int group_id = lid / per_group;
+  const int first_m = group_id * GROUP;
+  const int gsz = min(tiles_m - first_m, GROUP);
+  const int pid_m = first_m + (lid % per_group) % gsz;
+  const int pid_n = (lid % per_group) / gsz;
+  const int m0 = pid_m * BM;
+  const int n0 = pid_n * BN;
+
+  // ---- global -> register staging (rows past the edge are clamped: their results are never stored)
+  const uint16_t* xptr[XCH];
+  const uint16_t* wptr[WCH];
+  int xdst[XCH], wdst[WCH];
+#pragma unroll
+  for (int i = 0; i < XCH; i++) {
+    const int q = tid + i * NT;
+    const int r = (q >> 3) % BM, c = q & 7;
+    const int gr = min(m0 + r, p.M - 1);
+    xptr[i] = p.X + (int64_t)gr * p.ldx + c * 8;
+    xdst[i] = lds_off(r, c);
+  }
+#pragma unroll
+  for (int i = 0; i < WCH; i++) {
+    const int q = tid + i * NT;
+    const int r = (q >> 3) % BN, c = q & 7;
+    const int gr = min(n0 + r, p.N - 1);
+    wptr[i] = p.W + (int64_t)gr * p.ldw + c * 8;
+    wdst[i] = lds_off(r, c);
+  }
+  u32x4 xreg[XCH], wreg[WCH];
+
+  auto load_stage = [&](int s) __attribute__((always_inline)) {
+    const int k0 = s * BK;
+#pragma unroll
+    for (int i = 0; i < XCH; i++) {
+      if ((BM * 8) % NT == 0 || tid + i * NT < BM * 8) {
+        if (TREE || k0 + (tid & 7) * 8 < p.K)
+          xreg[i] = *reinterpret_cast<const u32x4*>(xptr[i] + k0);
+        else
+          xreg[i] = u32x4{0, 0, 0, 0};
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < WCH; i++) {
+      if ((BN * 8) % NT == 0 || tid + i * NT < BN * 8) {
+        if (TREE || k0 + (tid & 7) * 8 < p.K)
+          wreg[i] = *reinterpret_cast<const u32x4*>(wptr[i] + k0);
+        else
+          wreg[i] = u32x4{0, 0, 0, 0};
+      }
+    }
+  };
+  auto store_stage = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < XCH; i++)
+      if ((BM * 8) % NT == 0 || tid + i * NT < BM * 8) *reinterpret_cast<u32x4*>(smem + buf * STAGE + xdst[i]) = xreg[i];
+#pragma unroll
+    for (int i = 0; i < WCH; i++)
+      if ((BN * 8) % NT == 0 || tid + i * NT < BN * 8) *reinterpret_cast<u32x4*>(smem + buf * STAGE + BM * BK + wdst[i]) = wreg[i];
+  };
+
+  // ---- fragment addressing: lane l reads row (l%16), 16-byte chunk kk*4 + l/16
+  const int frow = lane & 15;
+  const int fchk = lane >> 4;
+
+  f32x4 acc[TM][TN];
+  uint32_t t[TM][TN][2];                 // current node, packed bf16 (n, n+1), (n+2, n+3)
+  uint32_t s0[TM][TN][2];                // level 0: running left-to-right sum
+  uint32_t sb[LBMAX > 0 ? LBMAX : 1][TM][TN][2];  // binary levels
+  int c0 = 0;                            // leaves absorbed at level 0
+  int g = 0;                             // groups completed (binary counter)
+
+  const int nstages = TREE ? p.T * LS : (p.K + BK - 1) / BK;
+  const int nouter = TREE ? p.T : (nstages + LS - 1) / LS;
+
+  load_stage(0);
+  store_stage(0);
+  __syncthreads();
+
+  for (int j = 0; j < nouter; j++) {
+#pragma unroll
+    for (int i = 0; i < LS; i++) {
+      const int s = j * LS + i;
+      if (TREE || s < nstages) {
+        // the stage after the last one re-reads the last one into the idle buffer: harmless, and it
+        // keeps the staging registers free of control flow
+        load_stage(min(s + 1, nstages - 1));
+        const uint16_t* bx = smem + (s & 1) * STAGE;
+        const uint16_t* bw = bx + BM * BK;
+#pragma unroll
+        for (int kk = 0; kk < 2; kk++) {
+          bf16x8 fx[TM], fw[TN];
+#pragma unroll
+          for (int a = 0; a < TM; a++) {
+            const int r = (wm * TM + a) * 16 + frow;
+            fx[a] = *reinterpret_cast<const bf16x8*>(bx + lds_off(r, kk * 4 + fchk));
+          }
+#pragma unroll
+          for (int b = 0; b < TN; b++) {
+            const int r = (wn * TN + b) * 16 + frow;
+            fw[b] = *reinterpret_cast<const bf16x8*>(bw + lds_off(r, kk * 4 + fchk));
+          }
+          const bool fresh = (i == 0 && kk == 0) && (TREE || j == 0);
+#pragma unroll
+          for (int a = 0; a < TM; a++)
+#pragma unroll
+            for (int b = 0; b < TN; b++) {
+              const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+              acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[b], fx[a], fresh ? zero : acc[a][b], 0, 0, 0);
+            }
+        }
+        store_stage((s + 1) & 1);
+        __syncthreads();
+      }
+    }
+    if (TREE) {
+      // leaf -> bf16, then the binary-counter merge (all conditions are uniform over the block)
+#pragma unroll
+      for (int a = 0; a < TM; a++)
+#pragma unroll
+        for (int b = 0; b < TN; b++) {
+          t[a][b][0] = pack_bf16x2(acc[a][b][0], acc[a][b][1]);
+          t[a][b][1] = pack_bf16x2(acc[a][b][2], acc[a][b][3]);
+        }
+      if (c0 != 0) {
+#pragma unroll
+        for (int a = 0; a < TM; a++)
+#pragma unroll
+          for (int b = 0; b < TN; b++) {
+            t[a][b][0] = add_bf16x2(s0[a][b][0], t[a][b][0]);
+            t[a][b][1] = add_bf16x2(s0[a][b][1], t[a][b][1]);
+          }
+      }
+      c0++;
+      if (c0 == p.flb) {
+        c0 = 0;
+        bool parked = false;
+#pragma unroll
+        for (int l = 0; l < LBMAX; l++) {
+          if (!parked && l < p.lb) {
+            if ((g >> l) & 1) {
+#pragma unroll
+              for (int a = 0; a < TM; a++)
+#pragma unroll
+                for (int b = 0; b < TN; b++) {
+                  t[a][b][0] = add_bf16x2(sb[l][a][b][0], t[a][b][0]);
+                  t[a][b][1] = add_bf16x2(sb[l][a][b][1], t[a][b][1]);
+                }
+            } else {
+#pragma unroll
+              for (int a = 0; a < TM; a++)
+#pragma unroll
+                for (int b = 0; b < TN; b++) {
+                  sb[l][a][b][0] = t[a][b][0];
+                  sb[l][a][b][1] = t[a][b][1];
+                }
+              parked = true;
+            }
+          }
+        }
+        g++;
+      } else {
+#pragma unroll
+        for (int a = 0; a < TM; a++)
+#pragma unroll
+          for (int b = 0; b < TN; b++) {
+            s0[a][b][0] = t[a][b][0];
+            s0[a][b][1] = t[a][b][1];
+          }
+      }
+    }
+  }
+
+  // ---- epilogue: (bias in fp32 for the single-accumulator GEMM, in bf16 after the tree), store
+#pragma unroll
+  for (int a = 0; a < TM; a++) {
+    const int m = m0 + (wm * TM + a) * 16 + frow;
+#pragma unroll
+    for (int b = 0; b < TN; b++) {
+      const int n = n0 + (wn * TN + b) * 16 + fchk * 4;
+      if (m >= p.M || n >= p.N) continue;
+      uint32_t lo, hi;
+      float bv[4] = {0.f, 0.f, 0.f, 0.f};
+      if (p.bias) {
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+          if (n + e < p.N) bv[e] = bf16_bits_to_f32(p.bias[n + e]);
+      }
+      if (TREE) {
+        lo = t[a][b][0];
+        hi = t[a][b][1];
+        if (p.bias) {
+          lo = add_bf16x2(lo, pack_bf16x2(bv[0], bv[1]));
+          hi = add_bf16x2(hi, pack_bf16x2(bv[2], bv[3]));
+        }
+      } else {
+        lo = pack_bf16x2(acc[a][b][0] + bv[0], acc[a][b][1] + bv[1]);
+        hi = pack_bf16x2(acc[a][b][2] + bv[2], acc[a][b][3] + bv[3]);
+      }
+      uint16_t* dst = p.C + (int64_t)m * p.ldc + n;
+      if (p.vec_store && n + 3 < p.N) {
+        *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);
+      } else {
+        const uint16_t v[4] = {(uint16_t)(lo & 0xffff), (uint16_t)(lo >> 16), (uint16_t)(hi & 0xffff), (uint16_t)(hi >> 16)};
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+          if (n + e < p.N) dst[e] = v[e];
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// host side
+// ------------------------------------------------------------------------------------------------
+template <int WAVES_M, int WAVES_N, int TM, int TN, int LS, int LBMAX, bool TREE>
+static int launch(const GemmArgs& a, hipStream_t stream) {
+  constexpr int NT = WAVES_M * WAVES_N * 64;
+  constexpr int BM = WAVES_M * TM * 16;
+  constexpr int BN = WAVES_N * TN * 16;
+  constexpr size_t smem = (size_t)2 * (BM + BN) * BK * sizeof(uint16_t);
+  auto kern = gemm_kernel<WAVES_M, WAVES_N, TM, TN, LS, LBMAX, TREE>;
+  if (smem > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return hip_code(e);
+  }
+  const int64_t tiles = (int64_t)((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
+  if (tiles <= 0 || tiles > 0x7fffffff) return TBIK_ERR_INVALID;
+  hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(NT), smem, stream, a);
+  return hip_code(hipGetLastError());
+}
+
+template <int LS, int LBMAX, bool TREE>
+static int launch_by_m(const GemmArgs& a, hipStream_t stream) {
+  if (a.M <= 16) return launch<1, 4, 1, 1, LS, LBMAX, TREE>(a, stream);
+  if (a.M <= 64) return launch<1, 4, 4, 2, LS, LBMAX, TREE>(a, stream);
+  return launch<2, 2, 4, 4, LS, LBMAX, TREE>(a, stream);
+}
+
+template <int LS>
+static int launch_tree(const GemmArgs& a, hipStream_t stream) {
+  if (a.lb <= 2) return launch_by_m<LS, 2, true>(a, stream);
+  if (a.lb <= 4) return launch_by_m<LS, 4, true>(a, stream);
+  if (a.lb <= 6) return launch_by_m<LS, 6, true>(a, stream);
+  return TBIK_ERR_UNSUPPORTED;
+}
+
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+int gemm_dispatch(bool tree, const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C,
+                  int64_t ldc, int M, int N, int K, int leaf_k, const void* bias, hipStream_t stream) {
+  if (!A || !B || !C || M < 0 || N < 0 || K <= 0) return TBIK_ERR_INVALID;
+  if (M == 0 || N == 0) return TBIK_OK;
+  if (ldb_k != 1) return TBIK_ERR_UNSUPPORTED;  // row-major [K,N] weights are repacked by the caller
+  if (lda < K || ldb_n < K || ldc < N) return TBIK_ERR_INVALID;
+  if (!aligned16(A) || !aligned16(B) || (lda & 7) || (ldb_n & 7) || (K & 7)) return TBIK_ERR_ALIGNMENT;
+  if (reinterpret_cast<uintptr_t>(C) & 1) return TBIK_ERR_ALIGNMENT;
+
+  GemmArgs a;
+  a.X = static_cast<const uint16_t*>(A);
+  a.W = static_cast<const uint16_t*>(B);
+  a.C = static_cast<uint16_t*>(C);
+  a.bias = static_cast<const uint16_t*>(bias);
+  a.ldx = lda;
+  a.ldw = ldb_n;
+  a.ldc = ldc;
+  a.M = M;
+  a.N = N;
+  a.K = K;
+  a.T = 0;
+  a.flb = 1;
+  a.lb = 0;
+  a.vec_store = ((reinterpret_cast<uintptr_t>(C) & 7) == 0 && (ldc & 3) == 0) ? 1 : 0;
+  if (!tree) return launch_by_m<4, 0, false>(a, stream);
+
+  int T, flb, level_k;
+  if (tbik_tree_params(K, leaf_k, &T, &flb, &level_k) != TBIK_OK) return TBIK_ERR_INVALID;
+  a.T = T;
+  a.flb = flb;
+  a.lb = level_k - 1;
+  if (leaf_k == 256) return launch_tree<4>(a, stream);
+  if (leaf_k == 128) return launch_tree<2>(a, stream);
+  return TBIK_ERR_UNSUPPORTED;
+}
+
+}  // namespace tbik

@@ -1,0 +1,108 @@
+// Shard combine: out[i] = adjacent-pair binary tree over up to 8 bf16 partials, every node rounded to
+// bf16.  This is the arithmetic of the reference's cross-GPU tree all-reduce
+// (src/tbik/tree_based_all_reduce.py:32-37; packed_tree_reduce,
+// mini_allreduce/tbik_kernel/csrc/allreduce/custom_all_reduce.cuh:203-234) applied to partials that
+// already sit in one GPU's memory.  HBM bound: (nparts + 1) * numel * 2 bytes.
+#include "common.h"
+
+namespace tbik {
+
+struct CombineArgs {
+  const uint16_t* parts[8];
+  uint16_t* out;
+  int64_t numel;
+};
+
+template <int NP>
+__device__ __forceinline__ uint32_t tree_node(const uint32_t (&v)[8]) {
+  uint32_t w[8];
+#pragma unroll
+  for (int i = 0; i < NP; i++) w[i] = v[i];
+#pragma unroll
+  for (int step = 1; step < NP; step <<= 1)
+#pragma unroll
+    for (int left = 0; left < NP; left += 2 * step) w[left] = add_bf16x2(w[left], w[left + step]);
+  return w[0];
+}
+
+// One thread per 16-byte pack (8 bf16); grid-stride so any numel fits one launch.
+template <int NP>
+__global__ __launch_bounds__(256) void combine_vec_kernel(const CombineArgs a, int64_t npacks) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < npacks; i += stride) {
+    uint4 in[NP];
+#pragma unroll
+    for (int p = 0; p < NP; p++) in[p] = reinterpret_cast<const uint4*>(a.parts[p])[i];
+    uint4 o;
+    uint32_t v[8];
+#pragma unroll
+    for (int p = 0; p < NP; p++) v[p] = in[p].x;
+    o.x = tree_node<NP>(v);
+#pragma unroll
+    for (int p = 0; p < NP; p++) v[p] = in[p].y;
+    o.y = tree_node<NP>(v);
+#pragma unroll
+    for (int p = 0; p < NP; p++) v[p] = in[p].z;
+    o.z = tree_node<NP>(v);
+#pragma unroll
+    for (int p = 0; p < NP; p++) v[p] = in[p].w;
+    o.w = tree_node<NP>(v);
+    reinterpret_cast<uint4*>(a.out)[i] = o;
+  }
+}
+
+// Scalar path for the tail and for buffers that are not 16-byte aligned.
+template <int NP>
+__global__ __launch_bounds__(256) void combine_scalar_kernel(const CombineArgs a, int64_t begin) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = begin + (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < a.numel; i += stride) {
+    uint32_t v[8];
+#pragma unroll
+    for (int p = 0; p < NP; p++) v[p] = a.parts[p][i];
+    a.out[i] = (uint16_t)(tree_node<NP>(v) & 0xffffu);
+  }
+}
+
+template <int NP>
+static int launch_combine(const CombineArgs& a, bool vec_ok, hipStream_t stream) {
+  const int64_t npacks = vec_ok ? a.numel / 8 : 0;
+  if (npacks > 0) {
+    const int64_t blocks = (npacks + 255) / 256;
+    const unsigned grid = (unsigned)(blocks < 8192 ? blocks : 8192);
+    hipLaunchKernelGGL(combine_vec_kernel<NP>, dim3(grid), dim3(256), 0, stream, a, npacks);
+  }
+  const int64_t begin = npacks * 8;
+  if (begin < a.numel) {
+    const int64_t rest = a.numel - begin;
+    const int64_t blocks = (rest + 255) / 256;
+    const unsigned grid = (unsigned)(blocks < 8192 ? blocks : 8192);
+    hipLaunchKernelGGL(combine_scalar_kernel<NP>, dim3(grid), dim3(256), 0, stream, a, begin);
+  }
+  return hip_code(hipGetLastError());
+}
+
+int tree_combine_dispatch(const void* const* parts, int nparts, void* out, int64_t numel, hipStream_t stream) {
+  if (!parts || !out || numel < 0) return TBIK_ERR_INVALID;
+  if (nparts != 1 && nparts != 2 && nparts != 4 && nparts != 8) return TBIK_ERR_INVALID;
+  if (numel == 0) return TBIK_OK;
+  CombineArgs a;
+  bool vec_ok = (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+  if (reinterpret_cast<uintptr_t>(out) & 1) return TBIK_ERR_ALIGNMENT;
+  for (int p = 0; p < 8; p++) a.parts[p] = nullptr;
+  for (int p = 0; p < nparts; p++) {
+    if (!parts[p]) return TBIK_ERR_INVALID;
+    if (reinterpret_cast<uintptr_t>(parts[p]) & 1) return TBIK_ERR_ALIGNMENT;
+    vec_ok = vec_ok && (reinterpret_cast<uintptr_t>(parts[p]) & 15) == 0;
+    a.parts[p] = static_cast<const uint16_t*>(parts[p]);
+  }
+  a.out = static_cast<uint16_t*>(out);
+  a.numel = numel;
+  switch (nparts) {
+    case 1: return launch_combine<1>(a, vec_ok, stream);
+    case 2: return launch_combine<2>(a, vec_ok, stream);
+    case 4: return launch_combine<4>(a, vec_ok, stream);
+    default: return launch_combine<8>(a, vec_ok, stream);
+  }
+}
+
+}  // namespace tbik

@@ -1,0 +1,209 @@
+"""Torch custom ops over the C ABI of libtbik_hip.so.
+
+Each op allocates its output with torch, passes raw device pointers, element strides and the current
+HIP stream to one `extern "C"` entry point, and raises on a non-zero return code.  The ops are
+registered for the GPU device type only: calling them on CPU tensors raises -- there is no CPU path.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import List, Optional
+
+import torch
+
+from . import _lib
+
+_DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _require_gpu(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("tbik ops run on the GPU only (HIP kernels); got a tensor on " + str(t.device))
+
+
+def _aligned16(t: torch.Tensor) -> bool:
+    return t.data_ptr() % 16 == 0
+
+
+def _rows16(t: torch.Tensor):
+    """(tensor, leading dimension) with a contiguous last dim and 16-byte aligned rows; copies if needed."""
+    ok = t.stride(1) == 1 and _aligned16(t) and t.shape[1] % 8 == 0
+    if ok and t.shape[0] == 1:
+        return t, t.shape[1]
+    if ok and t.stride(0) >= t.shape[1] and t.stride(0) % 8 == 0:
+        return t, t.stride(0)
+    c = t.contiguous()
+    if not _aligned16(c):
+        c = c.clone()
+    return c, c.shape[1]
+
+
+def _weight_nk(B: torch.Tensor):
+    """The [N,K] K-contiguous form of a [K,N] operand (the nn.Linear weight layout) and its leading
+    dimension; `weight.t()` is used as it is, a row-major [K,N] operand is repacked."""
+    return _rows16(B.t())
+
+
+# --------------------------------------------------------------------------------------------
+# tree-ordered GEMM
+# --------------------------------------------------------------------------------------------
+@torch.library.custom_op("tbik::gemm_tree_bf16", mutates_args=(), device_types="cuda")
+def gemm_tree_bf16(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.Tensor], leaf_k: int) -> torch.Tensor:
+    _require_gpu(A, B, bias)
+    M, K = A.shape
+    N = B.shape[1]
+    a, lda = _rows16(A)
+    w, ldw = _weight_nk(B)
+    b = None if bias is None else bias.contiguous()
+    C = torch.empty((M, N), device=A.device, dtype=torch.bfloat16)
+    rc = _lib.lib().tbik_gemm_bf16(a.data_ptr(), lda, w.data_ptr(), 1, ldw, C.data_ptr(), C.stride(0),
+                                   M, N, K, leaf_k, None if b is None else b.data_ptr(), _stream(A))
+    _lib.check(rc, "tbik_gemm_bf16")
+    return C
+
+
+@gemm_tree_bf16.register_fake
+def _(A, B, bias, leaf_k):
+    return A.new_empty((A.shape[0], B.shape[1]))
+
+
+@torch.library.custom_op("tbik::tree_combine_bf16", mutates_args=(), device_types="cuda")
+def tree_combine_bf16(parts: List[torch.Tensor]) -> torch.Tensor:
+    _require_gpu(*parts)
+    ps = [p.contiguous() for p in parts]
+    out = torch.empty_like(ps[0])
+    arr = (ctypes.c_void_p * len(ps))(*[p.data_ptr() for p in ps])
+    rc = _lib.lib().tbik_tree_combine_bf16(arr, len(ps), out.data_ptr(), out.numel(), _stream(out))
+    _lib.check(rc, "tbik_tree_combine_bf16")
+    return out
+
+
+@tree_combine_bf16.register_fake
+def _(parts):
+    return torch.empty_like(parts[0])
+
+
+# --------------------------------------------------------------------------------------------
+# batch-invariant ops
+# --------------------------------------------------------------------------------------------
+@torch.library.custom_op("tbik::bi_gemm_bf16", mutates_args=(), device_types="cuda")
+def bi_gemm_bf16(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
+    _require_gpu(A, B, bias)
+    M, K = A.shape
+    N = B.shape[1]
+    if K % 8 != 0:
+        # zero columns do not change a sequential fp32 accumulation
+        pad = (-K) % 8
+        A = torch.nn.functional.pad(A, (0, pad))
+        B = torch.nn.functional.pad(B, (0, 0, 0, pad))
+        K += pad
+    a, lda = _rows16(A)
+    w, ldw = _weight_nk(B)
+    b = None if bias is None else bias.contiguous()
+    C = torch.empty((M, N), device=A.device, dtype=torch.bfloat16)
+    rc = _lib.lib().bi_gemm_bf16(a.data_ptr(), lda, w.data_ptr(), 1, ldw, C.data_ptr(), C.stride(0),
+                                 M, N, K, None if b is None else b.data_ptr(), _stream(A))
+    _lib.check(rc, "bi_gemm_bf16")
+    return C
+
+
+@bi_gemm_bf16.register_fake
+def _(A, B, bias):
+    return A.new_empty((A.shape[0], B.shape[1]))
+
+
+@torch.library.custom_op("tbik::bi_rmsnorm_bf16", mutates_args=(), device_types="cuda")
+def bi_rmsnorm_bf16(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float) -> torch.Tensor:
+    _require_gpu(x, weight)
+    hidden = x.shape[-1]
+    x2, ldx = _rows16(x.reshape(-1, hidden))
+    out = torch.empty((x2.shape[0], hidden), device=x.device, dtype=torch.bfloat16)
+    w = None if weight is None else weight.contiguous()
+    rc = _lib.lib().bi_rmsnorm_bf16(x2.data_ptr(), ldx, None, 0, None if w is None else w.data_ptr(),
+                                    out.data_ptr(), out.stride(0), None, 0, x2.shape[0], hidden, eps, _stream(x))
+    _lib.check(rc, "bi_rmsnorm_bf16")
+    return out.reshape(x.shape)
+
+
+@bi_rmsnorm_bf16.register_fake
+def _(x, weight, eps):
+    return torch.empty_like(x)
+
+
+@torch.library.custom_op("tbik::bi_add_rmsnorm_bf16", mutates_args=(), device_types="cuda")
+def bi_add_rmsnorm_bf16(x: torch.Tensor, residual: torch.Tensor, weight: Optional[torch.Tensor],
+                        eps: float) -> List[torch.Tensor]:
+    _require_gpu(x, residual, weight)
+    hidden = x.shape[-1]
+    x2, ldx = _rows16(x.reshape(-1, hidden))
+    r2, ldr = _rows16(residual.reshape(-1, hidden))
+    out = torch.empty((x2.shape[0], hidden), device=x.device, dtype=torch.bfloat16)
+    rout = torch.empty_like(out)
+    w = None if weight is None else weight.contiguous()
+    rc = _lib.lib().bi_rmsnorm_bf16(x2.data_ptr(), ldx, r2.data_ptr(), ldr,
+                                    None if w is None else w.data_ptr(), out.data_ptr(), out.stride(0),
+                                    rout.data_ptr(), rout.stride(0), x2.shape[0], hidden, eps, _stream(x))
+    _lib.check(rc, "bi_rmsnorm_bf16")
+    return [out.reshape(x.shape), rout.reshape(x.shape)]
+
+
+@bi_add_rmsnorm_bf16.register_fake
+def _(x, residual, weight, eps):
+    return [torch.empty_like(x), torch.empty_like(x)]
+
+
+@torch.library.custom_op("tbik::bi_log_softmax_f32", mutates_args=(), device_types="cuda")
+def bi_log_softmax_f32(x: torch.Tensor, write_softmax: bool) -> torch.Tensor:
+    _require_gpu(x)
+    cols = x.shape[-1]
+    x2 = x.reshape(-1, cols)
+    if x2.stride(1) != 1 or (x2.shape[0] > 1 and x2.stride(0) < cols):
+        x2 = x2.contiguous()
+    rows = x2.shape[0]
+    out = torch.empty((rows, cols), device=x.device, dtype=torch.float32)
+    L = _lib.lib()
+    ws = torch.empty((max(L.bi_log_softmax_workspace_bytes(rows, cols), 4) + 3) // 4, device=x.device, dtype=torch.float32)
+    rc = L.bi_log_softmax_f32(x2.data_ptr(), x2.stride(0) if rows > 1 else cols, out.data_ptr(), out.stride(0),
+                              rows, cols, ws.data_ptr(), ws.numel() * 4, int(write_softmax), _stream(x))
+    _lib.check(rc, "bi_log_softmax_f32")
+    return out.reshape(x.shape)
+
+
+@bi_log_softmax_f32.register_fake
+def _(x, write_softmax):
+    return torch.empty_like(x)
+
+
+@torch.library.custom_op("tbik::bi_mean_dim", mutates_args=(), device_types="cuda")
+def bi_mean_dim(x: torch.Tensor, dim: int, keepdim: bool) -> torch.Tensor:
+    _require_gpu(x)
+    if x.dtype not in _DTYPE_CODE:
+        raise NotImplementedError(f"bi_mean_dim: unsupported dtype {x.dtype}")
+    dim = dim % x.ndim
+    shape = list(x.shape)
+    outer = 1
+    for s in shape[:dim]:
+        outer *= s
+    n = shape[dim]
+    inner = 1
+    for s in shape[dim + 1:]:
+        inner *= s
+    xc = x.contiguous()
+    out_shape = shape[:dim] + ([1] if keepdim else []) + shape[dim + 1:]
+    out = torch.empty(out_shape, device=x.device, dtype=x.dtype)
+    rc = _lib.lib().bi_mean_dim(xc.data_ptr(), out.data_ptr(), outer, n, inner, _DTYPE_CODE[x.dtype], _stream(x))
+    _lib.check(rc, "bi_mean_dim")
+    return out
+
+
+@bi_mean_dim.register_fake
+def _(x, dim, keepdim):
+    dim = dim % x.ndim
+    shape = list(x.shape)
+    out_shape = shape[:dim] + ([1] if keepdim else []) + shape[dim + 1:]
+    return x.new_empty(out_shape)

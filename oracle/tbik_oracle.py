@@ -1,0 +1,268 @@
+"""CPU oracle for the tree-ordered (TP-invariant) matmul and the batch-invariant reductions.
+
+TEST INFRASTRUCTURE ONLY.  Nothing in the shipped package may import this module: it is the
+checker for the HIP kernels (tests, the smoke check and the CPU-baseline leg of the benchmark),
+never the thing that is measured or shipped.
+
+Every function restates, on the CPU with plain PyTorch, the arithmetic of one piece of the
+reference and cites the lines it follows (paths relative to the reference checkout):
+
+* tree parameters ............ src/tbik/tree_based_matmul.py:240-249
+* leaf value ................. src/tbik/tree_based_matmul.py:121-136   (fp32 dot over one K chunk -> bf16)
+* carry / merge loop ......... src/tbik/tree_based_matmul.py:140-174   (literal emulation: `carry_merge`)
+* closed form of that loop ... `tree_reduce_leaves` (level 0 left-to-right over FLB leaves, then adjacent pairs)
+* shard combine .............. src/tbik/tree_based_all_reduce.py:32-35, simple_matmul.py:35-38,
+                               mini_allreduce/tbik_kernel/csrc/allreduce/custom_all_reduce.cuh:203-234
+* simulated TP ............... simple_matmul.py:23-43
+* batch-invariant mm ......... src/bio/batch_invariant_ops.py:98-123   (one fp32 accumulator over all of K)
+* log_softmax ................ src/bio/batch_invariant_ops.py:219-260
+* mean ....................... src/bio/batch_invariant_ops.py:331-349
+* RMSNorm .................... src/patch/patch_batch_invariant.py:9-16 -> vLLM RMSNorm.forward_native
+                               (vllm==0.11.0 is not vendored in the reference; the public formula is restated)
+
+Pin status (what checks each function independently of its own formula; see tests/test_oracle_*.py):
+
+* `tree_params`, `tree_reduce_leaves`, `tree_combine`: pinned.  The closed form is checked against
+  `carry_merge` (a line-by-line emulation of the reference's binary-counter loop), against an exact
+  rational-arithmetic brute force with an independent round-to-nearest-even, against the plain-C
+  restatement in oracle/tbik_oracle.c, and through the reference's own self-consistency checks
+  (simple_matmul.py:16-43: batch-slice invariance and simulated-TP invariance must be exactly 0).
+* `leaf_partials`: the intra-chunk fp32 accumulation order is hardware defined in the reference
+  (Triton `tl.dot`), so it is pinned bit-exactly only where the chunk sum is exactly representable
+  (integer-valued inputs), and to 1 bf16 ulp otherwise.  PARITY UNPINNED beyond that.
+* `rmsnorm`: PARITY UNPINNED against the reference (the arithmetic lives in vllm==0.11.0, absent);
+  pinned to the textbook formula in float64 and to closed-form cases.
+* `log_softmax`, `mean_lastdim`: pinned to float64 library routines and closed-form cases; the
+  reference's in-block reduction order (Triton `tl.sum`) is backend defined, so tolerance only.
+"""
+from __future__ import annotations
+
+import math
+from typing import List, Optional, Sequence, Tuple
+
+import torch
+
+LEAF_BF16 = 256  # BLOCK_SIZE_K of the bf16/fp16 configs, src/tbik/tree_based_matmul.py:206-222
+
+
+# --------------------------------------------------------------------------------------------
+# tree shape
+# --------------------------------------------------------------------------------------------
+def tree_params(K: int, leaf: int = LEAF_BF16) -> Tuple[int, int, int]:
+    """(T, FLB, LEVEL_K) for a K extent, following src/tbik/tree_based_matmul.py:242-249.
+
+    T leaves of `leaf` elements; FLB = T with factors of two removed while it is even and > 2;
+    LEVEL_K = number of halvings + 1, so T == FLB * 2**(LEVEL_K-1).
+    """
+    assert K % leaf == 0, "K must be a whole number of leaves"
+    T = K // leaf
+    flb, level_k = T, 1
+    while flb > 2 and flb % 2 == 0:
+        flb //= 2
+        level_k += 1
+    return T, flb, level_k
+
+
+# --------------------------------------------------------------------------------------------
+# leaves
+# --------------------------------------------------------------------------------------------
+def leaf_partials(A: torch.Tensor, B: torch.Tensor, leaf: int = LEAF_BF16) -> List[torch.Tensor]:
+    """One bf16 [M,N] partial per K chunk: fp32 dot over the chunk, rounded once to A's dtype.
+
+    Follows src/tbik/tree_based_matmul.py:121-136 (`acc = tl.dot(a, b).to(ACC_DTYPE)` with
+    ACC_DTYPE = A.dtype, :193-194).
+    """
+    M, K = A.shape
+    assert B.shape[0] == K
+    out = []
+    for k0 in range(0, K, leaf):
+        a = A[:, k0:k0 + leaf].float()
+        b = B[k0:k0 + leaf, :].float()
+        out.append(torch.matmul(a, b).to(A.dtype))
+    return out
+
+
+# --------------------------------------------------------------------------------------------
+# merge order: literal emulation and closed form
+# --------------------------------------------------------------------------------------------
+def carry_merge(leaves: Sequence[torch.Tensor], flb: int, level_k: int) -> torch.Tensor:
+    """Line-by-line emulation of the binary-counter loop, src/tbik/tree_based_matmul.py:119-174.
+
+    `count[level]` is the number of partials absorbed at that level; level 0 carries when it has
+    absorbed FLB leaves, every other level when it has absorbed 2.  Partials of levels 0..2 live in
+    acc1..acc3, deeper ones in S[level-3].  All adds are in the tensors' dtype (bf16).
+    """
+    manual_acc = 3
+    count = [0] * max(level_k, 1)
+    acc1 = acc2 = acc3 = None
+    S = {}
+    acc = None
+    for leaf in leaves:
+        acc = leaf.clone()
+        break_flag = False
+        for level in range(level_k):
+            if break_flag:
+                continue
+            count_value_added = count[level] + 1
+            table_value = flb if level == 0 else 2
+            carry_over = table_value == count_value_added
+            if count_value_added > 1:
+                if level == 0:
+                    acc = acc1 + acc
+                elif level == 1:
+                    acc = acc2 + acc
+                elif level == 2:
+                    acc = acc3 + acc
+                else:
+                    acc = S[level - manual_acc] + acc
+            count[level] = 0 if carry_over else count_value_added
+            if not carry_over:
+                break_flag = True
+                if level == 0:
+                    acc1 = acc
+                elif level == 1:
+                    acc2 = acc
+                elif level == 2:
+                    acc3 = acc
+                else:
+                    S[level - manual_acc] = acc
+    return acc
+
+
+def tree_combine(parts: Sequence[torch.Tensor]) -> torch.Tensor:
+    """Adjacent-pair binary tree over a power-of-two number of partials, adds in the parts' dtype.
+
+    Follows src/tbik/tree_based_all_reduce.py:26-37 (and simple_matmul.py:35-38,
+    custom_all_reduce.cuh:203-234): at level l, result[left] += result[left + 2**(l-1)].
+    """
+    n = len(parts)
+    if n & (n - 1) != 0 or n == 0:
+        raise ValueError("the number of partials must be a power of two")
+    result = [p.clone() for p in parts]
+    for level in range(1, n.bit_length()):
+        for left in range(0, n, 1 << level):
+            right = left + (1 << (level - 1))
+            result[left] += result[right]
+    return result[0]
+
+
+def tree_reduce_leaves(leaves: Sequence[torch.Tensor], flb: int) -> torch.Tensor:
+    """Closed form of `carry_merge`: left-to-right sums of FLB consecutive leaves, then `tree_combine`."""
+    assert len(leaves) % flb == 0
+    groups = []
+    for g in range(0, len(leaves), flb):
+        s = leaves[g].clone()
+        for j in range(1, flb):
+            s = s + leaves[g + j]
+        groups.append(s)
+    return tree_combine(groups)
+
+
+# --------------------------------------------------------------------------------------------
+# the operator and the simulated tensor-parallel harness
+# --------------------------------------------------------------------------------------------
+def matmul_tree(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                leaf: int = LEAF_BF16) -> torch.Tensor:
+    """CPU restatement of matmul_tp_persistent (src/tbik/tree_based_matmul.py:190-277)."""
+    assert A.shape[-1] == B.shape[-2], "Dim doesn't match"
+    _, flb, _ = tree_params(A.shape[1], leaf)
+    C = tree_reduce_leaves(leaf_partials(A, B, leaf), flb)
+    if bias is not None:
+        C += bias  # :275-276, added in the output dtype after the tree
+    return C
+
+
+def simulated_tp_matmul(A: torch.Tensor, B: torch.Tensor, num_shards: int,
+                        leaf: int = LEAF_BF16) -> torch.Tensor:
+    """K split into `num_shards` equal contiguous slices, one tree matmul each, then the shard tree.
+
+    Follows simple_matmul.py:23-38 (with the shard count no longer hard-coded to 4).
+    """
+    K = A.shape[1]
+    assert K % num_shards == 0
+    ks = K // num_shards
+    parts = [matmul_tree(A[:, i * ks:(i + 1) * ks], B[i * ks:(i + 1) * ks, :], leaf=leaf)
+             for i in range(num_shards)]
+    return tree_combine(parts)
+
+
+# --------------------------------------------------------------------------------------------
+# batch-invariant ops
+# --------------------------------------------------------------------------------------------
+def matmul_single_acc(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Batch-invariant mm/addmm: one fp32 accumulator over all of K, bias added in fp32, one rounding.
+
+    Follows src/bio/batch_invariant_ops.py:98-118.  The reference then rounds through fp16 before the
+    store converts to the output dtype (:119-123); that detour is deliberately not reproduced, the
+    result here is rounded once to the output dtype.
+    """
+    acc = torch.matmul(a.float(), b.float())
+    if bias is not None:
+        acc = acc + bias.float()
+    return acc.to(a.dtype)
+
+
+def log_softmax_lastdim(x: torch.Tensor) -> torch.Tensor:
+    """x - max - log(sum(exp(x - max))) per row in fp32; src/bio/batch_invariant_ops.py:219-260."""
+    xf = x.float()
+    m = xf.max(dim=-1, keepdim=True).values
+    s = torch.exp(xf - m).sum(dim=-1, keepdim=True)
+    return (xf - m - torch.log(s)).to(x.dtype)
+
+
+def mean_lastdim(x: torch.Tensor, keepdim: bool = False) -> torch.Tensor:
+    """fp32 sum over the last dim divided by its length; src/bio/batch_invariant_ops.py:331-349."""
+    n = x.shape[-1]
+    return (x.float().sum(dim=-1, keepdim=keepdim) / n).to(x.dtype)
+
+
+def rmsnorm(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float,
+            residual: Optional[torch.Tensor] = None):
+    """RMSNorm as vLLM's RMSNorm.forward_native computes it (reached through
+    src/patch/patch_batch_invariant.py:9-16; vllm==0.11.0 itself is not in the reference tree).
+
+    x -> fp32; optional `x += residual` with the sum rounded to the input dtype as the new residual;
+    var = mean(x^2) over the last dim; x * rsqrt(var + eps) rounded to the input dtype, THEN
+    multiplied by the weight in the input dtype.
+    """
+    orig = x.dtype
+    xf = x.float()
+    new_residual = None
+    if residual is not None:
+        xf = xf + residual.float()
+        new_residual = xf.to(orig)
+    var = xf.pow(2).mean(dim=-1, keepdim=True)
+    y = (xf * torch.rsqrt(var + eps)).to(orig)
+    if weight is not None:
+        y = y * weight
+    return y if residual is None else (y, new_residual)
+
+
+# --------------------------------------------------------------------------------------------
+# seeded synthetic inputs shared by the tests, the smoke check and the benchmark
+# --------------------------------------------------------------------------------------------
+def gaussian_bf16(shape, std: float, seed: int) -> torch.Tensor:
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g, dtype=torch.float32) * std).to(torch.bfloat16)
+
+
+def silu_gated_bf16(shape, seed: int) -> torch.Tensor:
+    """Activation of a SiLU-gated MLP: g1 * silu(g2) with g1, g2 ~ N(0,1), rounded to bf16."""
+    g = torch.Generator().manual_seed(seed)
+    g1 = torch.randn(shape, generator=g, dtype=torch.float32)
+    g2 = torch.randn(shape, generator=g, dtype=torch.float32)
+    return (g1 * torch.nn.functional.silu(g2)).to(torch.bfloat16)
+
+
+def integer_bf16(shape, lo: int, hi: int, seed: int) -> torch.Tensor:
+    """Uniform integers in [lo, hi]: every chunk sum is an integer, exact in fp32 in any order."""
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(lo, hi + 1, shape, generator=g).to(torch.bfloat16)
+
+
+def bf16_ulp_distance(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """Distance in units of bf16 representable values (sign-magnitude order), elementwise."""
+    def key(t):
+        i = t.contiguous().view(torch.int16).to(torch.int32) & 0xFFFF
+        return torch.where(i >= 0x8000, 0x8000 - i, i)
+    return (key(a) - key(b)).abs()

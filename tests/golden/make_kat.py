@@ -1,0 +1,107 @@
+"""Writes the integer known-answer fixtures for the tree matmul (tests/golden/kat_tree_matmul.npz).
+
+Inputs are small integers, so every leaf sum is an integer that fp32 holds exactly in ANY
+accumulation order; the expected output is then a function of the tree order and of round-to-
+nearest-even alone, and any implementation of the contract must reproduce it bit for bit.
+Expected values come from the rational-arithmetic brute force below (exact leaf sums as Python
+integers, explicit bf16 rounding), which shares no code with oracle/.
+
+    python tests/golden/make_kat.py
+"""
+import os
+import sys
+from fractions import Fraction
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def rn_bf16(x: Fraction) -> Fraction:
+    """Round a rational to the nearest bf16 value (8 significant bits), ties to even; no overflow handling."""
+    if x == 0:
+        return Fraction(0)
+    s = -1 if x < 0 else 1
+    a = abs(x)
+    e = 0
+    while a >= 2 ** (e + 1):
+        e += 1
+    while a < 2 ** e:
+        e -= 1
+    ulp = Fraction(2) ** (e - 7)
+    q = a / ulp
+    fl = q.numerator // q.denominator
+    rem = q - fl
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and fl % 2 == 1):
+        fl += 1
+    return s * fl * ulp
+
+
+def tree_params(T):
+    flb, lev = T, 1
+    while flb > 2 and flb % 2 == 0:
+        flb //= 2
+        lev += 1
+    return flb, lev
+
+
+def brute_force(A, B, leaf):
+    M, K = A.shape
+    N = B.shape[1]
+    T = K // leaf
+    flb, _ = tree_params(T)
+    out = np.zeros((M, N), dtype=np.float64)
+    for m in range(M):
+        for n in range(N):
+            leaves = [rn_bf16(Fraction(int(np.dot(A[m, j * leaf:(j + 1) * leaf], B[j * leaf:(j + 1) * leaf, n]))))
+                      for j in range(T)]
+            groups = []
+            for g in range(0, T, flb):
+                s = leaves[g]
+                for j in range(1, flb):
+                    s = rn_bf16(s + leaves[g + j])
+                groups.append(s)
+            while len(groups) > 1:
+                groups = [rn_bf16(groups[i] + groups[i + 1]) for i in range(0, len(groups), 2)]
+            out[m, n] = float(groups[0])
+    return out
+
+
+def to_bf16_bits(x: np.ndarray) -> np.ndarray:
+    f = x.astype(np.float32)
+    assert np.array_equal(f.astype(np.float64), x), "value not exact in fp32"
+    u = f.view(np.uint32)
+    assert np.all((u & 0xFFFF) == 0), "value not exact in bf16"
+    return (u >> 16).astype(np.uint16)
+
+
+CASES = [  # name, M, N, K, leaf, amax, bmax, seed
+    ("t1_flb1", 5, 8, 256, 256, 9, 7, 1),
+    ("t2_flb2", 4, 8, 512, 256, 9, 7, 2),
+    ("t3_flb3", 4, 8, 768, 256, 9, 7, 3),
+    ("t6_flb3_l2", 3, 8, 1536, 256, 9, 7, 4),
+    ("t8_flb2_l3", 3, 8, 2048, 256, 9, 7, 5),
+    ("t5_flb5", 3, 8, 1280, 256, 9, 7, 6),
+    ("t12_leaf128", 3, 8, 1536, 128, 9, 7, 7),
+    ("t25_leaf128", 2, 8, 3200, 128, 9, 7, 8),
+    ("t48_flb3_l5", 2, 4, 12288, 256, 9, 7, 9),
+]
+
+
+def main():
+    out = {}
+    for name, M, N, K, leaf, amax, bmax, seed in CASES:
+        rng = np.random.default_rng(seed)
+        A = rng.integers(-amax, amax + 1, size=(M, K)).astype(np.int64)
+        B = rng.integers(-bmax, bmax + 1, size=(K, N)).astype(np.int64)
+        C = brute_force(A, B, leaf)
+        out[name + "_A"] = A.astype(np.int8)
+        out[name + "_B"] = B.astype(np.int8)
+        out[name + "_C"] = to_bf16_bits(C)
+        out[name + "_leaf"] = np.array(leaf, dtype=np.int32)
+        print(name, "max |C| =", np.abs(C).max(), "rounded nodes matter:", bool(np.abs(C).max() > 256))
+    np.savez_compressed(os.path.join(HERE, "kat_tree_matmul.npz"), **out)
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,130 @@
+"""GPU parity and batch invariance of RMSNorm, log_softmax / softmax, mean and the single-accumulator mm."""
+import math
+
+import pytest
+import torch
+
+from oracle import tbik_oracle as O
+from llm_reproducibility_amd.bio import batch_invariant_ops as bio
+
+pytestmark = pytest.mark.gpu
+ROWS = (1, 7, 256, 4096)
+
+
+def test_rmsnorm_parity_and_batch_invariance(dev):
+    x = O.gaussian_bf16((4096, 4096), 1.0, 0)
+    w = (1.0 + 0.1 * torch.randn(4096, generator=torch.Generator().manual_seed(1))).to(torch.bfloat16)
+    xd, wd = x.to(dev), w.to(dev)
+    full = bio.rms_norm(xd, wd, 1e-6)
+    want = O.rmsnorm(x[:300], w, 1e-6)
+    ulp = O.bf16_ulp_distance(full[:300].cpu(), want)
+    assert ulp.max() <= 2 and (ulp > 0).float().mean() < 0.02, (ulp.max(), (ulp > 0).float().mean())
+    for r in ROWS:
+        assert torch.equal(bio.rms_norm(xd[:r], wd, 1e-6), full[:r]), r
+    assert torch.equal(bio.rms_norm(xd[1234:1235], wd, 1e-6), full[1234:1235])
+    # exact case: +-1 row with unit weight
+    s = torch.ones((3, 4096), dtype=torch.bfloat16)
+    s[:, ::2] = -1
+    assert torch.equal(bio.rms_norm(s.to(dev), torch.ones(4096, dtype=torch.bfloat16, device=dev), 1e-6).cpu(), s)
+
+
+def test_add_rmsnorm_parity(dev):
+    x = O.gaussian_bf16((64, 4096), 1.0, 2)
+    res = O.gaussian_bf16((64, 4096), 1.0, 3)
+    w = O.gaussian_bf16((4096,), 1.0, 4)
+    out, new_res = bio.rms_norm(x.to(dev), w.to(dev), 1e-6, residual=res.to(dev))
+    want, want_res = O.rmsnorm(x, w, 1e-6, residual=res)
+    assert torch.equal(new_res.cpu(), want_res)
+    assert O.bf16_ulp_distance(out.cpu(), want).max() <= 2
+    for hidden in (8, 64, 520, 1024, 5120, 8192):
+        xs = O.gaussian_bf16((5, hidden), 2.0, hidden)
+        ws = O.gaussian_bf16((hidden,), 1.0, hidden + 1)
+        got = bio.rms_norm(xs.to(dev), ws.to(dev), 1e-5)
+        assert O.bf16_ulp_distance(got.cpu(), O.rmsnorm(xs, ws, 1e-5)).max() <= 2, hidden
+
+
+def test_log_softmax_parity_and_batch_invariance(dev):
+    V = 151936
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn((256, V), generator=g) * 3.0
+    xd = x.to(dev)
+    full = bio.log_softmax(xd)
+    want = torch.log_softmax(x[:16].double(), dim=-1)
+    assert (full[:16].cpu().double() - want).abs().max() < 2e-5
+    for r in (1, 7, 256):
+        assert torch.equal(bio.log_softmax(xd[:r]), full[:r]), r
+    assert torch.equal(bio.log_softmax(xd[100:101]), full[100:101])
+    big = xd.repeat(16, 1)                                   # 4096 rows
+    out_big = bio.log_softmax(big)
+    assert torch.equal(out_big[:256], full) and torch.equal(out_big[-256:], full)
+    # softmax = exp(log_softmax), sums to 1
+    sm = bio.softmax(xd[:7])
+    assert (sm.sum(-1) - 1).abs().max() < 1e-4
+    assert (sm.cpu().double() - torch.softmax(x[:7].double(), -1)).abs().max() < 1e-6
+    # closed forms: constant row -> -log V; ragged widths incl. not a multiple of 4
+    c = torch.full((2, 1000), 4.25, device=dev)
+    assert torch.allclose(bio.log_softmax(c), torch.full_like(c, -math.log(1000.0)), atol=2e-6)
+    for cols in (1, 3, 5, 4095, 4096, 4097, 8191, 12289):
+        y = torch.randn((3, cols), generator=g)
+        got = bio.log_softmax(y.to(dev)).cpu()
+        assert (got.double() - torch.log_softmax(y.double(), -1)).abs().max() < 1e-5, cols
+    # bf16 input keeps its dtype
+    yb = torch.randn((4, 512), generator=g).to(torch.bfloat16)
+    assert bio.log_softmax(yb.to(dev)).dtype == torch.bfloat16
+
+
+def test_mean_parity_and_batch_invariance(dev):
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn((4096, 4096), generator=g)
+    xd = x.to(dev)
+    full = bio.mean_dim(xd, -1)
+    assert (full.cpu().double() - x.double().mean(-1)).abs().max() < 1e-6
+    for r in ROWS:
+        assert torch.equal(bio.mean_dim(xd[:r], -1), full[:r]), r
+    ints = torch.arange(0, 4096, dtype=torch.float32, device=dev).repeat(3, 1)
+    assert torch.equal(bio.mean_dim(ints, 1, keepdim=True), torch.full((3, 1), 2047.5, device=dev))
+    # long rows (block-per-row), a middle dimension, bf16
+    y = torch.randn((5, 20000), generator=g)
+    assert (bio.mean_dim(y.to(dev), 1).cpu().double() - y.double().mean(1)).abs().max() < 1e-6
+    z = torch.randn((6, 37, 10), generator=g)
+    assert (bio.mean_dim(z.to(dev), 1).cpu().double() - z.double().mean(1)).abs().max() < 1e-6
+    zb = z.to(torch.bfloat16)
+    got = bio.mean_dim(zb.to(dev), 2)
+    assert got.dtype == torch.bfloat16 and (got.cpu().float() - zb.float().mean(2)).abs().max() < 1e-2
+
+
+def test_single_accumulator_mm_parity_and_batch_invariance(dev):
+    a = O.gaussian_bf16((300, 4096), 1.0, 0)
+    w = O.gaussian_bf16((1000, 4096), 0.02, 1)                # [N,K] as nn.Linear stores it
+    bias = O.gaussian_bf16((1000,), 1.0, 2)
+    ad, wd, bd = a.to(dev), w.to(dev), bias.to(dev)
+    full = bio.matmul_persistent(ad, wd.t(), bd)
+    want = O.matmul_single_acc(a, w.t(), bias)
+    ulp = O.bf16_ulp_distance(full.cpu(), want)
+    assert ulp.max() <= 1 and (ulp > 0).float().mean() < 0.01
+    for m in (1, 7, 64, 129):
+        assert torch.equal(bio.matmul_persistent(ad[:m], wd.t(), bd), full[:m]), m
+    # exact on integers, K not a multiple of 64 nor of 8, row-major b
+    ai = O.integer_bf16((33, 1003), -9, 9, 3)
+    bi = O.integer_bf16((1003, 40), -7, 7, 4)
+    got = bio.matmul_persistent(ai.to(dev), bi.to(dev))
+    assert torch.equal(got.cpu(), O.matmul_single_acc(ai, bi))
+
+
+def test_aten_overrides_route_to_the_hip_kernels(dev):
+    a = O.gaussian_bf16((20, 512), 1.0, 0).to(dev)
+    w = O.gaussian_bf16((64, 512), 0.1, 1).to(dev)
+    b = O.gaussian_bf16((64,), 1.0, 2).to(dev)
+    logits = torch.randn((5, 3000), device=dev)
+    with bio.set_batch_invariant_mode(True):
+        assert bio.is_batch_invariant_mode_enabled()
+        assert torch.equal(torch.mm(a, w.t()), bio.matmul_persistent(a, w.t()))
+        assert torch.equal(torch.nn.functional.linear(a, w, b), bio.matmul_persistent(a, w.t(), b))
+        assert torch.equal(torch.log_softmax(logits, -1), bio.log_softmax(logits))
+        assert torch.equal(torch.softmax(logits, -1), bio.softmax(logits))
+        assert torch.equal(logits.mean(-1, keepdim=True), bio.mean_dim(logits, -1, keepdim=True))
+        m2 = logits.reshape(5, 30, 100).mean(dim=(1, 2))
+        assert (m2 - logits.mean(-1)).abs().max() < 1e-6
+    assert not bio.is_batch_invariant_mode_enabled()
+    ref = torch.log_softmax(logits, -1)              # stock kernel again after leaving the mode
+    assert (ref - bio.log_softmax(logits)).abs().max() < 1e-5

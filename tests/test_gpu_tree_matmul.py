@@ -1,0 +1,167 @@
+"""GPU parity of the tree-ordered matmul (tbik_gemm_bf16 through the C ABI) against the CPU oracle.
+
+Bit-exact on integer-valued inputs (every leaf sum exact, so only the tree order and the rounding
+decide the result); on Gaussian inputs each element must be within 1 bf16 ulp of the oracle OR within
+2^-8 of the output scale; invariance across simulated TP = 1/2/4/8 and across batch sizes is bitwise.
+"""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import tbik_oracle as O
+from llm_reproducibility_amd.tbik import choose_leaf_k, matmul_tp_persistent, tree_combine
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "kat_tree_matmul.npz")
+
+
+def bits(t):
+    return t.contiguous().view(torch.int16)
+
+
+def assert_bitwise(a, b, msg=""):
+    a, b = a.cpu(), b.cpu()
+    if not torch.equal(bits(a), bits(b)):
+        d = (a.float() - b.float()).abs()
+        raise AssertionError(f"{msg}: {int((bits(a) != bits(b)).sum())} of {a.numel()} elements differ, max |diff| {d.max().item()}")
+
+
+def assert_close_to_oracle(got, want, msg=""):
+    """<= 1 bf16 ulp, or |diff| <= 2^-8 * max|want| (the tolerance the contract states for random inputs)."""
+    got, want = got.cpu(), want.cpu()
+    ulp = O.bf16_ulp_distance(got, want)
+    diff = (got.float() - want.float()).abs()
+    scale = want.float().abs().max().item()
+    bad = (ulp > 1) & (diff > 2.0 ** -8 * scale)
+    assert not bad.any(), f"{msg}: {int(bad.sum())} elements off; max ulp {int(ulp.max())}, max diff {diff.max().item()}, scale {scale}"
+
+
+def sim_tp(A, W_kn, p, leaf_k):
+    K = A.shape[1]
+    ks = K // p
+    parts = [matmul_tp_persistent(A[:, r * ks:(r + 1) * ks], W_kn[r * ks:(r + 1) * ks, :], leaf_k=leaf_k) for r in range(p)]
+    return parts[0] if p == 1 else tree_combine(parts)
+
+
+def test_rational_known_answers(dev):
+    z = np.load(GOLDEN)
+    for n in sorted({k[:-2] for k in z.files if k.endswith("_A")}):
+        A = torch.from_numpy(z[n + "_A"].astype(np.float32)).to(torch.bfloat16).to(dev)
+        B = torch.from_numpy(z[n + "_B"].astype(np.float32)).to(torch.bfloat16).to(dev)
+        C = torch.from_numpy(z[n + "_C"].view(np.int16).copy()).view(torch.bfloat16)
+        leaf = int(z[n + "_leaf"])
+        print("case", n, tuple(A.shape), tuple(B.shape), leaf, flush=True)
+        assert_bitwise(matmul_tp_persistent(A, B, leaf_k=leaf), C, n)
+        # the weight as nn.Linear stores it ([N,K], handed over as weight.t())
+        Wnk = B.t().contiguous()
+        assert_bitwise(matmul_tp_persistent(A, Wnk.t(), leaf_k=leaf), C, n + " (weight.t())")
+
+
+# (M, N, K, leaf): tails in M and N, every tile configuration, FLB in {1,2,3,5,25}, 0..5 binary levels
+INT_SHAPES = [
+    (1, 64, 256, 256), (3, 72, 512, 256), (16, 128, 768, 256), (17, 200, 1536, 256), (64, 136, 2048, 256),
+    (65, 128, 1280, 256), (130, 264, 3072, 256), (257, 512, 4096, 256), (128, 128, 12288, 256),
+    (33, 96, 3200, 128), (129, 160, 6400, 128), (20, 64, 6400, 256), (8, 24, 8192, 256), (300, 4, 512, 256),
+]
+
+
+@pytest.mark.parametrize("M,N,K,leaf", INT_SHAPES)
+def test_integer_inputs_match_oracle_bitwise(dev, M, N, K, leaf):
+    print("case", M, N, K, leaf, flush=True)
+    A = O.integer_bf16((M, K), -9, 9, 10 + M)
+    B = O.integer_bf16((K, N), -7, 7, 20 + N)
+    want = O.matmul_tree(A, B, leaf=leaf)
+    Wnk = B.t().contiguous().to(dev)
+    got = matmul_tp_persistent(A.to(dev), Wnk.t(), leaf_k=leaf)
+    assert got.shape == (M, N) and got.dtype == torch.bfloat16 and got.is_contiguous()
+    assert_bitwise(got, want, f"{M}x{N}x{K}")
+
+
+def test_bias_strided_a_and_row_major_b(dev):
+    M, N, K = 70, 96, 1536
+    A_wide = O.integer_bf16((M, 2 * K), -9, 9, 1)
+    B = O.integer_bf16((K, N), -7, 7, 2)
+    bias = O.integer_bf16((N,), -300, 300, 3)
+    A = A_wide[:, K:]                      # row stride 2K, offset K: a shard's view of a wider activation
+    want = O.matmul_tree(A, B, bias)
+    Ad = A_wide.to(dev)[:, K:]
+    assert not Ad.is_contiguous()
+    got = matmul_tp_persistent(Ad, B.to(dev), bias.to(dev))     # row-major [K,N] operand
+    assert_bitwise(got, want, "bias + strided A + row-major B")
+    odd = A_wide.to(dev)[:, 3:3 + K]       # misaligned view: repacked by the wrapper, same bits
+    assert_bitwise(matmul_tp_persistent(odd, B.to(dev)), O.matmul_tree(A_wide[:, 3:3 + K], B), "misaligned A")
+
+
+@pytest.mark.parametrize("M,N,K", [(256, 4096, 4096), (128, 512, 12288), (16, 256, 12288), (1, 128, 8192)])
+def test_gaussian_inputs_within_one_ulp_of_oracle(dev, M, N, K):
+    print("case", M, N, K, flush=True)
+    A = O.gaussian_bf16((M, K), 1.0, 0) if K != 12288 else O.silu_gated_bf16((M, K), 0)
+    Wnk = O.gaussian_bf16((N, K), 0.02, 1)
+    want = O.matmul_tree(A, Wnk.t())
+    got = matmul_tp_persistent(A.to(dev), Wnk.to(dev).t())
+    assert_close_to_oracle(got, want, f"{M}x{N}x{K}")
+    for p in (2, 4, 8):
+        assert_bitwise(sim_tp(A.to(dev), Wnk.to(dev).t(), p, 256), got, f"TP={p}")
+
+
+def _invariance(dev, K, N, Ms, x_kind, max_m):
+    leaf = choose_leaf_k(K)
+    X = (O.silu_gated_bf16((max_m, K), 0) if x_kind == "silu" else O.gaussian_bf16((max_m, K), 1.0, 0)).to(dev)
+    Wt = O.gaussian_bf16((N, K), 0.02, 1).to(dev).t()
+    full = matmul_tp_persistent(X, Wt, leaf_k=leaf)
+    for p in (2, 4, 8):
+        print("case K", K, "TP", p, flush=True)
+        assert_bitwise(sim_tp(X, Wt, p, leaf), full, f"K={K} TP={p} M={max_m}")
+    for M in Ms:
+        print("case K", K, "M", M, flush=True)
+        sub = matmul_tp_persistent(X[:M], Wt, leaf_k=leaf)
+        assert_bitwise(sub, full[:M], f"K={K} batch prefix M={M}")
+        for p in (2, 8):
+            assert_bitwise(sim_tp(X[:M], Wt, p, leaf), full[:M], f"K={K} TP={p} M={M}")
+    # a row computed alone equals the same row inside the batch (row 777 of the large batch)
+    i = min(777, max_m - 1)
+    assert_bitwise(matmul_tp_persistent(X[i:i + 1], Wt, leaf_k=leaf), full[i:i + 1], f"K={K} row {i} alone")
+    torch.cuda.synchronize()
+
+
+def test_invariance_qwen3_8b_down_proj(dev):
+    _invariance(dev, 12288, 4096, (1, 16, 128), "silu", 2048)
+
+
+def test_invariance_qwen3_32b_o_proj(dev):
+    _invariance(dev, 8192, 5120, (1, 64, 512), "gauss", 4096)
+
+
+def test_invariance_qwen3_32b_down_proj_leaf128(dev):
+    # 25600 / 8 = 3200 is not a multiple of 256: the layer uses leaf 128 at EVERY TP degree
+    assert choose_leaf_k(25600) == 128
+    _invariance(dev, 25600, 5120, (1, 64, 512), "gauss", 4096)
+
+
+def test_reference_smoke_script_shape(dev):
+    # simple_matmul.py: M,K,N = 1024,6144,2048, both operands ~ N(0,1), row-major B, TP=4, batch halves
+    M, K, N = 1024, 6144, 2048
+    A = O.gaussian_bf16((M, K), 1.0, 0).to(dev)
+    B = O.gaussian_bf16((K, N), 1.0, 1).to(dev)
+    C = matmul_tp_persistent(A, B)
+    assert_bitwise(matmul_tp_persistent(A[:M // 2], B), C[:M // 2], "batch halves")
+    assert_bitwise(sim_tp(A, B, 4, 256), C, "TP=4")
+    want = O.matmul_tree(A[:64].cpu(), B.cpu())
+    assert_close_to_oracle(C[:64], want, "vs oracle")
+
+
+def test_tree_combine_matches_oracle_bitwise(dev):
+    for numel_shape in [(2048, 4096), (7, 33), (1, 5)]:
+        parts = [O.gaussian_bf16(numel_shape, 1.0, s) for s in range(8)]
+        for n in (1, 2, 4, 8):
+            got = tree_combine([p.to(dev) for p in parts[:n]])
+            assert_bitwise(got, O.tree_combine(parts[:n]), f"{numel_shape} n={n}")
+    # unaligned views take the scalar path: same bits
+    big = O.gaussian_bf16((4, 1001), 1.0, 9)
+    views = [big[i, 1:] for i in range(4)]
+    assert_bitwise(tree_combine([v.to(dev)[:] for v in views]), O.tree_combine(views), "unaligned")
+    flat = big.to(dev).reshape(-1)
+    shifted = [flat[1 + i * 1001: 1 + i * 1001 + 999] for i in range(4)]
+    assert_bitwise(tree_combine(shifted), O.tree_combine([s.cpu() for s in shifted]), "shifted views")

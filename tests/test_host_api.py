@@ -1,0 +1,153 @@
+"""Host-side contract of the plugin boundary and of the C ABI (no GPU, no compute calls)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import llm_reproducibility_amd as pkg
+from llm_reproducibility_amd import _lib, utils
+from llm_reproducibility_amd.tbik import choose_leaf_k, matmul_tp_persistent, tree_combine
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+FLAGS = ("VLLM_BATCH_INVARIANT", "VLLM_TP_INVARIANT", "ALIGN_TRAIN_INFERENCE", "TP_INVARIANT_MATMUL")
+
+
+@pytest.fixture(autouse=True)
+def clean_env(monkeypatch):
+    for f in FLAGS:
+        monkeypatch.delenv(f, raising=False)
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "tbik_hip.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b((?:tbik|bi)_[a-z0-9_]+)\s*\(", header))
+    assert declared == set(_lib.EXPORTS), declared ^ set(_lib.EXPORTS)
+    L = _lib.lib()
+    for name in declared:
+        assert hasattr(L, name), name
+    assert L.tbik_abi_version() == 1
+    assert L.tbik_error_string(0) == b"ok"
+    assert b"leaves" in L.tbik_error_string(1)
+
+
+def test_tree_params_through_the_c_abi():
+    assert _lib.tree_params(12288, 256) == (48, 3, 5)
+    assert _lib.tree_params(1536, 256) == (6, 3, 2)
+    assert _lib.tree_params(3200, 128) == (25, 25, 1)
+    with pytest.raises(ValueError):
+        _lib.tree_params(3200, 256)
+
+
+def test_host_argument_checks_fire_before_any_launch():
+    L = _lib.lib()
+    # null pointers / bad sizes are rejected on the host, so these are safe without a GPU
+    assert L.tbik_gemm_bf16(None, 0, None, 1, 0, None, 0, 4, 4, 256, 256, None, None) == _lib.TBIK_ERR_INVALID
+    buf = ctypes.create_string_buffer(64)
+    p = ctypes.addressof(buf)
+    p16 = (p + 15) & ~15
+    assert L.tbik_gemm_bf16(p16, 300, p16, 1, 300, p16, 8, 1, 8, 300, 256, None, None) == _lib.TBIK_ERR_ALIGNMENT
+    assert L.tbik_gemm_bf16(p16, 512, p16, 512, 1, p16, 8, 1, 8, 512, 256, None, None) == _lib.TBIK_ERR_UNSUPPORTED
+    assert L.tbik_gemm_bf16(p16 + 2, 512, p16, 1, 512, p16, 8, 1, 8, 512, 256, None, None) == _lib.TBIK_ERR_ALIGNMENT
+    assert L.tbik_gemm_bf16(p16, 384, p16, 1, 384, p16, 8, 1, 8, 384, 256, None, None) == _lib.TBIK_ERR_INVALID
+    arr = (ctypes.c_void_p * 3)(p16, p16, p16)
+    assert L.tbik_tree_combine_bf16(arr, 3, p16, 8, None) == _lib.TBIK_ERR_INVALID
+    assert L.bi_log_softmax_f32(p16, 8, p16, 8, 1, 8, None, 0, 0, None) == _lib.TBIK_ERR_WORKSPACE
+    assert L.bi_log_softmax_workspace_bytes(7, 151936) == 7 * 38 * 8
+    assert L.bi_rmsnorm_bf16(p16, 12, None, 0, None, p16, 12, None, 0, 1, 12, 1e-6, None) == _lib.TBIK_ERR_ALIGNMENT
+    assert L.bi_mean_dim(p16, p16, 1, 4, 1, 7, None) == _lib.TBIK_ERR_UNSUPPORTED
+    with pytest.raises(_lib.TbikError):
+        _lib.check(_lib.TBIK_ERR_ALIGNMENT, "x")
+
+
+def test_env_flags(monkeypatch):
+    assert not utils.batch_invariant_is_enabled() and not utils.tp_invariant_is_enabled()
+    monkeypatch.setenv("VLLM_BATCH_INVARIANT", "1")
+    assert utils.batch_invariant_is_enabled()
+    monkeypatch.setenv("VLLM_BATCH_INVARIANT", "yes")      # does not parse -> off
+    assert not utils.batch_invariant_is_enabled()
+    monkeypatch.setenv("VLLM_TP_INVARIANT", "1")
+    with pytest.raises(AssertionError):                     # TP invariance requires batch invariance
+        utils.tp_invariant_is_enabled()
+    monkeypatch.setenv("VLLM_BATCH_INVARIANT", "2")
+    assert utils.tp_invariant_is_enabled() and utils.check_invariant_compat()
+    monkeypatch.setenv("ALIGN_TRAIN_INFERENCE", "1")
+    assert utils.compatible_mode_is_enabled()
+    monkeypatch.setenv("TP_INVARIANT_MATMUL", "1")
+    assert utils.tp_invariant_matmul_is_enabled()
+
+
+def test_apply_patches_dispatch(monkeypatch, capsys):
+    from llm_reproducibility_amd import layers, patch
+    from llm_reproducibility_amd.bio import batch_invariant_ops as bio
+    import importlib
+    ptp = importlib.import_module("llm_reproducibility_amd.patch.patch_tp_invariant")
+    calls = []
+    monkeypatch.setattr(patch, "patch_batch_invariant", lambda: calls.append("bi"))
+    monkeypatch.setattr(patch, "patch_tp_invariant", lambda: calls.append("tp"))
+    monkeypatch.setattr(patch, "patch_align", lambda: calls.append("align"))
+    monkeypatch.setattr(patch, "patch_training_baseline", lambda: calls.append("base"))
+    pkg.apply_patches()
+    assert calls == ["base"]
+    calls.clear()
+    monkeypatch.setenv("VLLM_BATCH_INVARIANT", "1")
+    pkg.apply_patches()
+    assert calls == ["bi"]
+    calls.clear()
+    monkeypatch.setenv("VLLM_TP_INVARIANT", "1")
+    monkeypatch.setenv("ALIGN_TRAIN_INFERENCE", "1")
+    pkg.apply_patches()
+    assert calls == ["bi", "tp", "align"]
+    calls.clear()
+    monkeypatch.delenv("VLLM_BATCH_INVARIANT")
+    monkeypatch.delenv("VLLM_TP_INVARIANT")
+    pkg.apply_patches()
+    assert calls == ["base"]
+    monkeypatch.undo()
+    # the real TP patch swaps the forward of the row-parallel layer and can be undone
+    stock = layers.RowParallelLinear.forward
+    ptp.patch_tp_invariant()
+    assert layers.RowParallelLinear.forward is layers.tbik_row_parallel_forward
+    ptp.unpatch_row_linear()
+    assert layers.RowParallelLinear.forward is stock
+    # mode switches are idempotent and restorable
+    assert not bio.is_batch_invariant_mode_enabled()
+    with bio.set_batch_invariant_mode(True):
+        assert bio.is_batch_invariant_mode_enabled()
+        bio.enable_batch_invariant_mode()
+    assert not bio.is_batch_invariant_mode_enabled()
+    capsys.readouterr()
+
+
+def test_leaf_choice_is_a_property_of_the_layer():
+    assert choose_leaf_k(12288) == 256 and choose_leaf_k(8192) == 256 and choose_leaf_k(4096) == 256
+    assert choose_leaf_k(25600) == 128            # 25600 / 8 = 3200 = 25 * 128
+    assert choose_leaf_k(25600, max_tp=4) == 256
+    with pytest.raises(ValueError):
+        choose_leaf_k(1000)
+
+
+def test_operator_errors_match_the_reference_contract():
+    a = torch.zeros((4, 512), dtype=torch.bfloat16)
+    with pytest.raises(AssertionError, match="Dim doesn't match"):
+        matmul_tp_persistent(a, torch.zeros((256, 8), dtype=torch.bfloat16))
+    with pytest.raises(AssertionError):
+        matmul_tp_persistent(torch.zeros((4, 384), dtype=torch.bfloat16), torch.zeros((384, 8), dtype=torch.bfloat16))
+    with pytest.raises(NotImplementedError):
+        matmul_tp_persistent(a.float(), torch.zeros((512, 8)))
+    with pytest.raises(ValueError):
+        tree_combine([a, a, a])
+    # there is no CPU path: CPU tensors fail loudly instead of falling back
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        matmul_tp_persistent(a, torch.zeros((512, 8), dtype=torch.bfloat16))
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        tree_combine([a, a])
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libtbik_hip.so"))
+    with pytest.raises(RuntimeError, match="only implementation"):
+        _lib.lib()

@@ -1,0 +1,75 @@
+"""Pins the CPU oracles of the batch-invariant reductions against library routines and closed forms (no GPU)."""
+import math
+
+import pytest
+import torch
+
+from oracle import tbik_oracle as O
+
+
+def test_log_softmax_matches_float64_library_and_closed_forms():
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn((7, 151936), generator=g) * 3.0
+    want = torch.log_softmax(x.double(), dim=-1)
+    got = O.log_softmax_lastdim(x)
+    assert (got.double() - want).abs().max() < 2e-5
+    # constant row: -log(V) everywhere
+    c = torch.full((2, 1000), 4.25)
+    assert torch.allclose(O.log_softmax_lastdim(c), torch.full((2, 1000), -math.log(1000.0)), atol=1e-6)
+    # one dominant entry: ~0 there, ~(x - big) elsewhere
+    d = torch.zeros((1, 64))
+    d[0, 5] = 100.0
+    r = O.log_softmax_lastdim(d)
+    assert abs(r[0, 5].item()) < 1e-6 and abs(r[0, 0].item() + 100.0) < 1e-4
+    # (the CPU library reduction is itself not batch invariant -- its blocking depends on the shape --
+    # so rows computed alone agree with rows computed in a batch only to rounding)
+    assert (O.log_softmax_lastdim(x[2:3]) - got[2:3]).abs().max() < 1e-5
+
+
+def test_mean_matches_integers_and_float64():
+    x = torch.arange(0, 4096, dtype=torch.float32).repeat(3, 1)
+    assert torch.equal(O.mean_lastdim(x), torch.full((3,), 2047.5))
+    g = torch.Generator().manual_seed(1)
+    y = torch.randn((5, 4096), generator=g)
+    assert (O.mean_lastdim(y).double() - y.double().mean(-1)).abs().max() < 1e-6
+
+
+def test_rmsnorm_matches_textbook_float64_and_hf_module():
+    x = O.gaussian_bf16((9, 4096), 1.0, 2)
+    w = (1.0 + 0.1 * torch.randn(4096, generator=torch.Generator().manual_seed(3))).to(torch.bfloat16)
+    eps = 1e-6
+    got = O.rmsnorm(x, w, eps)
+    xd = x.double()
+    want = xd * torch.rsqrt(xd.pow(2).mean(-1, keepdim=True) + eps)
+    want = want.to(torch.bfloat16).double() * w.double()
+    assert O.bf16_ulp_distance(got, want.to(torch.bfloat16)).max() <= 1
+    # Hugging Face's Qwen3RMSNorm (installed library, same published formula up to where the weight is applied)
+    tr = pytest.importorskip("transformers.models.qwen3.modeling_qwen3")
+    mod = tr.Qwen3RMSNorm(4096, eps=eps)
+    with torch.no_grad():
+        mod.weight.copy_(w.float())
+    hf = mod(x.float())
+    assert (got.float() - hf).abs().max() <= 2 ** -7 * hf.abs().max()
+    # +-1 row, unit weight: x * rsqrt(1 + eps)
+    s = torch.ones((1, 4096), dtype=torch.bfloat16)
+    s[0, ::2] = -1
+    r = O.rmsnorm(s, torch.ones(4096, dtype=torch.bfloat16), eps)
+    assert torch.equal(r, s)
+
+
+def test_rmsnorm_residual_semantics():
+    x = O.gaussian_bf16((4, 512), 1.0, 4)
+    res = O.gaussian_bf16((4, 512), 1.0, 5)
+    w = torch.ones(512, dtype=torch.bfloat16)
+    y, new_res = O.rmsnorm(x, w, 1e-6, residual=res)
+    assert torch.equal(new_res, (x.float() + res.float()).to(torch.bfloat16))
+    s = x.float() + res.float()          # the normalisation sees the UNROUNDED fp32 sum
+    want = (s * torch.rsqrt(s.pow(2).mean(-1, keepdim=True) + 1e-6)).to(torch.bfloat16)
+    assert torch.equal(y, want)
+
+
+def test_single_accumulator_matmul_is_one_rounding_of_the_fp32_product():
+    a = O.gaussian_bf16((8, 320), 1.0, 6)
+    b = O.gaussian_bf16((320, 24), 0.1, 7)
+    bias = O.gaussian_bf16((24,), 1.0, 8)
+    assert torch.equal(O.matmul_single_acc(a, b, bias), (a.float() @ b.float() + bias.float()).to(torch.bfloat16))
