@@ -266,3 +266,11 @@ def bf16_ulp_distance(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
         i = t.contiguous().view(torch.int16).to(torch.int32) & 0xFFFF
         return torch.where(i >= 0x8000, 0x8000 - i, i)
     return (key(a) - key(b)).abs()
+
+
+def outside_tolerance(got: torch.Tensor, want: torch.Tensor) -> torch.Tensor:
+    """Mask of elements that violate the stated tolerance for random inputs: more than 1 bf16 ulp from the
+    oracle AND more than 2^-8 of the output scale (max |want|) away in absolute terms."""
+    got, want = got.cpu(), want.cpu()
+    scale = want.float().abs().max()
+    return (bf16_ulp_distance(got, want) > 1) & ((got.float() - want.float()).abs() > 2.0 ** -8 * scale)

@@ -27,7 +27,7 @@ def test_simulated_tp_row_linear_is_tp_and_batch_invariant(dev):
 
 def test_patched_row_parallel_linear_matches_tree_matmul(dev):
     ptp = importlib.import_module("llm_reproducibility_amd.patch.patch_tp_invariant")
-    layer = layers.RowParallelLinear(1536, 128, bias=True, tp_rank=0, tp_size=1, device=dev)
+    layer = layers.RowParallelLinear(1536, 128, bias=True, tp_rank=0, tp_size=1, max_tp=2, device=dev)
     layer.weight.copy_(O.integer_bf16((128, 1536), -7, 7, 0).to(dev))
     layer.bias.copy_(O.integer_bf16((128,), -100, 100, 1).to(dev))
     x = O.integer_bf16((3, 5, 1536), -9, 9, 2).to(dev)

