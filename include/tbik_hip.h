@@ -56,6 +56,7 @@ int tbik_tree_params(int K, int leaf_k, int* T, int* flb, int* level_k);
  *      weight.t()) is the native layout; ldb_n == 1 (row-major [K,N]) returns
  *      TBIK_ERR_UNSUPPORTED in this build and is repacked by the caller.
  *   C: element (m,n) at C[m*ldc + n]
+ *   workspace: at least tbik_gemm_workspace_bytes(M,N,K,leaf_k) bytes, 16-byte aligned (may be NULL when 0)
  * Replaces: matmul_tp_persistent + matmul_kernel_tp_persistent,
  *           src/tbik/tree_based_matmul.py:190-277 and :50-187.
  */
@@ -64,7 +65,16 @@ int tbik_gemm_bf16(const void* A, int64_t lda,
                    void* C, int64_t ldc,
                    int M, int N, int K, int leaf_k,
                    const void* bias_or_null,
+                   void* workspace, size_t workspace_bytes,
                    tbik_stream_t stream);
+
+/*
+ * Bytes of device workspace tbik_gemm_bf16 needs for this problem (0 for small problems).  The
+ * large-M kernel parks the upper levels of the merge tree there; its contents are scratch, but two
+ * launches that run concurrently must not share it.
+ * Replaces: the in-register tensor `S` of the reference kernel, src/tbik/tree_based_matmul.py:85.
+ */
+size_t tbik_gemm_workspace_bytes(int M, int N, int K, int leaf_k);
 
 /*
  * out[i] = adjacent-pair binary tree over parts[0..nparts-1][i], bf16 adds (round to nearest even

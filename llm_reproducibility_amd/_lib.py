@@ -11,6 +11,7 @@ import os
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG_DIR, "libtbik_hip.so")
 
+ABI_VERSION = 2
 TBIK_OK = 0
 TBIK_ERR_INVALID = 1
 TBIK_ERR_ALIGNMENT = 2
@@ -18,7 +19,8 @@ TBIK_ERR_UNSUPPORTED = 3
 TBIK_ERR_WORKSPACE = 4
 
 EXPORTS = (
-    "tbik_abi_version", "tbik_error_string", "tbik_tree_params", "tbik_gemm_bf16", "tbik_tree_combine_bf16",
+    "tbik_abi_version", "tbik_error_string", "tbik_tree_params", "tbik_gemm_bf16", "tbik_gemm_workspace_bytes",
+    "tbik_tree_combine_bf16",
     "bi_gemm_bf16", "bi_rmsnorm_bf16", "bi_log_softmax_workspace_bytes", "bi_log_softmax_f32", "bi_mean_dim",
 )
 
@@ -49,7 +51,9 @@ def lib() -> ctypes.CDLL:
     L.tbik_error_string.restype = ctypes.c_char_p
     L.tbik_tree_params.argtypes = [i32, i32, pi32, pi32, pi32]
     L.tbik_tree_params.restype = i32
-    L.tbik_gemm_bf16.argtypes = [vp, i64, vp, i64, i64, vp, i64, i32, i32, i32, i32, vp, vp]
+    L.tbik_gemm_bf16.argtypes = [vp, i64, vp, i64, i64, vp, i64, i32, i32, i32, i32, vp, vp, sz, vp]
+    L.tbik_gemm_workspace_bytes.argtypes = [i32, i32, i32, i32]
+    L.tbik_gemm_workspace_bytes.restype = sz
     L.tbik_gemm_bf16.restype = i32
     L.tbik_tree_combine_bf16.argtypes = [ctypes.POINTER(vp), i32, vp, i64, vp]
     L.tbik_tree_combine_bf16.restype = i32
@@ -63,8 +67,8 @@ def lib() -> ctypes.CDLL:
     L.bi_log_softmax_f32.restype = i32
     L.bi_mean_dim.argtypes = [vp, vp, i64, i64, i64, i32, vp]
     L.bi_mean_dim.restype = i32
-    if L.tbik_abi_version() != 1:
-        raise RuntimeError(f"{LIB_PATH}: ABI version {L.tbik_abi_version()} does not match this package (1)")
+    if L.tbik_abi_version() != ABI_VERSION:
+        raise RuntimeError(f"{LIB_PATH}: ABI version {L.tbik_abi_version()} does not match this package ({ABI_VERSION})")
     _lib = L
     return L
 

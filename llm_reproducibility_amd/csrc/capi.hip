@@ -4,7 +4,9 @@
 
 namespace tbik {
 int gemm_dispatch(bool tree, const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C,
-                  int64_t ldc, int M, int N, int K, int leaf_k, const void* bias, hipStream_t stream);
+                  int64_t ldc, int M, int N, int K, int leaf_k, const void* bias, void* ws, size_t ws_bytes,
+                  hipStream_t stream);
+size_t gemm_workspace_bytes(int M, int N, int K, int leaf_k);
 int tree_combine_dispatch(const void* const* parts, int nparts, void* out, int64_t numel, hipStream_t stream);
 int rmsnorm_dispatch(const void* x, int64_t ldx, const void* res, int64_t ldr, const void* w, void* out, int64_t ldo,
                      void* res_out, int64_t ldro, int64_t rows, int hidden, float eps, hipStream_t stream);
@@ -16,7 +18,7 @@ int mean_dispatch(const void* x, void* out, int64_t outer, int64_t n, int64_t in
 
 extern "C" {
 
-int tbik_abi_version(void) { return 1; }
+int tbik_abi_version(void) { return 2; }
 
 const char* tbik_error_string(int code) {
   switch (code) {
@@ -42,10 +44,13 @@ int tbik_tree_params(int K, int leaf_k, int* T, int* flb, int* level_k) {
   return TBIK_OK;
 }
 
+size_t tbik_gemm_workspace_bytes(int M, int N, int K, int leaf_k) { return tbik::gemm_workspace_bytes(M, N, K, leaf_k); }
+
 int tbik_gemm_bf16(const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C, int64_t ldc, int M,
-                   int N, int K, int leaf_k, const void* bias_or_null, tbik_stream_t stream) {
-  return tbik::gemm_dispatch(true, A, lda, B, ldb_k, ldb_n, C, ldc, M, N, K, leaf_k, bias_or_null,
-                             static_cast<hipStream_t>(stream));
+                   int N, int K, int leaf_k, const void* bias_or_null, void* workspace, size_t workspace_bytes,
+                   tbik_stream_t stream) {
+  return tbik::gemm_dispatch(true, A, lda, B, ldb_k, ldb_n, C, ldc, M, N, K, leaf_k, bias_or_null, workspace,
+                             workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
 int tbik_tree_combine_bf16(const void* const* parts, int nparts, void* out, int64_t numel, tbik_stream_t stream) {
@@ -54,7 +59,7 @@ int tbik_tree_combine_bf16(const void* const* parts, int nparts, void* out, int6
 
 int bi_gemm_bf16(const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C, int64_t ldc, int M,
                  int N, int K, const void* bias_or_null, tbik_stream_t stream) {
-  return tbik::gemm_dispatch(false, A, lda, B, ldb_k, ldb_n, C, ldc, M, N, K, 0, bias_or_null,
+  return tbik::gemm_dispatch(false, A, lda, B, ldb_k, ldb_n, C, ldc, M, N, K, 0, bias_or_null, nullptr, 0,
                              static_cast<hipStream_t>(stream));
 }
 

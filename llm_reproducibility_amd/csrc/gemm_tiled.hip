@@ -316,8 +316,37 @@ static int launch_tree(const GemmArgs& a, hipStream_t stream) {
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
+// large-M kernel (gemm_tree_wide.hip)
+struct WideArgs {
+  const uint16_t* X;
+  const uint16_t* W;
+  uint16_t* C;
+  const uint16_t* bias;
+  u32x4* ws;
+  int64_t ldx, ldw, ldc;
+  int M, N, K;
+  int T, flb, lb;
+  int vec_store;
+};
+size_t wide_workspace_bytes(int M, int N, int lb);
+int gemm_tree_wide_launch(const WideArgs& a, int leaf_k, hipStream_t stream);
+
+// The wide kernel pays off once its 128x256 tiles can occupy the chip; below that the 128x128 / 64x128 /
+// 16x64 tiles of this file give more work-groups.  The choice never changes the result.
+static bool use_wide(int M, int N) {
+  const int64_t wide_tiles = (int64_t)((M + 127) / 128) * ((N + 255) / 256);
+  return M > 64 && wide_tiles >= 128;
+}
+
+size_t gemm_workspace_bytes(int M, int N, int K, int leaf_k) {
+  int T, flb, level_k;
+  if (M <= 0 || N <= 0 || tbik_tree_params(K, leaf_k, &T, &flb, &level_k) != TBIK_OK) return 0;
+  return use_wide(M, N) ? wide_workspace_bytes(M, N, level_k - 1) : 0;
+}
+
 int gemm_dispatch(bool tree, const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C,
-                  int64_t ldc, int M, int N, int K, int leaf_k, const void* bias, hipStream_t stream) {
+                  int64_t ldc, int M, int N, int K, int leaf_k, const void* bias, void* ws, size_t ws_bytes,
+                  hipStream_t stream) {
   if (!A || !B || !C || M < 0 || N < 0 || K <= 0) return TBIK_ERR_INVALID;
   if (M == 0 || N == 0) return TBIK_OK;
   if (ldb_k != 1) return TBIK_ERR_UNSUPPORTED;  // row-major [K,N] weights are repacked by the caller
@@ -347,6 +376,13 @@ int gemm_dispatch(bool tree, const void* A, int64_t lda, const void* B, int64_t 
   a.T = T;
   a.flb = flb;
   a.lb = level_k - 1;
+  if (leaf_k != 256 && leaf_k != 128) return TBIK_ERR_UNSUPPORTED;
+  if (use_wide(M, N)) {
+    const size_t need = wide_workspace_bytes(M, N, a.lb);
+    if (need > 0 && (!ws || ws_bytes < need || !aligned16(ws))) return TBIK_ERR_WORKSPACE;
+    WideArgs w{a.X, a.W, a.C, a.bias, static_cast<u32x4*>(ws), a.ldx, a.ldw, a.ldc, M, N, K, T, flb, a.lb, a.vec_store};
+    return gemm_tree_wide_launch(w, leaf_k, stream);
+  }
   if (leaf_k == 256) return launch_tree<4>(a, stream);
   if (leaf_k == 128) return launch_tree<2>(a, stream);
   return TBIK_ERR_UNSUPPORTED;

@@ -61,8 +61,12 @@ def gemm_tree_bf16(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.Tensor
     w, ldw = _weight_nk(B)
     b = None if bias is None else bias.contiguous()
     C = torch.empty((M, N), device=A.device, dtype=torch.bfloat16)
-    rc = _lib.lib().tbik_gemm_bf16(a.data_ptr(), lda, w.data_ptr(), 1, ldw, C.data_ptr(), C.stride(0),
-                                   M, N, K, leaf_k, None if b is None else b.data_ptr(), _stream(A))
+    L = _lib.lib()
+    ws_bytes = L.tbik_gemm_workspace_bytes(M, N, K, leaf_k)
+    ws = torch.empty(ws_bytes, device=A.device, dtype=torch.uint8) if ws_bytes else None
+    rc = L.tbik_gemm_bf16(a.data_ptr(), lda, w.data_ptr(), 1, ldw, C.data_ptr(), C.stride(0),
+                          M, N, K, leaf_k, None if b is None else b.data_ptr(),
+                          None if ws is None else ws.data_ptr(), ws_bytes, _stream(A))
     _lib.check(rc, "tbik_gemm_bf16")
     return C
 

@@ -28,7 +28,7 @@ def test_library_exports_every_declared_symbol():
     L = _lib.lib()
     for name in declared:
         assert hasattr(L, name), name
-    assert L.tbik_abi_version() == 1
+    assert L.tbik_abi_version() == _lib.ABI_VERSION
     assert L.tbik_error_string(0) == b"ok"
     assert b"leaves" in L.tbik_error_string(1)
 
@@ -44,14 +44,14 @@ def test_tree_params_through_the_c_abi():
 def test_host_argument_checks_fire_before_any_launch():
     L = _lib.lib()
     # null pointers / bad sizes are rejected on the host, so these are safe without a GPU
-    assert L.tbik_gemm_bf16(None, 0, None, 1, 0, None, 0, 4, 4, 256, 256, None, None) == _lib.TBIK_ERR_INVALID
+    assert L.tbik_gemm_bf16(None, 0, None, 1, 0, None, 0, 4, 4, 256, 256, None, None, 0, None) == _lib.TBIK_ERR_INVALID
     buf = ctypes.create_string_buffer(64)
     p = ctypes.addressof(buf)
     p16 = (p + 15) & ~15
-    assert L.tbik_gemm_bf16(p16, 300, p16, 1, 300, p16, 8, 1, 8, 300, 256, None, None) == _lib.TBIK_ERR_ALIGNMENT
-    assert L.tbik_gemm_bf16(p16, 512, p16, 512, 1, p16, 8, 1, 8, 512, 256, None, None) == _lib.TBIK_ERR_UNSUPPORTED
-    assert L.tbik_gemm_bf16(p16 + 2, 512, p16, 1, 512, p16, 8, 1, 8, 512, 256, None, None) == _lib.TBIK_ERR_ALIGNMENT
-    assert L.tbik_gemm_bf16(p16, 384, p16, 1, 384, p16, 8, 1, 8, 384, 256, None, None) == _lib.TBIK_ERR_INVALID
+    assert L.tbik_gemm_bf16(p16, 300, p16, 1, 300, p16, 8, 1, 8, 300, 256, None, None, 0, None) == _lib.TBIK_ERR_ALIGNMENT
+    assert L.tbik_gemm_bf16(p16, 512, p16, 512, 1, p16, 8, 1, 8, 512, 256, None, None, 0, None) == _lib.TBIK_ERR_UNSUPPORTED
+    assert L.tbik_gemm_bf16(p16 + 2, 512, p16, 1, 512, p16, 8, 1, 8, 512, 256, None, None, 0, None) == _lib.TBIK_ERR_ALIGNMENT
+    assert L.tbik_gemm_bf16(p16, 384, p16, 1, 384, p16, 8, 1, 8, 384, 256, None, None, 0, None) == _lib.TBIK_ERR_INVALID
     arr = (ctypes.c_void_p * 3)(p16, p16, p16)
     assert L.tbik_tree_combine_bf16(arr, 3, p16, 8, None) == _lib.TBIK_ERR_INVALID
     assert L.bi_log_softmax_f32(p16, 8, p16, 8, 1, 8, None, 0, 0, None) == _lib.TBIK_ERR_WORKSPACE
