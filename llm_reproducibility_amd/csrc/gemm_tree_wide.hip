@@ -1,19 +1,25 @@
 // Tree-ordered bf16 GEMM for gfx950, large-M path: 128x256 output tile per work-group, 8 wavefronts
-// (2 per SIMD) of 64x64 each, K staged through LDS in 64-element slices.
+// (2 per SIMD) of 64x64 each, K streamed through a 3-slot LDS ring in 64-element slices.
 //
 // Same arithmetic contract as gemm_tiled.hip (and therefore the same bits): per leaf a chain of
 // 16x16x32 bf16 MFMAs over k in ascending order into a zeroed fp32 accumulator, one rounding to bf16,
 // then the binary-counter merge (level 0 left-to-right over FLB leaves, adjacent pairs above), every
 // node rounded to bf16.  Replaces matmul_kernel_tp_persistent, src/tbik/tree_based_matmul.py:50-187.
 //
-// What differs is where the partials live and when the merge runs:
-//   * only the running level-0 sum and the first binary level stay in registers; deeper levels are
-//     parked in a global workspace (each lane reads back exactly the bytes it wrote, 16 B per lane,
-//     fully coalesced).  They are touched once per 2, 4, 8 ... groups, so the traffic is a few percent
-//     of the operand traffic, and the register file keeps room for two waves per SIMD.
+// How it is arranged for CDNA4:
+//   * operands go global -> LDS directly (global_load_lds_dwordx4), two K slices ahead of the MFMAs;
+//     a lane picks the global chunk that belongs at its (linear) LDS position, which realises the XOR
+//     bank swizzle on the source side.  One barrier per slice.
+//   * the running level-0 sum and the first binary level of the merge tree stay in registers as packed
+//     bf16; deeper levels (touched once per 2, 4, ... groups) are parked in a global workspace, each
+//     lane reading back exactly the 16-byte words it wrote.  The level that is popped most often is
+//     brought back through the same direct global->LDS path one K slice ahead of its use.
 //   * the merge of leaf j is deferred into leaf j+1: the finished accumulator is only packed to bf16
-//     (which frees it for the next leaf's first MFMA), and a quarter of the tiles is merged in each of
-//     the next leaf's K slices, so the VALU work rides in the shadow of the MFMAs.
+//     (which frees it for the next leaf's first MFMA); a quarter of the tiles is merged in each of the
+//     next leaf's K slices.  The leaf body is instantiated once per merge kind so that every slice is
+//     straight-line code and the VALU work can issue in the shadow of the MFMAs.
+#include <type_traits>
+
 #include "common.h"
 
 namespace tbik {
@@ -33,15 +39,16 @@ struct WideArgs {
 namespace wide {
 constexpr int BM = 128, BN = 256, BK = 64;
 constexpr int NT = 512;
-constexpr int TM = 4, TN = 4;             // 16x16 MFMA tiles per wave: 64x64
-constexpr int STAGE = (BM + BN) * BK;     // bf16 elements per LDS stage
-constexpr int XCH = BM * 8 / NT;          // 16-byte chunks per thread per stage: 2
-constexpr int WCH = BN * 8 / NT;          // 4
-constexpr int RL = 1;                     // binary levels kept in registers
-constexpr int NTILE = TM * TN;            // 16 tiles, each 2 packed registers per lane
-constexpr int MAXLB = 12;
-
-__device__ __forceinline__ int lds_off(int r, int c) { return r * BK + ((c ^ (r & 7)) << 3); }
+constexpr int TM = 4, TN = 4;                 // 16x16 MFMA tiles per wave: 64x64
+constexpr int ROWS = BM + BN;                 // LDS rows per slice: X rows, then W rows
+constexpr int STAGE_BYTES = ROWS * BK * 2;    // 48 KiB
+constexpr int NSLOT = 3;
+constexpr int NDMA = ROWS / 8 / (NT / 64);    // direct loads per wave per slice: 6 (8 rows of 128 B each)
+constexpr int RL = 1;                         // binary levels kept in registers
+constexpr int SPARE_OFF = NSLOT * STAGE_BYTES; // 16 KiB behind the ring: staging of a parked level, 2 KiB per wave
+constexpr int NREG = TM * TN * 2;             // packed bf16x2 registers per lane per level: 32
+constexpr int MAXLB = 16;
+enum Kind { K_NONE = 0, K_ADD = 1, K_P0 = 2, K_P1 = 3, K_P2 = 4 };
 }  // namespace wide
 
 size_t wide_workspace_bytes(int M, int N, int lb) {
@@ -51,14 +58,22 @@ size_t wide_workspace_bytes(int M, int N, int lb) {
   return (size_t)(lb - RL) * tiles * (NT / 64) * 8 * 64 * sizeof(u32x4);
 }
 
+// One 16-byte-per-lane direct global->LDS load: lane l's 16 bytes land at lds_addr + 16*l.
+__device__ __forceinline__ void dma16(uint32_t lds_addr, uint32_t voff, const void* base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(base)
+               : "memory");
+}
+
 template <int LS>
 __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs p) {
   using namespace wide;
-  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 2;  // 0..1
   const int wn = wave & 3;   // 0..3
 
@@ -81,138 +96,144 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
   const int tile_id = pid_m * tiles_n + pid_n;
   const int ntiles = tiles_m * tiles_n;
 
-  // ---- global -> register -> LDS staging
-  const uint16_t* xptr[XCH];
-  const uint16_t* wptr[WCH];
-  int xdst[XCH], wdst[WCH];
+  // ---- direct global->LDS loads.  Wave w's i-th load of a slice fills LDS rows [8*(8i+w), +8): lane l
+  // lands at row 8*(8i+w) + l/8, physical 16-byte chunk l%8, so it fetches logical chunk (l%8)^(l/8).
+  const uint8_t* xbase = reinterpret_cast<const uint8_t*>(p.X + (int64_t)m0 * p.ldx);
+  const uint8_t* wbase = reinterpret_cast<const uint8_t*>(p.W + (int64_t)n0 * p.ldw);
+  uint32_t voff[NDMA];
+  {
+    const int r = lane >> 3, c = (lane & 7) ^ r;
 #pragma unroll
-  for (int i = 0; i < XCH; i++) {
-    const int q = tid + i * NT;
-    const int r = q >> 3, c = q & 7;
-    xptr[i] = p.X + (int64_t)min(m0 + r, p.M - 1) * p.ldx + c * 8;
-    xdst[i] = lds_off(r, c);
+    for (int i = 0; i < NDMA; i++) {
+      const int row = (i * 8 + wave) * 8 + r;  // 0..383
+      if (i < 2) {
+        const int gr = min(m0 + row, p.M - 1) - m0;
+        voff[i] = (uint32_t)((gr * p.ldx + c * 8) * 2);
+      } else {
+        const int gr = min(n0 + row - BM, p.N - 1) - n0;
+        voff[i] = (uint32_t)((gr * p.ldw + c * 8) * 2);
+      }
+    }
   }
+  const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
+  auto issue_slice = [&](int s, int slot) __attribute__((always_inline)) {
+    const uint8_t* xb = xbase + (int64_t)s * (BK * 2);
+    const uint8_t* wb = wbase + (int64_t)s * (BK * 2);
+    const uint32_t dst = lds0 + slot * STAGE_BYTES + wave * 1024;
 #pragma unroll
-  for (int i = 0; i < WCH; i++) {
-    const int q = tid + i * NT;
-    const int r = q >> 3, c = q & 7;
-    wptr[i] = p.W + (int64_t)min(n0 + r, p.N - 1) * p.ldw + c * 8;
-    wdst[i] = BM * BK + lds_off(r, c);
-  }
-  u32x4 xreg[XCH], wreg[WCH];
-  auto load_stage = [&](int s) __attribute__((always_inline)) {
-    const int k0 = s * BK;
-#pragma unroll
-    for (int i = 0; i < XCH; i++) xreg[i] = *reinterpret_cast<const u32x4*>(xptr[i] + k0);
-#pragma unroll
-    for (int i = 0; i < WCH; i++) wreg[i] = *reinterpret_cast<const u32x4*>(wptr[i] + k0);
-  };
-  auto store_stage = [&](int buf) __attribute__((always_inline)) {
-#pragma unroll
-    for (int i = 0; i < XCH; i++) *reinterpret_cast<u32x4*>(smem + buf * STAGE + xdst[i]) = xreg[i];
-#pragma unroll
-    for (int i = 0; i < WCH; i++) *reinterpret_cast<u32x4*>(smem + buf * STAGE + wdst[i]) = wreg[i];
+    for (int i = 0; i < NDMA; i++) dma16(dst + i * 8192, voff[i], i < 2 ? xb : wb);
   };
 
+  // ---- fragment addressing (bytes): lane l reads row (l%16), chunk (kk*4 + l/16) ^ (row & 7)
   const int frow = lane & 15;
   const int fchk = lane >> 4;
+  const uint32_t xfrag = ((wm * TM * 16 + frow) * BK + ((fchk ^ (frow & 7)) << 3)) * 2;
+  const uint32_t wfrag = (BM * BK + (wn * TN * 16 + frow) * BK + ((fchk ^ (frow & 7)) << 3)) * 2;
 
   f32x4 acc[TM][TN];
-  uint32_t t[NTILE][2];    // packed leaf waiting to be merged (leaf j while leaf j+1 is computed)
-  uint32_t s0[NTILE][2];   // level 0 running sum
-  uint32_t sb0[NTILE][2];  // first binary level
-  // merge state of the leaf held in t (uniform over the block)
-  int c0 = 0;  // leaves already absorbed at level 0 before that leaf
-  int g = 0;   // groups completed before that leaf
+  uint32_t t[NREG];    // packed leaf waiting to be merged (leaf j while leaf j+1 is computed)
+  uint32_t s0[NREG];   // level 0 running sum
+  uint32_t sb0[NREG];  // binary level 0
+  int c0 = 0;          // leaves absorbed at level 0 in the current group
+  int g = 0;           // groups completed
+  int g_pending = 0;   // value of g for the leaf held in t
 
-  // parked levels: level l >= RL, this wave's 8 chunks of 16 B per lane
   auto ws_ptr = [&](int l, int chunk) __attribute__((always_inline)) -> u32x4* {
     return p.ws + ((((int64_t)(l - RL) * ntiles + tile_id) * (NT / 64) + wave) * 8 + chunk) * 64 + lane;
   };
 
-  // Merge tiles [4q, 4q+4) of the leaf in t into the stack; returns with t = the node that left the stack
-  // when the whole tree completed (only meaningful for the last leaf).
-  auto merge_quarter = [&](int q) __attribute__((always_inline)) {
-    if (c0 != 0) {
+  // Parked levels for quarter q (tiles 4q..4q+3 = registers 8q..8q+7 = chunks 2q, 2q+1): continue the carry
+  // chain from level `from` with counter value gg.  Stops at the first clear bit (parks there) or after lb.
+  auto chain_parked = [&](int q, int from, int gg) __attribute__((always_inline)) {
+    for (int l = from; l < p.lb; l++) {
+      u32x4* w0 = ws_ptr(l, 2 * q);
+      u32x4* w1 = ws_ptr(l, 2 * q + 1);
+      if ((gg >> l) & 1) {
+        const u32x4 a = *w0, b = *w1;
 #pragma unroll
-      for (int i = 0; i < 4; i++) {
-        t[4 * q + i][0] = add_bf16x2(s0[4 * q + i][0], t[4 * q + i][0]);
-        t[4 * q + i][1] = add_bf16x2(s0[4 * q + i][1], t[4 * q + i][1]);
-      }
-    }
-    if (c0 + 1 == p.flb) {
-      bool parked = false;
-      if (p.lb > 0) {
-        if (g & 1) {
-#pragma unroll
-          for (int i = 0; i < 4; i++) {
-            t[4 * q + i][0] = add_bf16x2(sb0[4 * q + i][0], t[4 * q + i][0]);
-            t[4 * q + i][1] = add_bf16x2(sb0[4 * q + i][1], t[4 * q + i][1]);
-          }
-        } else {
-#pragma unroll
-          for (int i = 0; i < 4; i++) {
-            sb0[4 * q + i][0] = t[4 * q + i][0];
-            sb0[4 * q + i][1] = t[4 * q + i][1];
-          }
-          parked = true;
+        for (int e = 0; e < 4; e++) {
+          t[8 * q + e] = add_bf16x2(a[e], t[8 * q + e]);
+          t[8 * q + 4 + e] = add_bf16x2(b[e], t[8 * q + 4 + e]);
         }
-      }
-      for (int l = RL; l < p.lb && !parked; l++) {
-        u32x4* w0 = ws_ptr(l, 2 * q);
-        u32x4* w1 = ws_ptr(l, 2 * q + 1);
-        if ((g >> l) & 1) {
-          const u32x4 a = *w0, b = *w1;
-          t[4 * q + 0][0] = add_bf16x2(a[0], t[4 * q + 0][0]);
-          t[4 * q + 0][1] = add_bf16x2(a[1], t[4 * q + 0][1]);
-          t[4 * q + 1][0] = add_bf16x2(a[2], t[4 * q + 1][0]);
-          t[4 * q + 1][1] = add_bf16x2(a[3], t[4 * q + 1][1]);
-          t[4 * q + 2][0] = add_bf16x2(b[0], t[4 * q + 2][0]);
-          t[4 * q + 2][1] = add_bf16x2(b[1], t[4 * q + 2][1]);
-          t[4 * q + 3][0] = add_bf16x2(b[2], t[4 * q + 3][0]);
-          t[4 * q + 3][1] = add_bf16x2(b[3], t[4 * q + 3][1]);
-        } else {
-          *w0 = u32x4{t[4 * q + 0][0], t[4 * q + 0][1], t[4 * q + 1][0], t[4 * q + 1][1]};
-          *w1 = u32x4{t[4 * q + 2][0], t[4 * q + 2][1], t[4 * q + 3][0], t[4 * q + 3][1]};
-          parked = true;
-        }
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < 4; i++) {
-        s0[4 * q + i][0] = t[4 * q + i][0];
-        s0[4 * q + i][1] = t[4 * q + i][1];
+      } else {
+        *w0 = u32x4{t[8 * q], t[8 * q + 1], t[8 * q + 2], t[8 * q + 3]};
+        *w1 = u32x4{t[8 * q + 4], t[8 * q + 5], t[8 * q + 6], t[8 * q + 7]};
+        break;
       }
     }
   };
-  auto advance_counters = [&]() __attribute__((always_inline)) {
-    if (c0 + 1 == p.flb) {
-      c0 = 0;
-      g++;
-    } else {
-      c0++;
+
+  // Kinds of merge of the pending leaf (fixed per leaf, so each leaf body is straight-line code):
+  //   K_ADD  s0 += t                       (group not complete)
+  //   K_P0   sb0 = s0 + t                  (group complete, counter bit 0 clear)
+  //   K_P1   park level 1 <- sb0 + (s0+t)  (bit 0 set, bit 1 clear)
+  //   K_P2   t = lvl1 + (sb0 + (s0+t)), then the carry continues through the parked levels
+  // Level 1 of quarter q arrives in the LDS staging area (prefetch_parked) before it is needed.
+  const uint32_t spare_lds = lds0 + SPARE_OFF + wave * 2048;
+  auto prefetch_parked = [&](int q) __attribute__((always_inline)) {
+    const u32x4* src = p.ws + (((int64_t)tile_id * (NT / 64) + wave) * 8 + 2 * q) * 64;  // level RL, chunks 2q, 2q+1
+    dma16(spare_lds, lane * 16, src);
+    dma16(spare_lds + 1024, lane * 16, src + 64);
+  };
+  auto merge_quarter = [&](auto kind_c, int q) __attribute__((always_inline)) {
+    constexpr int KIND = decltype(kind_c)::value;
+    if (KIND == K_NONE) return;
+    u32x4 pf[2];
+    if (KIND == K_P2 && LS != 4) {
+      pf[0] = *ws_ptr(RL, 2 * q);
+      pf[1] = *ws_ptr(RL, 2 * q + 1);
     }
+    if (KIND == K_P2 && LS == 4) {
+      // everything older than the operand loads of this slice has landed, the staged level included
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA) : "memory");
+      pf[0] = *reinterpret_cast<const u32x4*>(smem + SPARE_OFF + wave * 2048 + lane * 16);
+      pf[1] = *reinterpret_cast<const u32x4*>(smem + SPARE_OFF + wave * 2048 + 1024 + lane * 16);
+    }
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      const int r = 8 * q + e;
+      const uint32_t l0 = add_bf16x2(s0[r], t[r]);
+      if (KIND == K_ADD) s0[r] = l0;
+      if (KIND == K_P0) sb0[r] = l0;
+      if (KIND == K_P1) t[r] = add_bf16x2(sb0[r], l0);
+      if (KIND == K_P2) t[r] = add_bf16x2(pf[e >> 2][e & 3], add_bf16x2(sb0[r], l0));
+    }
+    if (KIND == K_P1) {
+      *ws_ptr(RL, 2 * q) = u32x4{t[8 * q], t[8 * q + 1], t[8 * q + 2], t[8 * q + 3]};
+      *ws_ptr(RL, 2 * q + 1) = u32x4{t[8 * q + 4], t[8 * q + 5], t[8 * q + 6], t[8 * q + 7]};
+    }
+    if (KIND == K_P2) chain_parked(q, RL + 1, g_pending);
   };
 
   const int nstages = p.T * LS;
-  load_stage(0);
-  store_stage(0);
-  __syncthreads();
+  int slot = 0;  // ring slot of the slice being consumed
 
-  for (int j = 0; j < p.T; j++) {
+  issue_slice(0, 0);
+  issue_slice(min(1, nstages - 1), 1);
+
+  // One leaf: LS slices of MFMAs, with the pending leaf merged a quarter (LS=4) or a half (LS=2) per slice.
+  auto leaf_body = [&](auto kind_c, int j) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < LS; i++) {
       const int s = j * LS + i;
-      load_stage(min(s + 1, nstages - 1));
-      const uint16_t* bx = smem + (s & 1) * STAGE;
-      const uint16_t* bw = bx + BM * BK;
+      // slice s has landed (this wave's share), then everyone's
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA) : "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      if (decltype(kind_c)::value == K_P2 && LS == 4) prefetch_parked(i);
+      {
+        int ns = slot + 2;
+        ns = ns >= NSLOT ? ns - NSLOT : ns;
+        issue_slice(min(s + 2, nstages - 1), ns);
+      }
+      const uint8_t* base = smem + slot * STAGE_BYTES;
 #pragma unroll
       for (int kk = 0; kk < 2; kk++) {
         bf16x8 fx[TM], fw[TN];
 #pragma unroll
-        for (int a = 0; a < TM; a++) fx[a] = *reinterpret_cast<const bf16x8*>(bx + lds_off((wm * TM + a) * 16 + frow, kk * 4 + fchk));
+        for (int a = 0; a < TM; a++) fx[a] = *reinterpret_cast<const bf16x8*>(base + (xfrag ^ (kk * 64)) + a * 16 * BK * 2);
 #pragma unroll
-        for (int b = 0; b < TN; b++) fw[b] = *reinterpret_cast<const bf16x8*>(bw + lds_off((wn * TN + b) * 16 + frow, kk * 4 + fchk));
+        for (int b = 0; b < TN; b++) fw[b] = *reinterpret_cast<const bf16x8*>(base + (wfrag ^ (kk * 64)) + b * 16 * BK * 2);
 #pragma unroll
         for (int a = 0; a < TM; a++)
 #pragma unroll
@@ -221,27 +242,86 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
             acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[b], fx[a], (i == 0 && kk == 0) ? zero : acc[a][b], 0, 0, 0);
           }
       }
-      // deferred merge of the previous leaf: a quarter (LS == 4) or a half (LS == 2) per K slice
-      if (j > 0) {
 #pragma unroll
-        for (int q = i * (4 / LS); q < (i + 1) * (4 / LS); q++) merge_quarter(q);
+      for (int q = i * (4 / LS); q < (i + 1) * (4 / LS); q++) merge_quarter(kind_c, q);
+      // Issue order inside the slice: first fragment reads, a few merge ops while they are in flight,
+      // then one MFMA at a time with two merge ops (and the second half's fragment reads) in its shadow.
+      __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+      if (decltype(kind_c)::value != K_NONE) __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);
+#pragma unroll
+      for (int m = 0; m < 32; m++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if (m < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        if (decltype(kind_c)::value != K_NONE) __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
       }
-      store_stage((s + 1) & 1);
-      __syncthreads();
+      slot = slot + 1 == NSLOT ? 0 : slot + 1;
     }
-    if (j > 0) advance_counters();
-    // the finished leaf: round once to bf16; the accumulator is free again
+  };
+
+  int kind = K_NONE;
+  for (int j = 0; j < p.T; j++) {
+    switch (kind) {
+      case K_NONE: leaf_body(std::integral_constant<int, K_NONE>{}, j); break;
+      case K_ADD: leaf_body(std::integral_constant<int, K_ADD>{}, j); break;
+      case K_P0: leaf_body(std::integral_constant<int, K_P0>{}, j); break;
+      case K_P1: leaf_body(std::integral_constant<int, K_P1>{}, j); break;
+      default: leaf_body(std::integral_constant<int, K_P2>{}, j); break;
+    }
+    if (j == p.T - 1) break;  // the last leaf is packed and merged below
+    // the finished leaf: round once to bf16 (the accumulator is free again) and decide how it merges
+    if (c0 == 0 && p.flb > 1) {
+      // first leaf of a group: it simply becomes the running sum
 #pragma unroll
-    for (int a = 0; a < TM; a++)
+      for (int a = 0; a < TM; a++)
 #pragma unroll
-      for (int b = 0; b < TN; b++) {
-        t[a * TN + b][0] = pack_bf16x2(acc[a][b][0], acc[a][b][1]);
-        t[a * TN + b][1] = pack_bf16x2(acc[a][b][2], acc[a][b][3]);
+        for (int b = 0; b < TN; b++) {
+          s0[(a * TN + b) * 2] = pack_bf16x2(acc[a][b][0], acc[a][b][1]);
+          s0[(a * TN + b) * 2 + 1] = pack_bf16x2(acc[a][b][2], acc[a][b][3]);
+        }
+      kind = K_NONE;
+      c0 = 1;
+    } else {
+#pragma unroll
+      for (int a = 0; a < TM; a++)
+#pragma unroll
+        for (int b = 0; b < TN; b++) {
+          t[(a * TN + b) * 2] = pack_bf16x2(acc[a][b][0], acc[a][b][1]);
+          t[(a * TN + b) * 2 + 1] = pack_bf16x2(acc[a][b][2], acc[a][b][3]);
+        }
+      if (c0 + 1 < p.flb) {
+        kind = K_ADD;
+        c0++;
+      } else {
+        // the group completes: carry through the binary counter (this is never the last group here)
+        const int pops = __builtin_ctz(~g);
+        kind = pops == 0 ? K_P0 : (pops == 1 ? K_P1 : K_P2);
+        g_pending = g;
+        g++;
+        c0 = 0;
       }
+    }
   }
-  // merge of the last leaf: every level carries, t ends as the root
+
+  // ---- the last leaf: every level carries, t ends as the root
 #pragma unroll
-  for (int q = 0; q < 4; q++) merge_quarter(q);
+  for (int a = 0; a < TM; a++)
+#pragma unroll
+    for (int b = 0; b < TN; b++) {
+      t[(a * TN + b) * 2] = pack_bf16x2(acc[a][b][0], acc[a][b][1]);
+      t[(a * TN + b) * 2 + 1] = pack_bf16x2(acc[a][b][2], acc[a][b][3]);
+    }
+  if (c0 != 0) {
+#pragma unroll
+    for (int r = 0; r < NREG; r++) t[r] = add_bf16x2(s0[r], t[r]);
+  }
+  if (p.lb > 0) {
+#pragma unroll
+    for (int r = 0; r < NREG; r++) t[r] = add_bf16x2(sb0[r], t[r]);
+  }
+  if (p.lb > RL) {
+#pragma unroll
+    for (int q = 0; q < 4; q++) chain_parked(q, RL, g);
+  }
 
   // ---- store
 #pragma unroll
@@ -251,7 +331,7 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
     for (int b = 0; b < TN; b++) {
       const int n = n0 + (wn * TN + b) * 16 + fchk * 4;
       if (m >= p.M || n >= p.N) continue;
-      uint32_t lo = t[a * TN + b][0], hi = t[a * TN + b][1];
+      uint32_t lo = t[(a * TN + b) * 2], hi = t[(a * TN + b) * 2 + 1];
       if (p.bias) {
         float bv[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -275,9 +355,10 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
 
 int gemm_tree_wide_launch(const WideArgs& a, int leaf_k, hipStream_t stream) {
   using namespace wide;
-  constexpr size_t smem = (size_t)2 * STAGE * sizeof(uint16_t);  // 96 KiB
+  constexpr size_t smem = (size_t)NSLOT * STAGE_BYTES + 16384;  // 144 KiB ring + 16 KiB staging
   const int64_t tiles = (int64_t)((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
   if (tiles <= 0 || tiles > 0x7fffffff || a.lb > MAXLB) return TBIK_ERR_UNSUPPORTED;
+  if (a.ldx >= (1 << 22) || a.ldw >= (1 << 22)) return TBIK_ERR_UNSUPPORTED;  // 32-bit in-tile byte offsets
   if (leaf_k == 256) {
     auto kern = gemm_tree_wide_kernel<4>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
