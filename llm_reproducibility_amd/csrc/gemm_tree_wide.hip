@@ -244,16 +244,6 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
       }
 #pragma unroll
       for (int q = i * (4 / LS); q < (i + 1) * (4 / LS); q++) merge_quarter(kind_c, q);
-      // Issue order inside the slice: first fragment reads, a few merge ops while they are in flight,
-      // then one MFMA at a time with two merge ops (and the second half's fragment reads) in its shadow.
-      __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
-      if (decltype(kind_c)::value != K_NONE) __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);
-#pragma unroll
-      for (int m = 0; m < 32; m++) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        if (m < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        if (decltype(kind_c)::value != K_NONE) __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
-      }
       slot = slot + 1 == NSLOT ? 0 : slot + 1;
     }
   };
