@@ -221,11 +221,14 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
       __builtin_amdgcn_s_barrier();
       asm volatile("" ::: "memory");
       if (decltype(kind_c)::value == K_P2 && LS == 4) prefetch_parked(i);
-      {
-        int ns = slot + 2;
-        ns = ns >= NSLOT ? ns - NSLOT : ns;
-        issue_slice(min(s + 2, nstages - 1), ns);
-      }
+      // operand prefetch two slices ahead, spread over the slice: one load per four MFMAs (a burst of loads
+      // right after the barrier backs up the texture path and stalls every wave behind it)
+      int ns = slot + 2;
+      ns = ns >= NSLOT ? ns - NSLOT : ns;
+      const int ps = min(s + 2, nstages - 1);
+      const uint8_t* pxb = xbase + (int64_t)ps * (BK * 2);
+      const uint8_t* pwb = wbase + (int64_t)ps * (BK * 2);
+      const uint32_t pdst = lds0 + ns * STAGE_BYTES + wave * 1024;
       const uint8_t* base = smem + slot * STAGE_BYTES;
 #pragma unroll
       for (int kk = 0; kk < 2; kk++) {
@@ -235,12 +238,19 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
 #pragma unroll
         for (int b = 0; b < TN; b++) fw[b] = *reinterpret_cast<const bf16x8*>(base + (wfrag ^ (kk * 64)) + b * 16 * BK * 2);
 #pragma unroll
-        for (int a = 0; a < TM; a++)
+        for (int a = 0; a < TM; a++) {
 #pragma unroll
           for (int b = 0; b < TN; b++) {
             const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
             acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[b], fx[a], (i == 0 && kk == 0) ? zero : acc[a][b], 0, 0, 0);
           }
+          const int d = kk * TM + a;  // 0..7: loads 0..5 go out after MFMA rows 0..5
+          if (d < NDMA) {
+            __builtin_amdgcn_sched_barrier(0);
+            dma16(pdst + d * 8192, voff[d], d < 2 ? pxb : pwb);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        }
       }
 #pragma unroll
       for (int q = i * (4 / LS); q < (i + 1) * (4 / LS); q++) merge_quarter(kind_c, q);
