@@ -66,6 +66,11 @@ __device__ __forceinline__ void dma16(uint32_t lds_addr, uint32_t voff, const vo
                : "memory");
 }
 
+// 16-byte-per-lane store to (wave-uniform base) + voff, scalar-base addressing: no per-lane 64-bit pointer.
+__device__ __forceinline__ void store16_sbase(void* base, uint32_t voff, u32x4 v) {
+  asm volatile("global_store_dwordx4 %0, %1, %2" : : "v"(voff), "v"(v), "s"(base) : "memory");
+}
+
 template <int LS>
 __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs p) {
   using namespace wide;
@@ -138,8 +143,15 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
   int g = 0;           // groups completed
   int g_pending = 0;   // value of g for the leaf held in t
 
+  // parked level l, 16-byte word `chunk` of this wave: a wave-uniform base (scalar registers) plus 16*lane,
+  // so no per-lane pointer has to stay live across the K loop
+  const uint32_t lane16 = lane * 16;
+  auto ws_base = [&](int l, int chunk) __attribute__((always_inline)) -> uint8_t* {
+    return reinterpret_cast<uint8_t*>(p.ws) +
+           ((((int64_t)(l - RL) * ntiles + tile_id) * (NT / 64) + wave) * 8 + chunk) * (int64_t)1024;
+  };
   auto ws_ptr = [&](int l, int chunk) __attribute__((always_inline)) -> u32x4* {
-    return p.ws + ((((int64_t)(l - RL) * ntiles + tile_id) * (NT / 64) + wave) * 8 + chunk) * 64 + lane;
+    return reinterpret_cast<u32x4*>(ws_base(l, chunk) + lane16);
   };
 
   // Parked levels for quarter q (tiles 4q..4q+3 = registers 8q..8q+7 = chunks 2q, 2q+1): continue the carry
@@ -156,8 +168,8 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
           t[8 * q + 4 + e] = add_bf16x2(b[e], t[8 * q + 4 + e]);
         }
       } else {
-        *w0 = u32x4{t[8 * q], t[8 * q + 1], t[8 * q + 2], t[8 * q + 3]};
-        *w1 = u32x4{t[8 * q + 4], t[8 * q + 5], t[8 * q + 6], t[8 * q + 7]};
+        store16_sbase(ws_base(l, 2 * q), lane16, u32x4{t[8 * q], t[8 * q + 1], t[8 * q + 2], t[8 * q + 3]});
+        store16_sbase(ws_base(l, 2 * q + 1), lane16, u32x4{t[8 * q + 4], t[8 * q + 5], t[8 * q + 6], t[8 * q + 7]});
         break;
       }
     }
@@ -199,8 +211,8 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
       if (KIND == K_P2) t[r] = add_bf16x2(pf[e >> 2][e & 3], add_bf16x2(sb0[r], l0));
     }
     if (KIND == K_P1) {
-      *ws_ptr(RL, 2 * q) = u32x4{t[8 * q], t[8 * q + 1], t[8 * q + 2], t[8 * q + 3]};
-      *ws_ptr(RL, 2 * q + 1) = u32x4{t[8 * q + 4], t[8 * q + 5], t[8 * q + 6], t[8 * q + 7]};
+      store16_sbase(ws_base(RL, 2 * q), lane16, u32x4{t[8 * q], t[8 * q + 1], t[8 * q + 2], t[8 * q + 3]});
+      store16_sbase(ws_base(RL, 2 * q + 1), lane16, u32x4{t[8 * q + 4], t[8 * q + 5], t[8 * q + 6], t[8 * q + 7]});
     }
     if (KIND == K_P2) chain_parked(q, RL + 1, g_pending);
   };
