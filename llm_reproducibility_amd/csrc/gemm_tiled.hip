@@ -31,6 +31,9 @@ struct GemmArgs {
   int flb;    // leaves summed left to right at level 0
   int lb;     // binary levels above level 0
   int vec_store;  // C rows allow 8-byte stores
+  // K split into gridDim.y shards (aligned subtrees): shard y reads columns [y*k_shard, +K) of X and W and writes
+  // its bf16 partial at C + y*c_shard; the shard tree (tree_combine) then rebuilds the unsplit result bit for bit
+  int64_t k_shard, c_shard;
 };
 
 constexpr int BK = 64;  // K elements per LDS stage (8 chunks of 16 bytes per row)
@@ -75,6 +78,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
   const int m0 = pid_m * BM;
   const int n0 = pid_n * BN;
 
+  const uint16_t* Xs = p.X + blockIdx.y * p.k_shard;
+  const uint16_t* Ws = p.W + blockIdx.y * p.k_shard;
+  uint16_t* Cs = p.C + blockIdx.y * p.c_shard;
+
   // ---- global -> register staging (rows past the edge are clamped: their results are never stored)
   const uint16_t* xptr[XCH];
   const uint16_t* wptr[WCH];
@@ -84,7 +91,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
     const int q = tid + i * NT;
     const int r = (q >> 3) % BM, c = q & 7;
     const int gr = min(m0 + r, p.M - 1);
-    xptr[i] = p.X + (int64_t)gr * p.ldx + c * 8;
+    xptr[i] = Xs + (int64_t)gr * p.ldx + c * 8;
     xdst[i] = lds_off(r, c);
   }
 #pragma unroll
@@ -92,7 +99,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
     const int q = tid + i * NT;
     const int r = (q >> 3) % BN, c = q & 7;
     const int gr = min(n0 + r, p.N - 1);
-    wptr[i] = p.W + (int64_t)gr * p.ldw + c * 8;
+    wptr[i] = Ws + (int64_t)gr * p.ldw + c * 8;
     wdst[i] = lds_off(r, c);
   }
   u32x4 xreg[XCH], wreg[WCH];
@@ -265,7 +272,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
         lo = pack_bf16x2(acc[a][b][0] + bv[0], acc[a][b][1] + bv[1]);
         hi = pack_bf16x2(acc[a][b][2] + bv[2], acc[a][b][3] + bv[3]);
       }
-      uint16_t* dst = p.C + (int64_t)m * p.ldc + n;
+      uint16_t* dst = Cs + (int64_t)m * p.ldc + n;
       if (p.vec_store && n + 3 < p.N) {
         *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);
       } else {
@@ -282,7 +289,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
 // host side
 // ------------------------------------------------------------------------------------------------
 template <int WAVES_M, int WAVES_N, int TM, int TN, int LS, int LBMAX, bool TREE>
-static int launch(const GemmArgs& a, hipStream_t stream) {
+static int launch(const GemmArgs& a, int split, hipStream_t stream) {
   constexpr int NT = WAVES_M * WAVES_N * 64;
   constexpr int BM = WAVES_M * TM * 16;
   constexpr int BN = WAVES_N * TN * 16;
@@ -295,22 +302,22 @@ static int launch(const GemmArgs& a, hipStream_t stream) {
   }
   const int64_t tiles = (int64_t)((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
   if (tiles <= 0 || tiles > 0x7fffffff) return TBIK_ERR_INVALID;
-  hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(NT), smem, stream, a);
+  hipLaunchKernelGGL(kern, dim3((unsigned)tiles, (unsigned)split), dim3(NT), smem, stream, a);
   return hip_code(hipGetLastError());
 }
 
 template <int LS, int LBMAX, bool TREE>
-static int launch_by_m(const GemmArgs& a, hipStream_t stream) {
-  if (a.M <= 16) return launch<1, 4, 1, 1, LS, LBMAX, TREE>(a, stream);
-  if (a.M <= 64) return launch<1, 4, 4, 2, LS, LBMAX, TREE>(a, stream);
-  return launch<2, 2, 4, 4, LS, LBMAX, TREE>(a, stream);
+static int launch_by_m(const GemmArgs& a, int split, hipStream_t stream) {
+  if (a.M <= 16) return launch<1, 4, 1, 1, LS, LBMAX, TREE>(a, split, stream);
+  if (a.M <= 64) return launch<1, 4, 4, 2, LS, LBMAX, TREE>(a, split, stream);
+  return launch<2, 2, 4, 4, LS, LBMAX, TREE>(a, split, stream);
 }
 
 template <int LS>
-static int launch_tree(const GemmArgs& a, hipStream_t stream) {
-  if (a.lb <= 2) return launch_by_m<LS, 2, true>(a, stream);
-  if (a.lb <= 4) return launch_by_m<LS, 4, true>(a, stream);
-  if (a.lb <= 6) return launch_by_m<LS, 6, true>(a, stream);
+static int launch_tree(const GemmArgs& a, int split, hipStream_t stream) {
+  if (a.lb <= 2) return launch_by_m<LS, 2, true>(a, split, stream);
+  if (a.lb <= 4) return launch_by_m<LS, 4, true>(a, split, stream);
+  if (a.lb <= 6) return launch_by_m<LS, 6, true>(a, split, stream);
   return TBIK_ERR_UNSUPPORTED;
 }
 
@@ -327,21 +334,58 @@ struct WideArgs {
   int M, N, K;
   int T, flb, lb;
   int vec_store;
+  int64_t k_shard, c_shard;
 };
-size_t wide_workspace_bytes(int M, int N, int lb);
-int gemm_tree_wide_launch(const WideArgs& a, int leaf_k, hipStream_t stream);
+size_t wide_workspace_bytes(int M, int N, int lb, int split);
+int gemm_tree_wide_launch(const WideArgs& a, int leaf_k, int split, hipStream_t stream);
+int tree_combine_bias_dispatch(const void* const* parts, int nparts, void* out, int64_t numel, const void* bias, int N,
+                               hipStream_t stream);
 
-// The wide kernel pays off once its 128x256 tiles can occupy the chip; below that the 128x128 / 64x128 /
-// 16x64 tiles of this file give more work-groups.  The choice never changes the result.
-static bool use_wide(int M, int N) {
+// How one problem is run.  Small grids are filled by cutting K into `split` aligned subtrees (one grid.y slice
+// each) whose bf16 partials meet in the shard tree afterwards -- the same arithmetic as tensor-parallel shards, so
+// the bits do not change.  The wide kernel takes over once its 128x256 tiles (times the split) occupy the chip.
+struct Plan {
+  bool wide;
+  int split;       // power of two, divides 2^lb
+  int T, flb, lb;  // tree of ONE shard
+  size_t partial_bytes, parked_bytes;
+};
+
+static bool make_plan(int M, int N, int K, int leaf_k, Plan* pl) {
+  int T, flb, level_k;
+  if (M <= 0 || N <= 0 || tbik_tree_params(K, leaf_k, &T, &flb, &level_k) != TBIK_OK) return false;
+  const int lb = level_k - 1;
+  const int max_split = lb >= 3 ? 8 : (1 << lb);
   const int64_t wide_tiles = (int64_t)((M + 127) / 128) * ((N + 255) / 256);
-  return M > 64 && wide_tiles >= 128;
+  int split = 1;
+  bool wide = false;
+  if (M > 64) {
+    while (wide_tiles * split < 192 && split < max_split) split *= 2;
+    wide = wide_tiles * split >= 128;
+  }
+  if (!wide) {
+    const int bm = M <= 16 ? 16 : (M <= 64 ? 64 : 128), bn = M <= 16 ? 64 : 128;
+    const int64_t tiles = (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
+    split = 1;
+    while (tiles * split < 512 && split < max_split) split *= 2;
+  }
+  int ls = 0;
+  while ((1 << ls) < split) ls++;
+  pl->wide = wide;
+  pl->split = split;
+  pl->T = T / split;
+  pl->flb = flb;
+  pl->lb = lb - ls;
+  pl->partial_bytes = split > 1 ? (size_t)split * M * N * sizeof(uint16_t) : 0;
+  pl->partial_bytes = (pl->partial_bytes + 255) & ~(size_t)255;
+  pl->parked_bytes = wide ? wide_workspace_bytes(M, N, pl->lb, split) : 0;
+  return true;
 }
 
 size_t gemm_workspace_bytes(int M, int N, int K, int leaf_k) {
-  int T, flb, level_k;
-  if (M <= 0 || N <= 0 || tbik_tree_params(K, leaf_k, &T, &flb, &level_k) != TBIK_OK) return 0;
-  return use_wide(M, N) ? wide_workspace_bytes(M, N, level_k - 1) : 0;
+  Plan pl;
+  if (!make_plan(M, N, K, leaf_k, &pl)) return 0;
+  return pl.partial_bytes + pl.parked_bytes;
 }
 
 int gemm_dispatch(bool tree, const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C,
@@ -369,23 +413,47 @@ int gemm_dispatch(bool tree, const void* A, int64_t lda, const void* B, int64_t 
   a.flb = 1;
   a.lb = 0;
   a.vec_store = ((reinterpret_cast<uintptr_t>(C) & 7) == 0 && (ldc & 3) == 0) ? 1 : 0;
-  if (!tree) return launch_by_m<4, 0, false>(a, stream);
+  a.k_shard = 0;
+  a.c_shard = 0;
+  if (!tree) return launch_by_m<4, 0, false>(a, 1, stream);
 
-  int T, flb, level_k;
-  if (tbik_tree_params(K, leaf_k, &T, &flb, &level_k) != TBIK_OK) return TBIK_ERR_INVALID;
-  a.T = T;
-  a.flb = flb;
-  a.lb = level_k - 1;
   if (leaf_k != 256 && leaf_k != 128) return TBIK_ERR_UNSUPPORTED;
-  if (use_wide(M, N)) {
-    const size_t need = wide_workspace_bytes(M, N, a.lb);
-    if (need > 0 && (!ws || ws_bytes < need || !aligned16(ws))) return TBIK_ERR_WORKSPACE;
-    WideArgs w{a.X, a.W, a.C, a.bias, static_cast<u32x4*>(ws), a.ldx, a.ldw, a.ldc, M, N, K, T, flb, a.lb, a.vec_store};
-    return gemm_tree_wide_launch(w, leaf_k, stream);
+  Plan pl;
+  if (!make_plan(M, N, K, leaf_k, &pl)) return TBIK_ERR_INVALID;
+  const size_t need = pl.partial_bytes + pl.parked_bytes;
+  if (need > 0 && (!ws || ws_bytes < need || !aligned16(ws))) return TBIK_ERR_WORKSPACE;
+  uint8_t* wsb = static_cast<uint8_t*>(ws);
+  a.T = pl.T;
+  a.flb = pl.flb;
+  a.lb = pl.lb;
+  a.k_shard = K / pl.split;
+  a.K = K / pl.split;
+  if (pl.split > 1) {
+    // shards write contiguous [M,N] partials into the workspace; bias is applied after the shard tree
+    a.C = reinterpret_cast<uint16_t*>(wsb);
+    a.ldc = N;
+    a.c_shard = (int64_t)M * N;
+    a.vec_store = (N & 3) == 0 ? 1 : 0;
+    a.bias = nullptr;
   }
-  if (leaf_k == 256) return launch_tree<4>(a, stream);
-  if (leaf_k == 128) return launch_tree<2>(a, stream);
-  return TBIK_ERR_UNSUPPORTED;
+  int rc;
+  if (pl.wide) {
+    WideArgs w{a.X, a.W, a.C, a.bias, reinterpret_cast<u32x4*>(wsb + pl.partial_bytes), a.ldx, a.ldw, a.ldc, M, N, a.K,
+               a.T, a.flb, a.lb, a.vec_store, a.k_shard, a.c_shard};
+    rc = gemm_tree_wide_launch(w, leaf_k, pl.split, stream);
+  } else {
+    rc = leaf_k == 256 ? launch_tree<4>(a, pl.split, stream) : launch_tree<2>(a, pl.split, stream);
+  }
+  if (rc != TBIK_OK || pl.split == 1) return rc;
+  const void* parts[8];
+  for (int i = 0; i < pl.split; i++) parts[i] = wsb + (size_t)i * M * N * sizeof(uint16_t);
+  if (ldc == N) return tree_combine_bias_dispatch(parts, pl.split, C, (int64_t)M * N, bias, N, stream);
+  for (int m = 0; m < M && rc == TBIK_OK; m++) {  // strided C (rare): row by row
+    const void* rp[8];
+    for (int i = 0; i < pl.split; i++) rp[i] = static_cast<const uint8_t*>(parts[i]) + (size_t)m * N * sizeof(uint16_t);
+    rc = tree_combine_bias_dispatch(rp, pl.split, static_cast<uint16_t*>(C) + (int64_t)m * ldc, N, bias, N, stream);
+  }
+  return rc;
 }
 
 }  // namespace tbik

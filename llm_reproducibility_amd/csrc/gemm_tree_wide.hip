@@ -34,6 +34,7 @@ struct WideArgs {
   int M, N, K;
   int T, flb, lb;
   int vec_store;
+  int64_t k_shard, c_shard;  // K split over gridDim.y shards: operand column offset and partial-output offset per shard
 };
 
 namespace wide {
@@ -51,10 +52,10 @@ constexpr int MAXLB = 16;
 enum Kind { K_NONE = 0, K_ADD = 1, K_P0 = 2, K_P1 = 3, K_P2 = 4 };
 }  // namespace wide
 
-size_t wide_workspace_bytes(int M, int N, int lb) {
+size_t wide_workspace_bytes(int M, int N, int lb, int split) {
   using namespace wide;
   if (lb <= RL) return 0;
-  const size_t tiles = (size_t)((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  const size_t tiles = (size_t)((M + BM - 1) / BM) * ((N + BN - 1) / BN) * (size_t)split;
   return (size_t)(lb - RL) * tiles * (NT / 64) * 8 * 64 * sizeof(u32x4);
 }
 
@@ -98,13 +99,14 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
   const int pid_n = (lid % per_group) / gsz;
   const int m0 = pid_m * BM;
   const int n0 = pid_n * BN;
-  const int tile_id = pid_m * tiles_n + pid_n;
-  const int ntiles = tiles_m * tiles_n;
+  const int shard = blockIdx.y;
+  const int tile_id = (shard * tiles_m + pid_m) * tiles_n + pid_n;
+  const int ntiles = tiles_m * tiles_n * gridDim.y;
 
   // ---- direct global->LDS loads.  Wave w's i-th load of a slice fills LDS rows [8*(8i+w), +8): lane l
   // lands at row 8*(8i+w) + l/8, physical 16-byte chunk l%8, so it fetches logical chunk (l%8)^(l/8).
-  const uint8_t* xbase = reinterpret_cast<const uint8_t*>(p.X + (int64_t)m0 * p.ldx);
-  const uint8_t* wbase = reinterpret_cast<const uint8_t*>(p.W + (int64_t)n0 * p.ldw);
+  const uint8_t* xbase = reinterpret_cast<const uint8_t*>(p.X + (int64_t)m0 * p.ldx + shard * p.k_shard);
+  const uint8_t* wbase = reinterpret_cast<const uint8_t*>(p.W + (int64_t)n0 * p.ldw + shard * p.k_shard);
   uint32_t voff[NDMA];
   {
     const int r = lane >> 3, c = (lane & 7) ^ r;
@@ -352,7 +354,7 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
         lo = add_bf16x2(lo, pack_bf16x2(bv[0], bv[1]));
         hi = add_bf16x2(hi, pack_bf16x2(bv[2], bv[3]));
       }
-      uint16_t* dst = p.C + (int64_t)m * p.ldc + n;
+      uint16_t* dst = p.C + shard * p.c_shard + (int64_t)m * p.ldc + n;
       if (p.vec_store && n + 3 < p.N) {
         *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);
       } else {
@@ -365,7 +367,7 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
   }
 }
 
-int gemm_tree_wide_launch(const WideArgs& a, int leaf_k, hipStream_t stream) {
+int gemm_tree_wide_launch(const WideArgs& a, int leaf_k, int split, hipStream_t stream) {
   using namespace wide;
   constexpr size_t smem = (size_t)NSLOT * STAGE_BYTES + 16384;  // 144 KiB ring + 16 KiB staging
   const int64_t tiles = (int64_t)((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
@@ -375,12 +377,12 @@ int gemm_tree_wide_launch(const WideArgs& a, int leaf_k, hipStream_t stream) {
     auto kern = gemm_tree_wide_kernel<4>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return hip_code(e);
-    hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(NT), smem, stream, a);
+    hipLaunchKernelGGL(kern, dim3((unsigned)tiles, (unsigned)split), dim3(NT), smem, stream, a);
   } else if (leaf_k == 128) {
     auto kern = gemm_tree_wide_kernel<2>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return hip_code(e);
-    hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(NT), smem, stream, a);
+    hipLaunchKernelGGL(kern, dim3((unsigned)tiles, (unsigned)split), dim3(NT), smem, stream, a);
   } else {
     return TBIK_ERR_UNSUPPORTED;
   }

@@ -11,6 +11,8 @@ struct CombineArgs {
   const uint16_t* parts[8];
   uint16_t* out;
   int64_t numel;
+  const uint16_t* bias;  // optional [ncols] row vector added (in bf16) after the tree; element i is in column i % ncols
+  int ncols;
 };
 
 template <int NP>
@@ -47,6 +49,13 @@ __global__ __launch_bounds__(256) void combine_vec_kernel(const CombineArgs a, i
 #pragma unroll
     for (int p = 0; p < NP; p++) v[p] = in[p].w;
     o.w = tree_node<NP>(v);
+    if (a.bias) {  // ncols % 8 == 0 on this path: the pack stays inside one row
+      const uint4 bq = *reinterpret_cast<const uint4*>(a.bias + (i * 8) % a.ncols);
+      o.x = add_bf16x2(o.x, bq.x);
+      o.y = add_bf16x2(o.y, bq.y);
+      o.z = add_bf16x2(o.z, bq.z);
+      o.w = add_bf16x2(o.w, bq.w);
+    }
     reinterpret_cast<uint4*>(a.out)[i] = o;
   }
 }
@@ -59,7 +68,9 @@ __global__ __launch_bounds__(256) void combine_scalar_kernel(const CombineArgs a
     uint32_t v[8];
 #pragma unroll
     for (int p = 0; p < NP; p++) v[p] = a.parts[p][i];
-    a.out[i] = (uint16_t)(tree_node<NP>(v) & 0xffffu);
+    uint32_t r = tree_node<NP>(v);
+    if (a.bias) r = add_bf16x2(r, a.bias[i % a.ncols]);
+    a.out[i] = (uint16_t)(r & 0xffffu);
   }
 }
 
@@ -81,8 +92,9 @@ static int launch_combine(const CombineArgs& a, bool vec_ok, hipStream_t stream)
   return hip_code(hipGetLastError());
 }
 
-int tree_combine_dispatch(const void* const* parts, int nparts, void* out, int64_t numel, hipStream_t stream) {
-  if (!parts || !out || numel < 0) return TBIK_ERR_INVALID;
+int tree_combine_bias_dispatch(const void* const* parts, int nparts, void* out, int64_t numel, const void* bias, int N,
+                               hipStream_t stream) {
+  if (!parts || !out || numel < 0 || (bias && N <= 0)) return TBIK_ERR_INVALID;
   if (nparts != 1 && nparts != 2 && nparts != 4 && nparts != 8) return TBIK_ERR_INVALID;
   if (numel == 0) return TBIK_OK;
   CombineArgs a;
@@ -97,12 +109,19 @@ int tree_combine_dispatch(const void* const* parts, int nparts, void* out, int64
   }
   a.out = static_cast<uint16_t*>(out);
   a.numel = numel;
+  a.bias = static_cast<const uint16_t*>(bias);
+  a.ncols = N;
+  if (bias) vec_ok = vec_ok && (N & 7) == 0 && (reinterpret_cast<uintptr_t>(bias) & 15) == 0;
   switch (nparts) {
     case 1: return launch_combine<1>(a, vec_ok, stream);
     case 2: return launch_combine<2>(a, vec_ok, stream);
     case 4: return launch_combine<4>(a, vec_ok, stream);
     default: return launch_combine<8>(a, vec_ok, stream);
   }
+}
+
+int tree_combine_dispatch(const void* const* parts, int nparts, void* out, int64_t numel, hipStream_t stream) {
+  return tree_combine_bias_dispatch(parts, nparts, out, numel, nullptr, 0, stream);
 }
 
 }  // namespace tbik
