@@ -151,6 +151,24 @@ int bi_mean_dim(const void* x, void* out,
                 int dtype_code,
                 tbik_stream_t stream);
 
+/*
+ * Causal grouped-query attention with a fixed key order (tiles of 32 keys, ascending, online softmax, one
+ * pass, no split over keys), bf16, head_dim 128; the same kernel serves prefill and decode, and a
+ * token's output does not depend on the batch it is computed in.
+ *   q, out      [tokens, q_heads, 128]
+ *   k_cache     [batch, kv_heads, max_len, 128]
+ *   vt_cache    [batch, kv_heads, 128, max_len]   (V stored transposed; entries behind ctx_len must be finite)
+ *   q_start/q_len/ctx_len  device int32 [batch]: first token row, number of new tokens, cache length
+ *                          including the new tokens (query r of sequence b sits at position ctx_len-q_len+r)
+ * Replaces: the fixed-tile attention of the train/inference alignment patch,
+ *           _kernel_unified_attention_2d, src/patch/patch_training_inference_align.py:171-487 (its KV-order
+ *           rule, not vLLM's paged-cache plumbing).
+ */
+int bi_attention_bf16(const void* q, const void* k_cache, const void* vt_cache, void* out,
+                      const int32_t* q_start, const int32_t* q_len, const int32_t* ctx_len,
+                      int batch, int max_q_len, int q_heads, int kv_heads, int head_dim, int max_len,
+                      float scale, tbik_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

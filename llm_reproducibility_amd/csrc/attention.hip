@@ -1,0 +1,155 @@
+// Fixed-order causal attention for gfx950 (bf16, head_dim 128, grouped-query heads), one wavefront per
+// (16 consecutive queries of one sequence, one query head).
+//
+// Counterpart of the reference's fixed-tile attention for train/inference alignment
+// (_kernel_unified_attention_2d, src/patch/patch_training_inference_align.py:171-487: one pass over the
+// keys in tiles of 32, online softmax, no split over the key axis, the same kernel for prefill and decode).
+//
+// Invariance argument: a query row is owned by the four lanes {j, j+16, j+32, j+48}; its scores, its
+// running maximum / denominator and its output accumulators never mix with another row's.  Keys are
+// visited in ascending tiles of 32 whatever the batch or the block looks like; a tile that lies entirely
+// behind a row's causal horizon contributes exp(-inf) = 0 and a rescale by exactly 1.0, so the number of
+// tiles the BLOCK walks does not change the row.  Prefill (16 rows per block) and decode (1 valid row)
+// therefore produce the same bits for the same token, and heads can be sharded freely.
+//
+// Layouts: q/out [tokens, q_heads, 128]; K cache [batch, kv_heads, max_len, 128]; V cache TRANSPOSED
+// [batch, kv_heads, 128, max_len] so that the P*V MFMA operand (8 consecutive keys of one channel) is a
+// contiguous load.  Cache entries behind ctx_len must be finite (they are multiplied by an exact 0).
+#include "common.h"
+
+namespace tbik {
+
+struct AttnArgs {
+  const uint16_t* q;
+  const uint16_t* k_cache;
+  const uint16_t* vt_cache;
+  uint16_t* out;
+  const int* q_start;  // [batch] first token row of the sequence in q/out
+  const int* q_len;    // [batch] new tokens of the sequence
+  const int* ctx_len;  // [batch] keys visible to the LAST new token (cache length including the new tokens)
+  int q_heads, kv_heads, max_len;
+  float scale_log2;    // log2(e) / sqrt(head_dim): scores are kept in the base-2 domain
+};
+
+constexpr int HD = 128;
+
+__global__ __launch_bounds__(64) void attention_kernel(const AttnArgs a) {
+  const int b = blockIdx.z;
+  const int h = blockIdx.y;
+  const int qb = blockIdx.x;
+  const int qlen = a.q_len[b];
+  if (qb * 16 >= qlen) return;
+  const int lane = threadIdx.x;
+  const int j = lane & 15;   // query row inside the block (also: key row of a K fragment, channel row of a V fragment)
+  const int g = lane >> 4;   // lane group: which 8-wide k slice of an MFMA operand, which 4 rows of an MFMA result
+  const int ctx = a.ctx_len[b];
+  const int kvh = h / (a.q_heads / a.kv_heads);
+  const int qrow = qb * 16 + j;                     // row inside the sequence's new tokens
+  const bool qvalid = qrow < qlen;
+  const int qpos = ctx - qlen + min(qrow, qlen - 1);  // absolute position of this lane's query
+  const int last_pos = ctx - qlen + min(qb * 16 + 15, qlen - 1);
+
+  // Q as the MFMA "B" operand: lane (j, g) holds q[j][32c + 8g .. +7] for the four 32-wide channel chunks c
+  const uint16_t* qp = a.q + ((int64_t)(a.q_start[b] + min(qrow, qlen - 1)) * a.q_heads + h) * HD;
+  bf16x8 qf[4];
+#pragma unroll
+  for (int c = 0; c < 4; c++) qf[c] = *reinterpret_cast<const bf16x8*>(qp + c * 32 + g * 8);
+
+  const uint16_t* kbase = a.k_cache + ((int64_t)b * a.kv_heads + kvh) * a.max_len * HD;
+  const uint16_t* vbase = a.vt_cache + ((int64_t)b * a.kv_heads + kvh) * (int64_t)HD * a.max_len;
+
+  f32x4 o[8];  // output accumulators, transposed: lane (j, g) holds out[j][16t + 4g .. +3] for the channel tiles t
+#pragma unroll
+  for (int t = 0; t < 8; t++) o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY;  // running maximum (base-2 domain), identical in the four lanes of a row
+  float l = 0.f;        // running denominator
+
+  const int ntiles = last_pos / 32 + 1;
+  for (int tile = 0; tile < ntiles; tile++) {
+    const int k0 = tile * 32;
+    // ---- scores: two 16-key sub-tiles; lane (j, g) receives keys k0 + 16u + 4g + i of query j
+    f32x4 s[2];
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+      const int krow = min(k0 + 16 * u + j, a.max_len - 1);
+      const uint16_t* kp = kbase + (int64_t)krow * HD + g * 8;
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(kp + c * 32);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[c], acc, 0, 0, 0);
+      }
+      s[u] = acc;
+    }
+    float sv[8];
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < 2; u++)
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const int key = k0 + 16 * u + 4 * g + i;
+        const float v = (key <= qpos) ? s[u][i] * a.scale_log2 : -INFINITY;
+        sv[4 * u + i] = v;
+        tmax = fmaxf(tmax, v);
+      }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_new = fmaxf(m, tmax);          // key 0 is visible to every query: m_new is finite from tile 0 on
+    const float alpha = exp2f(m - m_new);         // exactly 1.0 when the tile adds nothing new
+    float psum = 0.f;
+    float pv[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      pv[e] = exp2f(sv[e] - m_new);
+      psum += pv[e];
+    }
+    psum += __shfl_xor(psum, 16, 64);
+    psum += __shfl_xor(psum, 32, 64);
+    l = l * alpha + psum;
+    m = m_new;
+    // P as the MFMA "B" operand: k slots 0..3 = keys k0+4g.., slots 4..7 = keys k0+16+4g..
+    const uint32_t p0 = pack_bf16x2(pv[0], pv[1]), p1 = pack_bf16x2(pv[2], pv[3]);
+    const uint32_t p2 = pack_bf16x2(pv[4], pv[5]), p3 = pack_bf16x2(pv[6], pv[7]);
+    const bf16x8 pf = __builtin_bit_cast(bf16x8, u32x4{p0, p1, p2, p3});
+    // ---- out^T += V^T * P: "A" operand lane (j, g) holds channel 16t + j, the same 8 key slots
+    const int kv0 = min(k0 + 4 * g, a.max_len - 4);
+    const int kv1 = min(k0 + 16 + 4 * g, a.max_len - 4);
+#pragma unroll
+    for (int t = 0; t < 8; t++) {
+      const uint16_t* vp = vbase + (int64_t)(16 * t + j) * a.max_len;
+      const uint2 va = *reinterpret_cast<const uint2*>(vp + kv0);
+      const uint2 vb = *reinterpret_cast<const uint2*>(vp + kv1);
+      const bf16x8 vf = __builtin_bit_cast(bf16x8, u32x4{va.x, va.y, vb.x, vb.y});
+      f32x4 scaled = {o[t][0] * alpha, o[t][1] * alpha, o[t][2] * alpha, o[t][3] * alpha};
+      o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, scaled, 0, 0, 0);
+    }
+  }
+  if (!qvalid) return;
+  const float inv = 1.0f / l;
+  uint16_t* op = a.out + ((int64_t)(a.q_start[b] + qrow) * a.q_heads + h) * HD;
+#pragma unroll
+  for (int t = 0; t < 8; t++) {
+    const uint32_t lo = pack_bf16x2(o[t][0] * inv, o[t][1] * inv);
+    const uint32_t hi = pack_bf16x2(o[t][2] * inv, o[t][3] * inv);
+    *reinterpret_cast<uint2*>(op + 16 * t + 4 * g) = make_uint2(lo, hi);
+  }
+}
+
+int attention_dispatch(const void* q, const void* k_cache, const void* vt_cache, void* out, const int* q_start,
+                       const int* q_len, const int* ctx_len, int batch, int max_q_len, int q_heads, int kv_heads,
+                       int head_dim, int max_len, float scale, hipStream_t stream) {
+  if (!q || !k_cache || !vt_cache || !out || !q_start || !q_len || !ctx_len) return TBIK_ERR_INVALID;
+  if (batch <= 0 || max_q_len <= 0 || q_heads <= 0 || kv_heads <= 0 || q_heads % kv_heads != 0) return TBIK_ERR_INVALID;
+  if (head_dim != HD) return TBIK_ERR_UNSUPPORTED;
+  if (max_len < 32 || (max_len & 3)) return TBIK_ERR_ALIGNMENT;
+  auto mis = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) != 0; };
+  if (mis(q) || mis(k_cache) || mis(vt_cache) || mis(out)) return TBIK_ERR_ALIGNMENT;
+  if (batch > 65535 || q_heads > 65535) return TBIK_ERR_INVALID;
+  AttnArgs a{static_cast<const uint16_t*>(q), static_cast<const uint16_t*>(k_cache), static_cast<const uint16_t*>(vt_cache),
+             static_cast<uint16_t*>(out), q_start, q_len, ctx_len, q_heads, kv_heads, max_len, scale * 1.4426950408889634f};
+  const dim3 grid((unsigned)((max_q_len + 15) / 16), (unsigned)q_heads, (unsigned)batch);
+  hipLaunchKernelGGL(attention_kernel, grid, dim3(64), 0, stream, a);
+  return hip_code(hipGetLastError());
+}
+
+}  // namespace tbik

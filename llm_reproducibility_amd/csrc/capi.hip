@@ -13,12 +13,15 @@ int rmsnorm_dispatch(const void* x, int64_t ldx, const void* res, int64_t ldr, c
 size_t lsm_workspace_bytes(int64_t rows, int64_t cols);
 int log_softmax_dispatch(const void* x, int64_t ldx, void* out, int64_t ldo, int64_t rows, int64_t cols, void* ws,
                          size_t ws_bytes, int write_softmax, hipStream_t stream);
+int attention_dispatch(const void* q, const void* k_cache, const void* vt_cache, void* out, const int* q_start,
+                       const int* q_len, const int* ctx_len, int batch, int max_q_len, int q_heads, int kv_heads,
+                       int head_dim, int max_len, float scale, hipStream_t stream);
 int mean_dispatch(const void* x, void* out, int64_t outer, int64_t n, int64_t inner, int dtype_code, hipStream_t stream);
 }  // namespace tbik
 
 extern "C" {
 
-int tbik_abi_version(void) { return 2; }
+int tbik_abi_version(void) { return 3; }
 
 const char* tbik_error_string(int code) {
   switch (code) {
@@ -80,6 +83,13 @@ int bi_log_softmax_f32(const void* x, int64_t ldx, void* out, int64_t ldo, int64
 
 int bi_mean_dim(const void* x, void* out, int64_t outer, int64_t n, int64_t inner, int dtype_code, tbik_stream_t stream) {
   return tbik::mean_dispatch(x, out, outer, n, inner, dtype_code, static_cast<hipStream_t>(stream));
+}
+
+int bi_attention_bf16(const void* q, const void* k_cache, const void* vt_cache, void* out, const int32_t* q_start,
+                      const int32_t* q_len, const int32_t* ctx_len, int batch, int max_q_len, int q_heads, int kv_heads,
+                      int head_dim, int max_len, float scale, tbik_stream_t stream) {
+  return tbik::attention_dispatch(q, k_cache, vt_cache, out, q_start, q_len, ctx_len, batch, max_q_len, q_heads, kv_heads,
+                                  head_dim, max_len, scale, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

@@ -90,7 +90,7 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
     const int nwg = gridDim.x;
     if ((nwg & 7) == 0) lid = (lid & 7) * (nwg >> 3) + (lid >> 3);  // consecutive ids share an XCD
   }
-  constexpr int GROUP = 4;
+  constexpr int GROUP = 8;
   const int per_group = GROUP * tiles_n;
   const int group_id = lid / per_group;
   const int first_m = group_id * GROUP;

@@ -1,0 +1,154 @@
+"""A self-contained Qwen3-architecture decoder that drives the invariant kernels end to end.
+
+It plays the role the vLLM engine plays for the reference (simple_inference.py:62-105: same prompts, different
+(TP, batch) settings, compare outputs): RMSNorm -> qkv projection (batch-invariant mm) -> per-head q/k RMSNorm ->
+rotary embedding -> fixed-order attention -> o_proj (tree matmul, K sharded over `tp_size` simulated ranks and
+combined in the all-reduce tree order) -> gated MLP with down_proj as a tree matmul -> lm_head -> greedy argmax.
+Every op either is elementwise or fixes its reduction order per row, so the generated token ids are identical
+for every simulated TP degree and every batch composition.
+
+Random-initialised weights only (N(0, 0.02), norm weights 1): this is a correctness and benchmarking vehicle,
+not a checkpoint loader.
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+from typing import List, Optional
+
+import torch
+
+from . import ops
+from .bio.batch_invariant_ops import matmul_persistent, rms_norm
+from .layers import SimulatedTPRowLinear
+from .patch.patch_training_inference_align import compute_inv_freq
+
+
+@dataclass
+class DecoderConfig:
+    vocab_size: int = 151936
+    hidden_size: int = 4096
+    num_layers: int = 36
+    num_q_heads: int = 32
+    num_kv_heads: int = 8
+    head_dim: int = 128
+    intermediate_size: int = 12288
+    rope_theta: float = 1e6
+    rms_eps: float = 1e-6
+
+
+class _Layer:
+    def __init__(self, cfg: DecoderConfig, tp_size: int, gen: torch.Generator, device):
+        def w(*shape):
+            return (torch.randn(shape, generator=gen, dtype=torch.float32) * 0.02).to(torch.bfloat16).to(device)
+        H, D = cfg.hidden_size, cfg.head_dim
+        self.input_norm = torch.ones(H, dtype=torch.bfloat16, device=device)
+        self.post_norm = torch.ones(H, dtype=torch.bfloat16, device=device)
+        self.q_norm = torch.ones(D, dtype=torch.bfloat16, device=device)
+        self.k_norm = torch.ones(D, dtype=torch.bfloat16, device=device)
+        self.qkv_w = w((cfg.num_q_heads + 2 * cfg.num_kv_heads) * D, H)          # column-parallel in a real TP run
+        self.gate_up_w = w(2 * cfg.intermediate_size, H)
+        self.o_proj = SimulatedTPRowLinear(w(H, cfg.num_q_heads * D), tp_size)    # row-parallel: K sharded
+        self.down_proj = SimulatedTPRowLinear(w(H, cfg.intermediate_size), tp_size)
+
+
+class Qwen3Decoder:
+    def __init__(self, cfg: DecoderConfig, tp_size: int = 1, seed: int = 0, device="cuda:0"):
+        assert cfg.head_dim == 128, "the attention kernel is built for head_dim 128"
+        self.cfg, self.tp_size, self.device = cfg, tp_size, torch.device(device)
+        gen = torch.Generator().manual_seed(seed)
+        emb = lambda *shape: (torch.randn(shape, generator=gen, dtype=torch.float32) * 0.02).to(torch.bfloat16).to(self.device)  # noqa: E731
+        self.embed = emb(cfg.vocab_size, cfg.hidden_size)
+        self.layers = [_Layer(cfg, tp_size, gen, self.device) for _ in range(cfg.num_layers)]
+        self.final_norm = torch.ones(cfg.hidden_size, dtype=torch.bfloat16, device=self.device)
+        self.lm_head = emb(cfg.vocab_size, cfg.hidden_size)
+        self.inv_freq = compute_inv_freq(cfg.head_dim, cfg.rope_theta, self.device)  # fp32 table built on the CPU
+        self.scale = 1.0 / math.sqrt(cfg.head_dim)
+
+    # ------------------------------------------------------------------------------------------
+    def _rope(self, x: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
+        """Rotate-half rotary embedding in fp32, rounded once to bf16 (elementwise: batch invariant)."""
+        ang = positions.to(torch.float32)[:, None] * self.inv_freq[None, :]            # [tokens, D/2]
+        cos, sin = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+        xf = x.float()
+        x1, x2 = xf[..., : x.shape[-1] // 2], xf[..., x.shape[-1] // 2:]
+        return torch.cat((x1 * cos - x2 * sin, x2 * cos + x1 * sin), dim=-1).to(torch.bfloat16)
+
+    def _forward(self, token_ids: torch.Tensor, positions: torch.Tensor, seq_of_token: torch.Tensor,
+                 q_start: torch.Tensor, q_len: torch.Tensor, ctx_len: torch.Tensor, max_q_len: int, cache) -> torch.Tensor:
+        cfg = self.cfg
+        Hq, Hkv, D = cfg.num_q_heads, cfg.num_kv_heads, cfg.head_dim
+        x = self.embed[token_ids]                                   # [tokens, H]
+        residual: Optional[torch.Tensor] = None
+        for li, layer in enumerate(self.layers):
+            if residual is None:
+                residual = x
+                h = rms_norm(x, layer.input_norm, cfg.rms_eps)
+            else:
+                h, residual = rms_norm(x, layer.input_norm, cfg.rms_eps, residual=residual)
+            qkv = matmul_persistent(h, layer.qkv_w.t())
+            q = qkv[:, : Hq * D].reshape(-1, Hq, D)
+            k = qkv[:, Hq * D: (Hq + Hkv) * D].reshape(-1, Hkv, D)
+            v = qkv[:, (Hq + Hkv) * D:].reshape(-1, Hkv, D)
+            q = self._rope(rms_norm(q.contiguous(), layer.q_norm, cfg.rms_eps), positions)
+            k = self._rope(rms_norm(k.contiguous(), layer.k_norm, cfg.rms_eps), positions)
+            k_cache, vt_cache = cache[li]
+            k_cache[seq_of_token, :, positions] = k                 # [tokens, Hkv, D] -> [B, Hkv, L, D]
+            vt_cache[seq_of_token, :, :, positions] = v             # stored transposed: [B, Hkv, D, L]
+            attn = ops.bi_attention_bf16(q, k_cache, vt_cache, q_start, q_len, ctx_len, max_q_len, self.scale)
+            x = layer.o_proj(attn.reshape(-1, Hq * D))
+            h, residual = rms_norm(x, layer.post_norm, cfg.rms_eps, residual=residual)
+            gu = matmul_persistent(h, layer.gate_up_w.t())
+            act = torch.nn.functional.silu(gu[:, : cfg.intermediate_size]) * gu[:, cfg.intermediate_size:]
+            x = layer.down_proj(act)
+        h, _ = rms_norm(x, self.final_norm, cfg.rms_eps, residual=residual)
+        return h
+
+    @staticmethod
+    def _greedy(logits: torch.Tensor) -> torch.Tensor:
+        """argmax with ties resolved to the lowest index (exact: a max and a min, no order dependence)."""
+        mx = logits.max(dim=-1, keepdim=True).values
+        idx = torch.arange(logits.shape[-1], device=logits.device)
+        return torch.where(logits == mx, idx, logits.shape[-1]).min(dim=-1).values
+
+    # ------------------------------------------------------------------------------------------
+    @torch.no_grad()
+    def generate(self, prompts: List[List[int]], max_new_tokens: int, return_logits: bool = False):
+        """Greedy decoding of a batch of prompts (ragged lengths allowed). Returns [batch, max_new_tokens] ids."""
+        cfg, dev = self.cfg, self.device
+        B = len(prompts)
+        lens = [len(p) for p in prompts]
+        max_len = ((max(lens) + max_new_tokens + 31) // 32) * 32
+        cache = [(torch.zeros((B, cfg.num_kv_heads, max_len, cfg.head_dim), dtype=torch.bfloat16, device=dev),
+                  torch.zeros((B, cfg.num_kv_heads, cfg.head_dim, max_len), dtype=torch.bfloat16, device=dev))
+                 for _ in range(cfg.num_layers)]
+        # ---- prefill: all prompt tokens, token-major
+        tok = torch.tensor([t for p in prompts for t in p], dtype=torch.long, device=dev)
+        pos = torch.tensor([i for n in lens for i in range(n)], dtype=torch.long, device=dev)
+        seq = torch.tensor([b for b, n in enumerate(lens) for _ in range(n)], dtype=torch.long, device=dev)
+        starts = [0]
+        for n in lens[:-1]:
+            starts.append(starts[-1] + n)
+        q_start = torch.tensor(starts, dtype=torch.int32, device=dev)
+        q_len = torch.tensor(lens, dtype=torch.int32, device=dev)
+        ctx = torch.tensor(lens, dtype=torch.int32, device=dev)
+        h = self._forward(tok, pos, seq, q_start, q_len, ctx, max(lens), cache)
+        last = torch.tensor([s + n - 1 for s, n in zip(starts, lens)], dtype=torch.long, device=dev)
+        logits = matmul_persistent(h[last].contiguous(), self.lm_head.t())
+        out_ids = [self._greedy(logits)]
+        all_logits = [logits] if return_logits else None
+        # ---- decode: one token per sequence per step
+        q_start = torch.arange(B, dtype=torch.int32, device=dev)
+        q_len = torch.ones(B, dtype=torch.int32, device=dev)
+        seq = torch.arange(B, dtype=torch.long, device=dev)
+        cur = torch.tensor(lens, dtype=torch.long, device=dev)
+        for _ in range(max_new_tokens - 1):
+            ctx = (cur + 1).to(torch.int32)
+            h = self._forward(out_ids[-1], cur, seq, q_start, q_len, ctx, 1, cache)
+            logits = matmul_persistent(h, self.lm_head.t())
+            out_ids.append(self._greedy(logits))
+            if return_logits:
+                all_logits.append(logits)
+            cur = cur + 1
+        ids = torch.stack(out_ids, dim=1)
+        return (ids, torch.stack(all_logits, dim=1)) if return_logits else ids

@@ -2,7 +2,11 @@
 
 Each op allocates its output with torch, passes raw device pointers, element strides and the current
 HIP stream to one `extern "C"` entry point, and raises on a non-zero return code.  The ops are
-registered for the GPU device type only: calling them on CPU tensors raises -- there is no CPU path.
+registered as `torch.ops.tbik.*` for the GPU device type only; there is no CPU path, CPU tensors raise.
+
+Eager callers reach the same implementation function directly (the dispatcher round trip of a Python
+custom op costs ~10 us per call, more than most of these kernels take); under torch.compile the
+registered op is used so the call stays a single opaque node.
 """
 from __future__ import annotations
 
@@ -52,8 +56,7 @@ def _weight_nk(B: torch.Tensor):
 # --------------------------------------------------------------------------------------------
 # tree-ordered GEMM
 # --------------------------------------------------------------------------------------------
-@torch.library.custom_op("tbik::gemm_tree_bf16", mutates_args=(), device_types="cuda")
-def gemm_tree_bf16(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.Tensor], leaf_k: int) -> torch.Tensor:
+def _gemm_tree_bf16_impl(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.Tensor], leaf_k: int) -> torch.Tensor:
     _require_gpu(A, B, bias)
     M, K = A.shape
     N = B.shape[1]
@@ -71,13 +74,21 @@ def gemm_tree_bf16(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.Tensor
     return C
 
 
-@gemm_tree_bf16.register_fake
+_gemm_tree_bf16_op = torch.library.custom_op("tbik::gemm_tree_bf16", _gemm_tree_bf16_impl, mutates_args=(), device_types="cuda")
+
+
+def gemm_tree_bf16(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.Tensor], leaf_k: int) -> torch.Tensor:
+    if torch.compiler.is_compiling():
+        return _gemm_tree_bf16_op(A, B, bias, leaf_k)
+    return _gemm_tree_bf16_impl(A, B, bias, leaf_k)
+
+
+@_gemm_tree_bf16_op.register_fake
 def _(A, B, bias, leaf_k):
     return A.new_empty((A.shape[0], B.shape[1]))
 
 
-@torch.library.custom_op("tbik::tree_combine_bf16", mutates_args=(), device_types="cuda")
-def tree_combine_bf16(parts: List[torch.Tensor]) -> torch.Tensor:
+def _tree_combine_bf16_impl(parts: List[torch.Tensor]) -> torch.Tensor:
     _require_gpu(*parts)
     ps = [p.contiguous() for p in parts]
     out = torch.empty_like(ps[0])
@@ -87,7 +98,16 @@ def tree_combine_bf16(parts: List[torch.Tensor]) -> torch.Tensor:
     return out
 
 
-@tree_combine_bf16.register_fake
+_tree_combine_bf16_op = torch.library.custom_op("tbik::tree_combine_bf16", _tree_combine_bf16_impl, mutates_args=(), device_types="cuda")
+
+
+def tree_combine_bf16(parts: List[torch.Tensor]) -> torch.Tensor:
+    if torch.compiler.is_compiling():
+        return _tree_combine_bf16_op(parts)
+    return _tree_combine_bf16_impl(parts)
+
+
+@_tree_combine_bf16_op.register_fake
 def _(parts):
     return torch.empty_like(parts[0])
 
@@ -95,8 +115,7 @@ def _(parts):
 # --------------------------------------------------------------------------------------------
 # batch-invariant ops
 # --------------------------------------------------------------------------------------------
-@torch.library.custom_op("tbik::bi_gemm_bf16", mutates_args=(), device_types="cuda")
-def bi_gemm_bf16(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
+def _bi_gemm_bf16_impl(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
     _require_gpu(A, B, bias)
     M, K = A.shape
     N = B.shape[1]
@@ -116,13 +135,21 @@ def bi_gemm_bf16(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.Tensor])
     return C
 
 
-@bi_gemm_bf16.register_fake
+_bi_gemm_bf16_op = torch.library.custom_op("tbik::bi_gemm_bf16", _bi_gemm_bf16_impl, mutates_args=(), device_types="cuda")
+
+
+def bi_gemm_bf16(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
+    if torch.compiler.is_compiling():
+        return _bi_gemm_bf16_op(A, B, bias)
+    return _bi_gemm_bf16_impl(A, B, bias)
+
+
+@_bi_gemm_bf16_op.register_fake
 def _(A, B, bias):
     return A.new_empty((A.shape[0], B.shape[1]))
 
 
-@torch.library.custom_op("tbik::bi_rmsnorm_bf16", mutates_args=(), device_types="cuda")
-def bi_rmsnorm_bf16(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float) -> torch.Tensor:
+def _bi_rmsnorm_bf16_impl(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float) -> torch.Tensor:
     _require_gpu(x, weight)
     hidden = x.shape[-1]
     x2, ldx = _rows16(x.reshape(-1, hidden))
@@ -134,13 +161,21 @@ def bi_rmsnorm_bf16(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float)
     return out.reshape(x.shape)
 
 
-@bi_rmsnorm_bf16.register_fake
+_bi_rmsnorm_bf16_op = torch.library.custom_op("tbik::bi_rmsnorm_bf16", _bi_rmsnorm_bf16_impl, mutates_args=(), device_types="cuda")
+
+
+def bi_rmsnorm_bf16(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float) -> torch.Tensor:
+    if torch.compiler.is_compiling():
+        return _bi_rmsnorm_bf16_op(x, weight, eps)
+    return _bi_rmsnorm_bf16_impl(x, weight, eps)
+
+
+@_bi_rmsnorm_bf16_op.register_fake
 def _(x, weight, eps):
     return torch.empty_like(x)
 
 
-@torch.library.custom_op("tbik::bi_add_rmsnorm_bf16", mutates_args=(), device_types="cuda")
-def bi_add_rmsnorm_bf16(x: torch.Tensor, residual: torch.Tensor, weight: Optional[torch.Tensor],
+def _bi_add_rmsnorm_bf16_impl(x: torch.Tensor, residual: torch.Tensor, weight: Optional[torch.Tensor],
                         eps: float) -> List[torch.Tensor]:
     _require_gpu(x, residual, weight)
     hidden = x.shape[-1]
@@ -156,13 +191,22 @@ def bi_add_rmsnorm_bf16(x: torch.Tensor, residual: torch.Tensor, weight: Optiona
     return [out.reshape(x.shape), rout.reshape(x.shape)]
 
 
-@bi_add_rmsnorm_bf16.register_fake
+_bi_add_rmsnorm_bf16_op = torch.library.custom_op("tbik::bi_add_rmsnorm_bf16", _bi_add_rmsnorm_bf16_impl, mutates_args=(), device_types="cuda")
+
+
+def bi_add_rmsnorm_bf16(x: torch.Tensor, residual: torch.Tensor, weight: Optional[torch.Tensor],
+                        eps: float) -> List[torch.Tensor]:
+    if torch.compiler.is_compiling():
+        return _bi_add_rmsnorm_bf16_op(x, residual, weight, eps)
+    return _bi_add_rmsnorm_bf16_impl(x, residual, weight, eps)
+
+
+@_bi_add_rmsnorm_bf16_op.register_fake
 def _(x, residual, weight, eps):
     return [torch.empty_like(x), torch.empty_like(x)]
 
 
-@torch.library.custom_op("tbik::bi_log_softmax_f32", mutates_args=(), device_types="cuda")
-def bi_log_softmax_f32(x: torch.Tensor, write_softmax: bool) -> torch.Tensor:
+def _bi_log_softmax_f32_impl(x: torch.Tensor, write_softmax: bool) -> torch.Tensor:
     _require_gpu(x)
     cols = x.shape[-1]
     x2 = x.reshape(-1, cols)
@@ -178,13 +222,21 @@ def bi_log_softmax_f32(x: torch.Tensor, write_softmax: bool) -> torch.Tensor:
     return out.reshape(x.shape)
 
 
-@bi_log_softmax_f32.register_fake
+_bi_log_softmax_f32_op = torch.library.custom_op("tbik::bi_log_softmax_f32", _bi_log_softmax_f32_impl, mutates_args=(), device_types="cuda")
+
+
+def bi_log_softmax_f32(x: torch.Tensor, write_softmax: bool) -> torch.Tensor:
+    if torch.compiler.is_compiling():
+        return _bi_log_softmax_f32_op(x, write_softmax)
+    return _bi_log_softmax_f32_impl(x, write_softmax)
+
+
+@_bi_log_softmax_f32_op.register_fake
 def _(x, write_softmax):
     return torch.empty_like(x)
 
 
-@torch.library.custom_op("tbik::bi_mean_dim", mutates_args=(), device_types="cuda")
-def bi_mean_dim(x: torch.Tensor, dim: int, keepdim: bool) -> torch.Tensor:
+def _bi_mean_dim_impl(x: torch.Tensor, dim: int, keepdim: bool) -> torch.Tensor:
     _require_gpu(x)
     if x.dtype not in _DTYPE_CODE:
         raise NotImplementedError(f"bi_mean_dim: unsupported dtype {x.dtype}")
@@ -205,9 +257,55 @@ def bi_mean_dim(x: torch.Tensor, dim: int, keepdim: bool) -> torch.Tensor:
     return out
 
 
-@bi_mean_dim.register_fake
+_bi_mean_dim_op = torch.library.custom_op("tbik::bi_mean_dim", _bi_mean_dim_impl, mutates_args=(), device_types="cuda")
+
+
+def bi_mean_dim(x: torch.Tensor, dim: int, keepdim: bool) -> torch.Tensor:
+    if torch.compiler.is_compiling():
+        return _bi_mean_dim_op(x, dim, keepdim)
+    return _bi_mean_dim_impl(x, dim, keepdim)
+
+
+@_bi_mean_dim_op.register_fake
 def _(x, dim, keepdim):
     dim = dim % x.ndim
     shape = list(x.shape)
     out_shape = shape[:dim] + ([1] if keepdim else []) + shape[dim + 1:]
     return x.new_empty(out_shape)
+
+
+# --------------------------------------------------------------------------------------------
+# fixed-order attention
+# --------------------------------------------------------------------------------------------
+def _bi_attention_bf16_impl(q: torch.Tensor, k_cache: torch.Tensor, vt_cache: torch.Tensor, q_start: torch.Tensor,
+                            q_len: torch.Tensor, ctx_len: torch.Tensor, max_q_len: int, scale: float) -> torch.Tensor:
+    _require_gpu(q, k_cache, vt_cache, q_start, q_len, ctx_len)
+    tokens, q_heads, head_dim = q.shape
+    batch, kv_heads, max_len, _ = k_cache.shape
+    assert vt_cache.shape == (batch, kv_heads, head_dim, max_len)
+    assert q.dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16 and vt_cache.dtype == torch.bfloat16
+    assert q_start.dtype == torch.int32 and q_len.dtype == torch.int32 and ctx_len.dtype == torch.int32
+    q = q.contiguous()
+    assert k_cache.is_contiguous() and vt_cache.is_contiguous()
+    out = torch.empty_like(q)
+    rc = _lib.lib().bi_attention_bf16(q.data_ptr(), k_cache.data_ptr(), vt_cache.data_ptr(), out.data_ptr(),
+                                      q_start.data_ptr(), q_len.data_ptr(), ctx_len.data_ptr(), batch, max_q_len,
+                                      q_heads, kv_heads, head_dim, max_len, scale, _stream(q))
+    _lib.check(rc, "bi_attention_bf16")
+    return out
+
+
+_bi_attention_bf16_op = torch.library.custom_op("tbik::bi_attention_bf16", _bi_attention_bf16_impl, mutates_args=(),
+                                                device_types="cuda")
+
+
+def bi_attention_bf16(q: torch.Tensor, k_cache: torch.Tensor, vt_cache: torch.Tensor, q_start: torch.Tensor,
+                      q_len: torch.Tensor, ctx_len: torch.Tensor, max_q_len: int, scale: float) -> torch.Tensor:
+    if torch.compiler.is_compiling():
+        return _bi_attention_bf16_op(q, k_cache, vt_cache, q_start, q_len, ctx_len, max_q_len, scale)
+    return _bi_attention_bf16_impl(q, k_cache, vt_cache, q_start, q_len, ctx_len, max_q_len, scale)
+
+
+@_bi_attention_bf16_op.register_fake
+def _(q, k_cache, vt_cache, q_start, q_len, ctx_len, max_q_len, scale):
+    return torch.empty_like(q)

@@ -1,0 +1,141 @@
+"""Fixed-order attention and the end-to-end greedy decode (the reference's simple_inference.py check: same prompts
+under different (TP, batch) settings must give the same outputs), on a small random-init Qwen3-architecture model."""
+import math
+
+import pytest
+import torch
+
+from llm_reproducibility_amd import ops
+from llm_reproducibility_amd.decoder import DecoderConfig, Qwen3Decoder
+
+pytestmark = pytest.mark.gpu
+
+
+def _ref_attention(q, k, v, scale):
+    """fp32 causal attention of one sequence: q [n, Hq, D] are the LAST n positions of k/v [L, Hkv, D]."""
+    n, Hq, D = q.shape
+    L, Hkv, _ = k.shape
+    rep = Hq // Hkv
+    kf = k.float().repeat_interleave(rep, dim=1)
+    vf = v.float().repeat_interleave(rep, dim=1)
+    s = torch.einsum("qhd,khd->hqk", q.float(), kf) * scale
+    qpos = torch.arange(L - n, L, device=q.device)[:, None]
+    kpos = torch.arange(L, device=q.device)[None, :]
+    s = s.masked_fill(kpos > qpos, float("-inf"))
+    return torch.einsum("hqk,khd->qhd", torch.softmax(s, dim=-1), vf)
+
+
+def _make_cache(ks, vs, max_len, dev):
+    B, Hkv, D = len(ks), ks[0].shape[1], ks[0].shape[2]
+    kc = torch.zeros((B, Hkv, max_len, D), dtype=torch.bfloat16, device=dev)
+    vt = torch.zeros((B, Hkv, D, max_len), dtype=torch.bfloat16, device=dev)
+    for b, (k, v) in enumerate(zip(ks, vs)):
+        kc[b, :, : k.shape[0]] = k.transpose(0, 1)
+        vt[b, :, :, : v.shape[0]] = v.permute(1, 2, 0)
+    return kc, vt
+
+
+def test_attention_matches_fp32_reference_and_is_batch_and_phase_invariant(dev):
+    torch.manual_seed(0)
+    Hq, Hkv, D, scale = 8, 2, 128, 1.0 / math.sqrt(128)
+    lens = [70, 33, 1, 128, 17]
+    ks = [torch.randn((n, Hkv, D), device=dev).to(torch.bfloat16) for n in lens]
+    vs = [torch.randn((n, Hkv, D), device=dev).to(torch.bfloat16) for n in lens]
+    qs = [torch.randn((n, Hq, D), device=dev).to(torch.bfloat16) for n in lens]
+    max_len = 160
+    kc, vt = _make_cache(ks, vs, max_len, dev)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)  # noqa: E731
+    starts = [sum(lens[:i]) for i in range(len(lens))]
+    # prefill of the whole ragged batch
+    out = ops.bi_attention_bf16(torch.cat(qs), kc, vt, i32(starts), i32(lens), i32(lens), max(lens), scale)
+    for b, n in enumerate(lens):
+        want = _ref_attention(qs[b], ks[b], vs[b], scale)
+        got = out[starts[b]: starts[b] + n].float()
+        assert (got - want).abs().max() < 2e-2, (b, (got - want).abs().max())
+    # a sequence alone == the same sequence inside the batch (bitwise)
+    for b in (0, 3):
+        kc1, vt1 = _make_cache([ks[b]], [vs[b]], max_len, dev)
+        alone = ops.bi_attention_bf16(qs[b], kc1, vt1, i32([0]), i32([lens[b]]), i32([lens[b]]), lens[b], scale)
+        assert torch.equal(alone, out[starts[b]: starts[b] + lens[b]]), b
+    # decode phase: the last token of every sequence as a single-query call == its prefill row (bitwise)
+    q_last = torch.stack([q[-1] for q in qs])
+    dec = ops.bi_attention_bf16(q_last, kc, vt, i32(list(range(len(lens)))), i32([1] * len(lens)), i32(lens), 1, scale)
+    for b, n in enumerate(lens):
+        assert torch.equal(dec[b], out[starts[b] + n - 1]), b
+    # chunked prefill: the last 5 tokens of sequence 0 against the cache == the same rows of the full prefill
+    tail = ops.bi_attention_bf16(qs[0][-5:], kc[:1], vt[:1], i32([0]), i32([5]), i32([lens[0]]), 5, scale)
+    assert torch.equal(tail, out[starts[0] + lens[0] - 5: starts[0] + lens[0]])
+
+
+SMALL = DecoderConfig(vocab_size=3000, hidden_size=1024, num_layers=2, num_q_heads=16, num_kv_heads=4, head_dim=128,
+                      intermediate_size=4096)
+
+
+def _prompts(n, seed=1):
+    g = torch.Generator().manual_seed(seed)
+    lens = [37, 64, 5, 48, 21, 33, 16, 50][:n]
+    return [torch.randint(0, SMALL.vocab_size, (L,), generator=g).tolist() for L in lens]
+
+
+def test_greedy_decode_is_identical_across_tp_and_batch(dev):
+    prompts = _prompts(8)
+    new = 10
+    base_model = Qwen3Decoder(SMALL, tp_size=1, seed=0, device=dev)
+    base_ids, base_logits = base_model.generate(prompts, new, return_logits=True)
+    assert base_ids.shape == (8, new)
+    assert torch.isfinite(base_logits.float()).all()
+    # batch composition: each prompt alone, and a sub-batch, must reproduce its row bit for bit (logits included)
+    for b in (0, 2, 7):
+        ids, logits = base_model.generate([prompts[b]], new, return_logits=True)
+        assert torch.equal(ids[0], base_ids[b]), b
+        assert torch.equal(logits[0], base_logits[b]), b
+    ids3 = base_model.generate(prompts[2:5], new)
+    assert torch.equal(ids3, base_ids[2:5])
+    del base_model
+    # simulated tensor parallelism: same seed -> same weights, row-split layers sharded 2/4/8 ways
+    for tp in (2, 4, 8):
+        m = Qwen3Decoder(SMALL, tp_size=tp, seed=0, device=dev)
+        ids, logits = m.generate(prompts, new, return_logits=True)
+        assert torch.equal(ids, base_ids), tp
+        assert torch.equal(logits, base_logits), tp
+        one = m.generate([prompts[5]], new)
+        assert torch.equal(one[0], base_ids[5]), tp
+        del m
+
+
+def test_decoder_logits_agree_with_plain_pytorch_math(dev):
+    """Tolerance check of the whole stack against a straightforward fp32 PyTorch forward of the same weights."""
+    cfg = DecoderConfig(vocab_size=512, hidden_size=512, num_layers=2, num_q_heads=8, num_kv_heads=2, head_dim=128,
+                        intermediate_size=2048)
+    m = Qwen3Decoder(cfg, tp_size=2, seed=3, device=dev)
+    g = torch.Generator().manual_seed(5)
+    prompt = torch.randint(0, cfg.vocab_size, (29,), generator=g).tolist()
+    _, logits = m.generate([prompt], 1, return_logits=True)
+
+    def norm(x, w):
+        return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + cfg.rms_eps) * w.float()
+
+    x = m.embed[torch.tensor(prompt, device=dev)].float()
+    pos = torch.arange(len(prompt), device=dev)
+    ang = pos.float()[:, None] * m.inv_freq[None, :]
+    cos, sin = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+
+    def rope(t):
+        a, b = t[..., :64], t[..., 64:]
+        return torch.cat((a * cos - b * sin, b * cos + a * sin), -1)
+
+    Hq, Hkv, D = cfg.num_q_heads, cfg.num_kv_heads, cfg.head_dim
+    for layer in m.layers:
+        h = norm(x, layer.input_norm)
+        qkv = h @ layer.qkv_w.float().t()
+        q = rope(norm(qkv[:, : Hq * D].reshape(-1, Hq, D), layer.q_norm))
+        k = rope(norm(qkv[:, Hq * D: (Hq + Hkv) * D].reshape(-1, Hkv, D), layer.k_norm))
+        v = qkv[:, (Hq + Hkv) * D:].reshape(-1, Hkv, D)
+        att = _ref_attention(q, k, v, m.scale).reshape(-1, Hq * D)
+        x = x + att @ layer.o_proj.weight.float().t()
+        h = norm(x, layer.post_norm)
+        gu = h @ layer.gate_up_w.float().t()
+        x = x + (torch.nn.functional.silu(gu[:, : cfg.intermediate_size]) * gu[:, cfg.intermediate_size:]) @ layer.down_proj.weight.float().t()
+    want = norm(x[-1:], m.final_norm) @ m.lm_head.float().t()
+    got = logits[0, 0].float()
+    assert (got - want[0]).abs().max() <= 0.05 * want.abs().max() + 0.02, ((got - want[0]).abs().max(), want.abs().max())
