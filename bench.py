@@ -85,6 +85,12 @@ def table(steps, warmup):
         gemm_row(f"o_proj 32B    M={M} K=8192 N=5120", M, 8192, 5120, 256)
     for M in (1, 64, 512, 4096):
         gemm_row(f"down_proj 32B M={M} K=25600 N=5120 leaf128", M, 25600, 5120, choose_leaf_k(25600))
+    for name, M, K, N in (("qkv 8B", 2048, 4096, 6144), ("gate_up 8B", 2048, 4096, 24576), ("lm_head 8B", 128, 4096, 151936)):
+        X = torch.randn((M, K), device=dev).to(torch.bfloat16)
+        W = (torch.randn((N, K), device=dev) * 0.02).to(torch.bfloat16)
+        ms, _ = hip_time_ms(lambda: bio.matmul_persistent(X, W.t()), steps, warmup)
+        rows.append((f"batch-invariant mm {name} M={M} K={K} N={N}", ms * 1e3, 2.0 * M * N * K / ms / 1e9,
+                     2.0 * (M * K + K * N + M * N) / ms / 1e6))
     for p in (2, 4, 8):
         parts = [torch.randn((2048, 4096), device=dev).to(torch.bfloat16) for _ in range(p)]
         ms, _ = hip_time_ms(lambda: tree_combine(parts), steps, warmup)

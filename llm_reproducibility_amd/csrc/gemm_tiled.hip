@@ -415,7 +415,16 @@ int gemm_dispatch(bool tree, const void* A, int64_t lda, const void* B, int64_t 
   a.vec_store = ((reinterpret_cast<uintptr_t>(C) & 7) == 0 && (ldc & 3) == 0) ? 1 : 0;
   a.k_shard = 0;
   a.c_shard = 0;
-  if (!tree) return launch_by_m<4, 0, false>(a, 1, stream);
+  if (!tree) {
+    // large problems whose K is a whole number of 256-wide spans take the wide pipeline (same MFMA chain per
+    // element, so the same bits as the tiled kernel)
+    const int64_t wide_tiles = (int64_t)((M + 127) / 128) * ((N + 255) / 256);
+    if (M > 64 && wide_tiles >= 128 && (K & 255) == 0) {
+      WideArgs w{a.X, a.W, a.C, a.bias, nullptr, a.ldx, a.ldw, a.ldc, M, N, K, K / 256, 1, 0, a.vec_store, 0, 0};
+      return gemm_tree_wide_launch(w, 0, 1, stream);
+    }
+    return launch_by_m<4, 0, false>(a, 1, stream);
+  }
 
   if (leaf_k != 256 && leaf_k != 128) return TBIK_ERR_UNSUPPORTED;
   Plan pl;

@@ -72,7 +72,9 @@ __device__ __forceinline__ void store16_sbase(void* base, uint32_t voff, u32x4 v
   asm volatile("global_store_dwordx4 %0, %1, %2" : : "v"(voff), "v"(v), "s"(base) : "memory");
 }
 
-template <int LS>
+// TREE = false: the same pipeline with ONE fp32 accumulator run over all of K (the batch-invariant mm); T counts
+// 256-wide spans of K, nothing is merged, and a bias is added in fp32 before the single rounding.
+template <int LS, bool TREE = true>
 __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs p) {
   using namespace wide;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -256,7 +258,7 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
 #pragma unroll
           for (int b = 0; b < TN; b++) {
             const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-            acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[b], fx[a], (i == 0 && kk == 0) ? zero : acc[a][b], 0, 0, 0);
+            acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[b], fx[a], (i == 0 && kk == 0 && (TREE || j == 0)) ? zero : acc[a][b], 0, 0, 0);
           }
           const int d = kk * TM + a;  // 0..7: loads 0..5 go out after MFMA rows 0..5
           if (d < NDMA) {
@@ -274,6 +276,10 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
 
   int kind = K_NONE;
   for (int j = 0; j < p.T; j++) {
+    if (!TREE) {
+      leaf_body(std::integral_constant<int, K_NONE>{}, j);
+      continue;
+    }
     switch (kind) {
       case K_NONE: leaf_body(std::integral_constant<int, K_NONE>{}, j); break;
       case K_ADD: leaf_body(std::integral_constant<int, K_ADD>{}, j); break;
@@ -317,22 +323,24 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
   }
 
   // ---- the last leaf: every level carries, t ends as the root
+  if (TREE) {
 #pragma unroll
-  for (int a = 0; a < TM; a++)
+    for (int a = 0; a < TM; a++)
 #pragma unroll
-    for (int b = 0; b < TN; b++) {
-      t[(a * TN + b) * 2] = pack_bf16x2(acc[a][b][0], acc[a][b][1]);
-      t[(a * TN + b) * 2 + 1] = pack_bf16x2(acc[a][b][2], acc[a][b][3]);
-    }
-  if (c0 != 0) {
+      for (int b = 0; b < TN; b++) {
+        t[(a * TN + b) * 2] = pack_bf16x2(acc[a][b][0], acc[a][b][1]);
+        t[(a * TN + b) * 2 + 1] = pack_bf16x2(acc[a][b][2], acc[a][b][3]);
+      }
+  }
+  if (TREE && c0 != 0) {
 #pragma unroll
     for (int r = 0; r < NREG; r++) t[r] = add_bf16x2(s0[r], t[r]);
   }
-  if (p.lb > 0) {
+  if (TREE && p.lb > 0) {
 #pragma unroll
     for (int r = 0; r < NREG; r++) t[r] = add_bf16x2(sb0[r], t[r]);
   }
-  if (p.lb > RL) {
+  if (TREE && p.lb > RL) {
 #pragma unroll
     for (int q = 0; q < 4; q++) chain_parked(q, RL, g);
   }
@@ -345,14 +353,23 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
     for (int b = 0; b < TN; b++) {
       const int n = n0 + (wn * TN + b) * 16 + fchk * 4;
       if (m >= p.M || n >= p.N) continue;
-      uint32_t lo = t[(a * TN + b) * 2], hi = t[(a * TN + b) * 2 + 1];
+      float bv[4] = {0.f, 0.f, 0.f, 0.f};
       if (p.bias) {
-        float bv[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int e = 0; e < 4; e++)
           if (n + e < p.N) bv[e] = bf16_bits_to_f32(p.bias[n + e]);
-        lo = add_bf16x2(lo, pack_bf16x2(bv[0], bv[1]));
-        hi = add_bf16x2(hi, pack_bf16x2(bv[2], bv[3]));
+      }
+      uint32_t lo, hi;
+      if (TREE) {
+        lo = t[(a * TN + b) * 2];
+        hi = t[(a * TN + b) * 2 + 1];
+        if (p.bias) {
+          lo = add_bf16x2(lo, pack_bf16x2(bv[0], bv[1]));
+          hi = add_bf16x2(hi, pack_bf16x2(bv[2], bv[3]));
+        }
+      } else {
+        lo = pack_bf16x2(acc[a][b][0] + bv[0], acc[a][b][1] + bv[1]);
+        hi = pack_bf16x2(acc[a][b][2] + bv[2], acc[a][b][3] + bv[3]);
       }
       uint16_t* dst = p.C + shard * p.c_shard + (int64_t)m * p.ldc + n;
       if (p.vec_store && n + 3 < p.N) {
@@ -378,6 +395,11 @@ int gemm_tree_wide_launch(const WideArgs& a, int leaf_k, int split, hipStream_t 
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return hip_code(e);
     hipLaunchKernelGGL(kern, dim3((unsigned)tiles, (unsigned)split), dim3(NT), smem, stream, a);
+  } else if (leaf_k == 0) {  // single accumulator over K (a multiple of 256)
+    auto kern = gemm_tree_wide_kernel<4, false>;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return hip_code(e);
+    hipLaunchKernelGGL(kern, dim3((unsigned)tiles, 1u), dim3(NT), smem, stream, a);
   } else if (leaf_k == 128) {
     auto kern = gemm_tree_wide_kernel<2>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);

@@ -111,6 +111,22 @@ def test_single_accumulator_mm_parity_and_batch_invariance(dev):
     assert torch.equal(got.cpu(), O.matmul_single_acc(ai, bi))
 
 
+def test_single_accumulator_mm_large_and_small_kernels_agree_bitwise(dev):
+    # M=2048 takes the wide pipeline, M<=64 the small-tile kernel: same MFMA chain per element, same bits
+    a = O.gaussian_bf16((2048, 1024), 1.0, 5)
+    w = O.gaussian_bf16((4096, 1024), 0.05, 6)
+    bias = O.gaussian_bf16((4096,), 1.0, 7)
+    ad, wd, bd = a.to(dev), w.to(dev), bias.to(dev)
+    full = bio.matmul_persistent(ad, wd.t(), bd)
+    for m in (1, 16, 64, 300):
+        assert torch.equal(bio.matmul_persistent(ad[:m], wd.t(), bd), full[:m]), m
+    want = O.matmul_single_acc(a[:256], w.t(), bias)
+    assert not O.outside_tolerance(full[:256], want).any()
+    ai = O.integer_bf16((2048, 512), -9, 9, 8)
+    wi = O.integer_bf16((4096, 512), -7, 7, 9)
+    assert torch.equal(bio.matmul_persistent(ai.to(dev), wi.to(dev).t()).cpu(), O.matmul_single_acc(ai, wi.t()))
+
+
 def test_aten_overrides_route_to_the_hip_kernels(dev):
     a = O.gaussian_bf16((20, 512), 1.0, 0).to(dev)
     w = O.gaussian_bf16((64, 512), 0.1, 1).to(dev)
