@@ -1,0 +1,191 @@
+// Batch-invariant bf16 GEMM (one fp32 accumulator per element, K strictly ascending) for gfx950, large-M path:
+// 128x256 output tile per work-group, 4 wavefronts (one per SIMD) of 64x128 each, K streamed through a 3-slot
+// LDS ring in 64-element slices.  Replaces matmul_kernel_persistent, src/bio/batch_invariant_ops.py:42-124, for
+// shapes that fill the chip; per element it issues the same MFMA chain as the small-tile kernel in gemm_tiled.hip,
+// so the two produce identical bits and a row never sees M.
+//
+// Schedule (each choice measured on MI355X):
+//   * one wave per SIMD with a 64x128 tile keeps the LDS traffic at 24 B per MFMA clock, below the ~31 B/clk a
+//     single wave can pull from LDS (64x64 tiles need 32);
+//   * operands go global -> LDS directly (global_load_lds_dwordx4), ONE load per group of four MFMAs -- bursts of
+//     loads back up the texture path and stall the in-order wave -- two to three slices ahead; a lane fetches the
+//     global chunk that belongs at its linear LDS position, which realises the XOR bank swizzle on the source side;
+//   * one barrier per slice, placed BETWEEN its two 32-wide k steps, so fragment reads always run one k step
+//     ahead of the MFMAs, also across the barrier; scheduling fences keep that order in the generated code.
+#include "common.h"
+
+namespace tbik {
+
+struct QuadArgs {
+  const uint16_t* X;   // [M,K], row stride ldx
+  const uint16_t* W;   // [N,K], row stride ldw
+  uint16_t* C;         // [M,N], row stride ldc
+  const uint16_t* bias;
+  int64_t ldx, ldw, ldc;
+  int M, N, K;
+  int vec_store;
+};
+
+namespace quad {
+constexpr int BM = 128, BN = 256, BK = 64, NT = 256, NWAVE = 4, TM = 4, TN = 8;
+constexpr int ROWS = BM + BN, STAGE_BYTES = ROWS * BK * 2, NSLOT = 3;
+constexpr int NDMA = ROWS / 8 / NWAVE;  // 12 direct loads per wave per slice (8 rows of 128 B each)
+constexpr int XDMA = BM / 8 / NWAVE;    // of which X rows: 4
+}  // namespace quad
+
+__device__ __forceinline__ void quad_dma16(uint32_t lds_addr, uint32_t voff, const void* base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(base) : "memory");
+}
+
+__global__ __launch_bounds__(quad::NT) void gemm_single_acc_quad_kernel(const QuadArgs p) {
+  using namespace quad;
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+
+  const int tiles_m = (p.M + BM - 1) / BM;
+  const int tiles_n = (p.N + BN - 1) / BN;
+  int lid = blockIdx.x;
+  {
+    const int nwg = gridDim.x;
+    if ((nwg & 7) == 0) lid = (lid & 7) * (nwg >> 3) + (lid >> 3);  // consecutive ids share an XCD
+  }
+  constexpr int GROUP = 8;
+  const int per_group = GROUP * tiles_n;
+  const int group_id = lid / per_group;
+  const int first_m = group_id * GROUP;
+  const int gsz = min(tiles_m - first_m, GROUP);
+  const int pid_m = first_m + (lid % per_group) % gsz;
+  const int pid_n = (lid % per_group) / gsz;
+  const int m0 = pid_m * BM, n0 = pid_n * BN;
+
+  const uint8_t* xbase = reinterpret_cast<const uint8_t*>(p.X + (int64_t)m0 * p.ldx);
+  const uint8_t* wbase = reinterpret_cast<const uint8_t*>(p.W + (int64_t)n0 * p.ldw);
+  uint32_t voff[NDMA];
+  {
+    const int r = lane >> 3, c = (lane & 7) ^ r;
+#pragma unroll
+    for (int i = 0; i < NDMA; i++) {
+      const int row = (i * NWAVE + wave) * 8 + r;  // 0..383: X rows, then W rows; rows past the edge are clamped
+      if (i < XDMA) voff[i] = (uint32_t)(((min(m0 + row, p.M - 1) - m0) * p.ldx + c * 8) * 2);
+      else voff[i] = (uint32_t)(((min(n0 + row - BM, p.N - 1) - n0) * p.ldw + c * 8) * 2);
+    }
+  }
+  const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
+  const int nstages = p.K / BK;
+  auto dma_one = [&](int s, int slot, int i) __attribute__((always_inline)) {
+    const uint8_t* b = (i < XDMA ? xbase : wbase) + (int64_t)min(s, nstages - 1) * (BK * 2);
+    quad_dma16(lds0 + slot * STAGE_BYTES + (i * NWAVE + wave) * 1024, voff[i], b);
+  };
+  const int frow = lane & 15, fchk = lane >> 4;
+  const uint32_t xfrag = ((wm * TM * 16 + frow) * BK + ((fchk ^ (frow & 7)) << 3)) * 2;
+  const uint32_t wfrag = (BM * BK + (wn * TN * 16 + frow) * BK + ((fchk ^ (frow & 7)) << 3)) * 2;
+
+  f32x4 acc[TM][TN];
+  bf16x8 fx[2][TM], fw[2][TN];
+  auto read_x = [&](int buf, int slot, int kk, int a) __attribute__((always_inline)) {
+    fx[buf][a] = *reinterpret_cast<const bf16x8*>(smem + slot * STAGE_BYTES + (xfrag ^ (kk * 64)) + a * 16 * BK * 2);
+  };
+  auto read_w = [&](int buf, int slot, int kk, int b) __attribute__((always_inline)) {
+    fw[buf][b] = *reinterpret_cast<const bf16x8*>(smem + slot * STAGE_BYTES + (wfrag ^ (kk * 64)) + b * 16 * BK * 2);
+  };
+
+  // prologue: three slices in flight, slice 0 visible, fragments of the first k step loaded
+#pragma unroll
+  for (int s = 0; s < NSLOT; s++)
+#pragma unroll
+    for (int i = 0; i < NDMA; i++) dma_one(s, s, i);
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(2 * NDMA) : "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+#pragma unroll
+  for (int a = 0; a < TM; a++) read_x(0, 0, 0, a);
+#pragma unroll
+  for (int b = 0; b < TN; b++) read_w(0, 0, 0, b);
+
+  int slot = 0;
+  for (int s = 0; s < nstages; s++) {
+    const int nslot = slot + 1 == NSLOT ? 0 : slot + 1;
+    const int pslot = slot == 0 ? NSLOT - 1 : slot - 1;
+#pragma unroll
+    for (int kk = 0; kk < 2; kk++) {
+#pragma unroll
+      for (int q = 0; q < 8; q++) {
+#pragma unroll
+        for (int bb = 0; bb < 4; bb++) {
+          const int a = q >> 1, b = (q & 1) * 4 + bb;
+          const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+          acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[kk][b], fx[kk][a], (s == 0 && kk == 0) ? zero : acc[a][b], 0, 0, 0);
+        }
+        // fragments of the next k step: (s,1) from this slot, or (s+1,0) from the next slot, which the mid-slice
+        // barrier has made visible
+        if (q < 6) {
+          const int rslot = kk == 0 ? slot : nslot;
+          if (q < 2) {
+            read_x(kk ^ 1, rslot, kk ^ 1, 2 * q);
+            read_x(kk ^ 1, rslot, kk ^ 1, 2 * q + 1);
+          } else {
+            read_w(kk ^ 1, rslot, kk ^ 1, 2 * (q - 2));
+            read_w(kk ^ 1, rslot, kk ^ 1, 2 * (q - 2) + 1);
+          }
+        }
+        // operand prefetch, one load per group: slice s+3 goes into the slot slice s vacates at the mid-slice
+        // barrier (first half of its loads in the second k step of s, second half in the first k step of s+1)
+        if (kk == 1 && q < NDMA / 2) dma_one(s + 3, slot, q);
+        if (kk == 0 && q < NDMA / 2 && s > 0) dma_one(s + 2, pslot, NDMA / 2 + q);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (kk == 0) {
+        // mid-slice: slice s+1 has landed (this wave's share) and every fragment read of slice s is done
+        asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NDMA) : "memory");
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+      }
+    }
+    slot = nslot;
+  }
+
+#pragma unroll
+  for (int a = 0; a < TM; a++) {
+    const int m = m0 + (wm * TM + a) * 16 + frow;
+#pragma unroll
+    for (int b = 0; b < TN; b++) {
+      const int n = n0 + (wn * TN + b) * 16 + fchk * 4;
+      if (m >= p.M || n >= p.N) continue;
+      float bv[4] = {0.f, 0.f, 0.f, 0.f};
+      if (p.bias) {
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+          if (n + e < p.N) bv[e] = bf16_bits_to_f32(p.bias[n + e]);
+      }
+      const uint32_t lo = pack_bf16x2(acc[a][b][0] + bv[0], acc[a][b][1] + bv[1]);
+      const uint32_t hi = pack_bf16x2(acc[a][b][2] + bv[2], acc[a][b][3] + bv[3]);
+      uint16_t* dst = p.C + (int64_t)m * p.ldc + n;
+      if (p.vec_store && n + 3 < p.N) {
+        *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);
+      } else {
+        const uint16_t v[4] = {(uint16_t)(lo & 0xffff), (uint16_t)(lo >> 16), (uint16_t)(hi & 0xffff), (uint16_t)(hi >> 16)};
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+          if (n + e < p.N) dst[e] = v[e];
+      }
+    }
+  }
+}
+
+int gemm_single_acc_quad_launch(const QuadArgs& a, hipStream_t stream) {
+  using namespace quad;
+  constexpr size_t smem = (size_t)NSLOT * STAGE_BYTES;  // 144 KiB
+  const int64_t tiles = (int64_t)((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
+  if (tiles <= 0 || tiles > 0x7fffffff || a.K < BK || (a.K % BK) != 0) return TBIK_ERR_UNSUPPORTED;
+  if (a.ldx >= (1 << 22) || a.ldw >= (1 << 22)) return TBIK_ERR_UNSUPPORTED;  // 32-bit in-tile byte offsets
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_single_acc_quad_kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+  if (e != hipSuccess) return hip_code(e);
+  hipLaunchKernelGGL(gemm_single_acc_quad_kernel, dim3((unsigned)tiles), dim3(NT), smem, stream, a);
+  return hip_code(hipGetLastError());
+}
+
+}  // namespace tbik

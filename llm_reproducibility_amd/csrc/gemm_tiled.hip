@@ -341,6 +341,18 @@ int gemm_tree_wide_launch(const WideArgs& a, int leaf_k, int split, hipStream_t 
 int tree_combine_bias_dispatch(const void* const* parts, int nparts, void* out, int64_t numel, const void* bias, int N,
                                hipStream_t stream);
 
+// one-wave-per-SIMD single-accumulator kernel (gemm_single_acc_quad.hip)
+struct QuadArgs {
+  const uint16_t* X;
+  const uint16_t* W;
+  uint16_t* C;
+  const uint16_t* bias;
+  int64_t ldx, ldw, ldc;
+  int M, N, K;
+  int vec_store;
+};
+int gemm_single_acc_quad_launch(const QuadArgs& a, hipStream_t stream);
+
 // How one problem is run.  Small grids are filled by cutting K into `split` aligned subtrees (one grid.y slice
 // each) whose bf16 partials meet in the shard tree afterwards -- the same arithmetic as tensor-parallel shards, so
 // the bits do not change.  The wide kernel takes over once its 128x256 tiles (times the split) occupy the chip.
@@ -416,12 +428,12 @@ int gemm_dispatch(bool tree, const void* A, int64_t lda, const void* B, int64_t 
   a.k_shard = 0;
   a.c_shard = 0;
   if (!tree) {
-    // large problems whose K is a whole number of 256-wide spans take the wide pipeline (same MFMA chain per
-    // element, so the same bits as the tiled kernel)
+    // large problems whose K is a whole number of 64-wide slices take the one-wave-per-SIMD pipeline (same MFMA
+    // chain per element, so the same bits as the tiled kernel)
     const int64_t wide_tiles = (int64_t)((M + 127) / 128) * ((N + 255) / 256);
-    if (M > 64 && wide_tiles >= 128 && (K & 255) == 0) {
-      WideArgs w{a.X, a.W, a.C, a.bias, nullptr, a.ldx, a.ldw, a.ldc, M, N, K, K / 256, 1, 0, a.vec_store, 0, 0};
-      return gemm_tree_wide_launch(w, 0, 1, stream);
+    if (M > 64 && wide_tiles >= 128 && (K & 63) == 0 && lda < (1 << 22) && ldb_n < (1 << 22)) {
+      QuadArgs qa{a.X, a.W, a.C, a.bias, a.ldx, a.ldw, a.ldc, M, N, K, a.vec_store};
+      return gemm_single_acc_quad_launch(qa, stream);
     }
     return launch_by_m<4, 0, false>(a, 1, stream);
   }
