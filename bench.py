@@ -22,6 +22,11 @@ if ROOT not in sys.path:
 M_, K_, N_ = 2048, 12288, 4096
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+# HBM bytes one headline launch moves, from the hardware counters (not measured live: counters need the profiler).
+# FETCH_SIZE 259,879 KiB x 1.999 (a plain copy of 49,152 KiB reads 24,592) + WRITE_SIZE 133,120 KiB x 1.000;
+# profiles/gemm_tree_wide_headline_counters.txt holds the runs.  Algorithmic bytes are 167.8 MB: the rest is the
+# seven parked tree levels (written and read back once each) and one operand fetch per XCD-local L2.
+TRAFFIC_BYTES_PER_LAUNCH = 668.2e6
 
 
 def hip_time_ms(fn, steps, warmup):
@@ -41,25 +46,26 @@ def hip_time_ms(fn, steps, warmup):
     return s.elapsed_time(e) / steps, wall_ms / steps
 
 
-def cpu_baseline(rows=512, repeats=3):
-    """The CPU oracle (PyTorch restatement of the reference's tree order) on the first `rows` rows of the
-    same workload, all host threads, median of `repeats` after one warm-up."""
+def cpu_baseline(budget_s=12.0, max_runs=30):
+    """The CPU oracle (PyTorch restatement of the reference's tree order) on the whole headline workload, all host
+    threads: one warm-up, then repeated until about `budget_s` seconds of CPU work are spent; the median is reported."""
     import torch
     from oracle import tbik_oracle as O
-    X = O.silu_gated_bf16((rows, K_), 0)
+    X = O.silu_gated_bf16((M_, K_), 0)
     W = O.gaussian_bf16((N_, K_), 0.02, 1)
     Wt = W.t()
-    O.matmul_tree(X[:64], Wt)
-    ts = []
-    for _ in range(repeats):
+    O.matmul_tree(X[:256], Wt)
+    ts, spent = [], 0.0
+    while spent < budget_s and len(ts) < max_runs:
         t0 = time.perf_counter()
         O.matmul_tree(X, Wt)
         ts.append(time.perf_counter() - t0)
+        spent += ts[-1]
     t = statistics.median(ts)
-    return {"value": round(2.0 * rows * N_ * K_ / t / 1e12, 4), "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+    return {"value": round(2.0 * M_ * N_ * K_ / t / 1e12, 4), "unit": "TFLOP/s", "cores": torch.get_num_threads(),
             "kind": "port",
-            "sample": f"oracle matmul_tree on the first {rows} of {M_} rows of the same X and W "
-                      f"(median of {repeats}, {t:.2f} s each)"}
+            "sample": f"oracle matmul_tree on the full X[{M_},{K_}] and W[{N_},{K_}] of the headline workload, "
+                      f"{len(ts)} runs in {spent:.1f} s, median {t:.2f} s each"}
 
 
 def table(steps, warmup):
@@ -108,6 +114,11 @@ def table(steps, warmup):
         x = torch.randn((r, 4096), device=dev)
         ms, _ = hip_time_ms(lambda: bio.mean_dim(x, -1), steps, warmup)
         rows.append((f"mean rows={r} n=4096", ms * 1e3, 0.0, r * 4096 * 4 / ms / 1e6))
+    from llm_reproducibility_amd import ops
+    for r in (1, 256, 4096):
+        x = torch.randn((r, 2 * 12288), device=dev).to(torch.bfloat16)
+        ms, _ = hip_time_ms(lambda: ops.bi_silu_mul_bf16(x), steps, warmup)
+        rows.append((f"silu_mul rows={r} inter=12288 (6 B/elem)", ms * 1e3, 0.0, r * 12288 * 6 / ms / 1e6))
     print(f"{'case':52s} {'us':>10s} {'TFLOP/s':>9s} {'%MFMA':>6s} {'GB/s':>9s} {'%HBM':>6s}", file=sys.stderr)
     for name, us, tf, gbs in rows:
         print(f"{name:52s} {us:10.1f} {tf:9.1f} {100 * tf / PEAK_BF16_TFLOPS:6.1f} {gbs:9.1f} {100 * gbs / PEAK_HBM_GBS:6.1f}",
@@ -121,6 +132,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--table", action="store_true", help="also print the per-shape table to stderr")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run 5 plain device copies of X (50,331,648 B read + as many written each) so that a "
+                         "counter run can scale FETCH_SIZE / WRITE_SIZE by what a copy of known size reads")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -143,6 +157,13 @@ def main():
     assert torch.equal(tree_combine(parts), C), "TP=4 result differs from TP=1"
     del parts
 
+    if args.calibrate_copy:
+        Y = torch.empty_like(X)
+        for _ in range(5):
+            Y.copy_(X)
+        torch.cuda.synchronize()
+        del Y
+
     ms, wall_ms = hip_time_ms(step, args.steps, args.warmup)
     flops = 2.0 * M_ * N_ * K_
     algo_bytes = 2.0 * (M_ * K_ + K_ * N_ + M_ * N_)
@@ -157,7 +178,7 @@ def main():
         "pct_bf16_mfma_peak": round(100 * tflops / PEAK_BF16_TFLOPS, 2),
         "algorithmic_GBps": round(algo_bytes / (ms * 1e-3) / 1e9, 1),
         "roofline": {"bound": "mfma", "achieved": round(tflops, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(tflops / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "frac": round(tflops / PEAK_BF16_TFLOPS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH,
                      "kernel_avg_us": round(ms * 1e3, 2)},
     }
     if not args.no_cpu_baseline:

@@ -169,6 +169,19 @@ int bi_attention_bf16(const void* q, const void* k_cache, const void* vt_cache, 
                       int batch, int max_q_len, int q_heads, int kv_heads, int head_dim, int max_len,
                       float scale, tbik_stream_t stream);
 
+/*
+ * Gated activation in front of the row-split down projection:
+ *   out[r, i] = bf16( bf16(silu(gate_up[r, i])) * gate_up[r, inter + i] ),  i < inter,  silu in fp32.
+ * gate_up [rows, >= 2*inter] with row stride ld_in, out [rows, inter] with row stride ld_out (elements);
+ * inter, ld_in, ld_out multiples of 8, 16-byte aligned pointers.  Elementwise (batch invariant).
+ * Replaces: the unfused SiluAndMul that produces the input of the patched RowParallelLinear forward
+ *           (down_proj), src/patch/patch_tp_invariant.py:10-48; model wiring simple_rl.py:320-338.
+ */
+int bi_silu_mul_bf16(const void* gate_up, int64_t ld_in,
+                     void* out, int64_t ld_out,
+                     int64_t rows, int inter,
+                     tbik_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

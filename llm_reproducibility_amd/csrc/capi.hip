@@ -17,11 +17,13 @@ int attention_dispatch(const void* q, const void* k_cache, const void* vt_cache,
                        const int* q_len, const int* ctx_len, int batch, int max_q_len, int q_heads, int kv_heads,
                        int head_dim, int max_len, float scale, hipStream_t stream);
 int mean_dispatch(const void* x, void* out, int64_t outer, int64_t n, int64_t inner, int dtype_code, hipStream_t stream);
+int silu_mul_dispatch(const void* gate_up, int64_t ld_in, void* out, int64_t ld_out, int64_t rows, int inter,
+                      hipStream_t stream);
 }  // namespace tbik
 
 extern "C" {
 
-int tbik_abi_version(void) { return 3; }
+int tbik_abi_version(void) { return 4; }
 
 const char* tbik_error_string(int code) {
   switch (code) {
@@ -90,6 +92,11 @@ int bi_attention_bf16(const void* q, const void* k_cache, const void* vt_cache, 
                       int head_dim, int max_len, float scale, tbik_stream_t stream) {
   return tbik::attention_dispatch(q, k_cache, vt_cache, out, q_start, q_len, ctx_len, batch, max_q_len, q_heads, kv_heads,
                                   head_dim, max_len, scale, static_cast<hipStream_t>(stream));
+}
+
+int bi_silu_mul_bf16(const void* gate_up, int64_t ld_in, void* out, int64_t ld_out, int64_t rows, int inter,
+                     tbik_stream_t stream) {
+  return tbik::silu_mul_dispatch(gate_up, ld_in, out, ld_out, rows, inter, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

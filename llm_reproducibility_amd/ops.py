@@ -309,3 +309,36 @@ def bi_attention_bf16(q: torch.Tensor, k_cache: torch.Tensor, vt_cache: torch.Te
 @_bi_attention_bf16_op.register_fake
 def _(q, k_cache, vt_cache, q_start, q_len, ctx_len, max_q_len, scale):
     return torch.empty_like(q)
+
+
+# --------------------------------------------------------------------------------------------
+# gated activation in front of down_proj
+# --------------------------------------------------------------------------------------------
+def _bi_silu_mul_bf16_impl(gate_up: torch.Tensor) -> torch.Tensor:
+    _require_gpu(gate_up)
+    if gate_up.dtype != torch.bfloat16:
+        raise NotImplementedError(f"bi_silu_mul_bf16: unsupported dtype {gate_up.dtype}")
+    two_i = gate_up.shape[-1]
+    if two_i % 16 != 0:
+        raise ValueError(f"bi_silu_mul_bf16: last dimension {two_i} must be a multiple of 16")
+    inter = two_i // 2
+    g2, ld = _rows16(gate_up.reshape(-1, two_i))
+    out = torch.empty((g2.shape[0], inter), device=gate_up.device, dtype=torch.bfloat16)
+    rc = _lib.lib().bi_silu_mul_bf16(g2.data_ptr(), ld, out.data_ptr(), out.stride(0), g2.shape[0], inter, _stream(gate_up))
+    _lib.check(rc, "bi_silu_mul_bf16")
+    return out.reshape(*gate_up.shape[:-1], inter)
+
+
+_bi_silu_mul_bf16_op = torch.library.custom_op("tbik::bi_silu_mul_bf16", _bi_silu_mul_bf16_impl, mutates_args=(), device_types="cuda")
+
+
+def bi_silu_mul_bf16(gate_up: torch.Tensor) -> torch.Tensor:
+    """act = silu(gate_up[..., :I]) * gate_up[..., I:] (I = half the last dimension), fused, bf16."""
+    if torch.compiler.is_compiling():
+        return _bi_silu_mul_bf16_op(gate_up)
+    return _bi_silu_mul_bf16_impl(gate_up)
+
+
+@_bi_silu_mul_bf16_op.register_fake
+def _(gate_up):
+    return gate_up.new_empty((*gate_up.shape[:-1], gate_up.shape[-1] // 2))

@@ -32,6 +32,9 @@ Pin status (what checks each function independently of its own formula; see test
   (integer-valued inputs), and to 1 bf16 ulp otherwise.  PARITY UNPINNED beyond that.
 * `rmsnorm`: PARITY UNPINNED against the reference (the arithmetic lives in vllm==0.11.0, absent);
   pinned to the textbook formula in float64 and to closed-form cases.
+* `silu_mul`: PARITY UNPINNED against the reference (vLLM's SiluAndMul is absent); pinned to the
+  library routine `torch.nn.functional.silu` (bit-equal on bf16 inputs up to 1 ulp of the device exp),
+  to closed forms (silu(0) = 0, silu(x) -> x for large x) and to a float64 evaluation.
 * `log_softmax`, `mean_lastdim`: pinned to float64 library routines and closed-form cases; the
   reference's in-block reduction order (Triton `tl.sum`) is backend defined, so tolerance only.
 """
@@ -236,6 +239,18 @@ def rmsnorm(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float,
     if weight is not None:
         y = y * weight
     return y if residual is None else (y, new_residual)
+
+
+def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
+    """act = silu(gate) * up for gate_up = [gate | up] on the last dimension, the way an unfused
+    `F.silu(gate) * up` on bf16 tensors rounds: silu in fp32 rounded to the input dtype, then the product
+    rounded again.  This is the producer of down_proj's input (the patched RowParallelLinear forward,
+    src/patch/patch_tp_invariant.py:10-48); the activation itself lives in vLLM (not in the reference tree).
+    """
+    inter = gate_up.shape[-1] // 2
+    g, u = gate_up[..., :inter].float(), gate_up[..., inter:]
+    s = (g / (1.0 + torch.exp(-g))).to(gate_up.dtype)
+    return s * u
 
 
 # --------------------------------------------------------------------------------------------

@@ -127,6 +127,28 @@ def test_single_accumulator_mm_large_and_small_kernels_agree_bitwise(dev):
     assert torch.equal(bio.matmul_persistent(ai.to(dev), wi.to(dev).t()).cpu(), O.matmul_single_acc(ai, wi.t()))
 
 
+def test_silu_mul_parity_and_batch_invariance(dev):
+    from llm_reproducibility_amd import ops
+    g = torch.Generator().manual_seed(11)
+    gu = (torch.randn((300, 2 * 12288), generator=g) * 2).to(torch.bfloat16)
+    want = O.silu_mul(gu)
+    got = ops.bi_silu_mul_bf16(gu.to(dev))
+    assert got.shape == want.shape
+    assert O.bf16_ulp_distance(got.cpu(), want).max().item() <= 1   # device exp vs host exp: at most one rounding flip
+    for rows in (1, 7, 256):
+        assert torch.equal(ops.bi_silu_mul_bf16(gu[:rows].to(dev)), got[:rows])
+    # a strided view (row stride larger than the row) and a 3-D input
+    wide = torch.zeros((16, 2 * 256 + 64), dtype=torch.bfloat16)
+    wide[:, :512] = gu[:16, :512]
+    assert torch.equal(ops.bi_silu_mul_bf16(wide.to(dev)[:, :512]).cpu(), ops.bi_silu_mul_bf16(gu[:16, :512].contiguous().to(dev)).cpu())
+    assert ops.bi_silu_mul_bf16(gu[:12, :64].reshape(3, 4, 64).to(dev)).shape == (3, 4, 32)
+    # exact cases: silu(0) * u = 0, silu(40) = 40
+    z = torch.zeros((1, 16), dtype=torch.bfloat16)
+    z[0, 1] = 40.0
+    z[0, 8:] = 2.0
+    assert ops.bi_silu_mul_bf16(z.to(dev)).cpu().tolist() == [[0.0, 80.0, 0, 0, 0, 0, 0, 0]]
+
+
 def test_aten_overrides_route_to_the_hip_kernels(dev):
     a = O.gaussian_bf16((20, 512), 1.0, 0).to(dev)
     w = O.gaussian_bf16((64, 512), 0.1, 1).to(dev)

@@ -58,6 +58,8 @@ def test_host_argument_checks_fire_before_any_launch():
     assert L.bi_log_softmax_workspace_bytes(7, 151936) == 7 * 38 * 8
     assert L.bi_rmsnorm_bf16(p16, 12, None, 0, None, p16, 12, None, 0, 1, 12, 1e-6, None) == _lib.TBIK_ERR_ALIGNMENT
     assert L.bi_mean_dim(p16, p16, 1, 4, 1, 7, None) == _lib.TBIK_ERR_UNSUPPORTED
+    assert L.bi_silu_mul_bf16(p16, 24, p16, 12, 1, 12, None) == _lib.TBIK_ERR_ALIGNMENT
+    assert L.bi_silu_mul_bf16(p16, 16, p16, 16, 1, 16, None) == _lib.TBIK_ERR_INVALID   # ld_in < 2 * inter
     with pytest.raises(_lib.TbikError):
         _lib.check(_lib.TBIK_ERR_ALIGNMENT, "x")
 

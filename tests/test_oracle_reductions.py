@@ -73,3 +73,21 @@ def test_single_accumulator_matmul_is_one_rounding_of_the_fp32_product():
     b = O.gaussian_bf16((320, 24), 0.1, 7)
     bias = O.gaussian_bf16((24,), 1.0, 8)
     assert torch.equal(O.matmul_single_acc(a, b, bias), (a.float() @ b.float() + bias.float()).to(torch.bfloat16))
+
+
+def test_silu_mul_matches_library_float64_and_closed_forms():
+    g = torch.Generator().manual_seed(5)
+    gu = (torch.randn((33, 512), generator=g) * 3).to(torch.bfloat16)
+    got = O.silu_mul(gu)
+    assert got.shape == (33, 256) and got.dtype == torch.bfloat16
+    # library routine on the same bf16 tensors (two roundings: silu, then the product)
+    lib = torch.nn.functional.silu(gu[:, :256]) * gu[:, 256:]
+    assert O.bf16_ulp_distance(got, lib).max().item() <= 1
+    # float64 evaluation with the two roundings applied explicitly
+    g64 = gu[:, :256].double()
+    s = (g64 / (1 + torch.exp(-g64))).to(torch.bfloat16)
+    want = (s.double() * gu[:, 256:].double()).to(torch.bfloat16)
+    assert O.bf16_ulp_distance(got, want).max().item() <= 1
+    # closed forms: silu(0) = 0; silu(x) = x once exp(-x) underflows against 1; silu(-large) = -0 * ... = 0
+    gu = torch.tensor([[0.0, 40.0, -100.0, 2.0, 2.0, 2.0]], dtype=torch.bfloat16)
+    assert O.silu_mul(gu).tolist() == [[0.0, 80.0, -0.0]]
