@@ -69,7 +69,9 @@ __device__ __forceinline__ void dma16(uint32_t lds_addr, uint32_t voff, const vo
 
 // 16-byte-per-lane store to (wave-uniform base) + voff, scalar-base addressing: no per-lane 64-bit pointer.
 __device__ __forceinline__ void store16_sbase(void* base, uint32_t voff, u32x4 v) {
-  asm volatile("global_store_dwordx4 %0, %1, %2" : : "v"(voff), "v"(v), "s"(base) : "memory");
+  // the wait states keep the next instruction from overwriting the data registers while the store still reads
+  // them (a hazard the compiler handles for its own stores, but cannot see inside an asm statement)
+  asm volatile("global_store_dwordx4 %0, %1, %2\n\ts_nop 1" : : "v"(voff), "v"(v), "s"(base) : "memory");
 }
 
 // TREE = false: the same pipeline with ONE fp32 accumulator run over all of K (the batch-invariant mm); T counts
@@ -141,6 +143,8 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
 
   f32x4 acc[TM][TN];
   uint32_t t[NREG];    // packed leaf waiting to be merged (leaf j while leaf j+1 is computed)
+#pragma unroll
+  for (int r = 0; r < NREG; r++) t[r] = 0;
   uint32_t s0[NREG];   // level 0 running sum
   uint32_t sb0[NREG];  // binary level 0
   int c0 = 0;          // leaves absorbed at level 0 in the current group
@@ -193,7 +197,13 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
   };
   auto merge_quarter = [&](auto kind_c, int q) __attribute__((always_inline)) {
     constexpr int KIND = decltype(kind_c)::value;
-    if (KIND == K_NONE) return;
+    if (KIND == K_NONE) {
+      if (TREE) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) s0[8 * q + e] = t[8 * q + e];
+      }
+      return;
+    }
     u32x4 pf[2];
     if (KIND == K_P2 && LS != 4) {
       pf[0] = *ws_ptr(RL, 2 * q);
@@ -227,6 +237,15 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
   issue_slice(0, 0);
   issue_slice(min(1, nstages - 1), 1);
 
+  // rows of the pending buffer that are merged before the last slice of a leaf (quarter q = MFMA row q)
+  constexpr int EARLY_ROWS = (LS - 1) * (4 / LS);
+  auto pack_row = [&](int a) __attribute__((always_inline)) {
+#pragma unroll
+    for (int b = 0; b < TN; b++) {
+      t[(a * TN + b) * 2] = pack_bf16x2(acc[a][b][0], acc[a][b][1]);
+      t[(a * TN + b) * 2 + 1] = pack_bf16x2(acc[a][b][2], acc[a][b][3]);
+    }
+  };
   // One leaf: LS slices of MFMAs, with the pending leaf merged a quarter (LS=4) or a half (LS=2) per slice.
   auto leaf_body = [&](auto kind_c, int j) __attribute__((always_inline)) {
 #pragma unroll
@@ -260,6 +279,10 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
             const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
             acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[b], fx[a], (i == 0 && kk == 0 && (TREE || j == 0)) ? zero : acc[a][b], 0, 0, 0);
           }
+          // The finished leaf is rounded to bf16 (into the pending buffer) one MFMA row behind the row that
+          // completes it, so the rounding never waits for the MFMA pipeline; rows whose pending registers are
+          // merged only at the end of this slice follow after that merge.
+          if (TREE && i == LS - 1 && kk == 1 && a >= 1 && a - 1 < EARLY_ROWS) pack_row(a - 1);
           const int d = kk * TM + a;  // 0..7: loads 0..5 go out after MFMA rows 0..5
           if (d < NDMA) {
             __builtin_amdgcn_sched_barrier(0);
@@ -270,6 +293,10 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
       }
 #pragma unroll
       for (int q = i * (4 / LS); q < (i + 1) * (4 / LS); q++) merge_quarter(kind_c, q);
+      if (TREE && i == LS - 1) {
+#pragma unroll
+        for (int a = EARLY_ROWS; a < TM; a++) pack_row(a);
+      }
       slot = slot + 1 == NSLOT ? 0 : slot + 1;
     }
   };
@@ -288,50 +315,24 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
       default: leaf_body(std::integral_constant<int, K_P2>{}, j); break;
     }
     if (j == p.T - 1) break;  // the last leaf is packed and merged below
-    // the finished leaf: round once to bf16 (the accumulator is free again) and decide how it merges
+    // the finished leaf sits in the pending buffer; decide how it merges
     if (c0 == 0 && p.flb > 1) {
-      // first leaf of a group: it simply becomes the running sum
-#pragma unroll
-      for (int a = 0; a < TM; a++)
-#pragma unroll
-        for (int b = 0; b < TN; b++) {
-          s0[(a * TN + b) * 2] = pack_bf16x2(acc[a][b][0], acc[a][b][1]);
-          s0[(a * TN + b) * 2 + 1] = pack_bf16x2(acc[a][b][2], acc[a][b][3]);
-        }
-      kind = K_NONE;
+      kind = K_NONE;  // first leaf of a group: it simply becomes the running sum
       c0 = 1;
+    } else if (c0 + 1 < p.flb) {
+      kind = K_ADD;
+      c0++;
     } else {
-#pragma unroll
-      for (int a = 0; a < TM; a++)
-#pragma unroll
-        for (int b = 0; b < TN; b++) {
-          t[(a * TN + b) * 2] = pack_bf16x2(acc[a][b][0], acc[a][b][1]);
-          t[(a * TN + b) * 2 + 1] = pack_bf16x2(acc[a][b][2], acc[a][b][3]);
-        }
-      if (c0 + 1 < p.flb) {
-        kind = K_ADD;
-        c0++;
-      } else {
-        // the group completes: carry through the binary counter (this is never the last group here)
-        const int pops = __builtin_ctz(~g);
-        kind = pops == 0 ? K_P0 : (pops == 1 ? K_P1 : K_P2);
-        g_pending = g;
-        g++;
-        c0 = 0;
-      }
+      // the group completes: carry through the binary counter (this is never the last group here)
+      const int pops = __builtin_ctz(~g);
+      kind = pops == 0 ? K_P0 : (pops == 1 ? K_P1 : K_P2);
+      g_pending = g;
+      g++;
+      c0 = 0;
     }
   }
 
   // ---- the last leaf: every level carries, t ends as the root
-  if (TREE) {
-#pragma unroll
-    for (int a = 0; a < TM; a++)
-#pragma unroll
-      for (int b = 0; b < TN; b++) {
-        t[(a * TN + b) * 2] = pack_bf16x2(acc[a][b][0], acc[a][b][1]);
-        t[(a * TN + b) * 2 + 1] = pack_bf16x2(acc[a][b][2], acc[a][b][3]);
-      }
-  }
   if (TREE && c0 != 0) {
 #pragma unroll
     for (int r = 0; r < NREG; r++) t[r] = add_bf16x2(s0[r], t[r]);
