@@ -23,10 +23,10 @@ M_, K_, N_ = 2048, 12288, 4096
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # HBM bytes one headline launch moves, from the hardware counters (not measured live: counters need the profiler).
-# FETCH_SIZE 259,879 KiB x 1.999 (a plain copy of 49,152 KiB reads 24,592) + WRITE_SIZE 133,120 KiB x 1.000;
+# FETCH_SIZE 256,867 KiB x 1.999 (a plain copy of 49,152 KiB reads 24,592) + WRITE_SIZE 131,072 KiB x 1.000;
 # profiles/gemm_tree_wide_headline_counters.txt holds the runs.  Algorithmic bytes are 167.8 MB: the rest is the
 # seven parked tree levels (written and read back once each) and one operand fetch per XCD-local L2.
-TRAFFIC_BYTES_PER_LAUNCH = 668.2e6
+TRAFFIC_BYTES_PER_LAUNCH = 659.9e6
 
 
 def hip_time_ms(fn, steps, warmup):
