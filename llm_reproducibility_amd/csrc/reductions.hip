@@ -188,12 +188,25 @@ __global__ __launch_bounds__(256) void lsm_partial_kernel(const LsmArgs a) {
 __global__ __launch_bounds__(256) void lsm_write_kernel(const LsmArgs a) {
   const int64_t row = blockIdx.x / a.segs;
   const int seg = blockIdx.x % a.segs;
-  const float* w = a.ws + (int64_t)row * a.segs * 2;
-  float gm = -INFINITY;
-  for (int s = 0; s < a.segs; s++) gm = fmaxf(gm, w[2 * s]);
-  float gl = 0.f;
-  for (int s = 0; s < a.segs; s++) gl += w[2 * s + 1] * expf(w[2 * s] - gm);
-  const float lg = logf(gl);
+  // The row's segment pairs are merged by the first wavefront only (lane l takes segments l, l+64, ... in
+  // ascending order, then a fixed butterfly): the order is a function of `segs` alone, and the other 192
+  // threads do not repeat the work.
+  __shared__ float stat[2];
+  if (threadIdx.x < 64) {
+    const float* w = a.ws + (int64_t)row * a.segs * 2;
+    float lm = -INFINITY;
+    for (int s = threadIdx.x; s < a.segs; s += 64) lm = fmaxf(lm, w[2 * s]);
+    const float gmax = wave_max(lm);
+    float ls = 0.f;
+    for (int s = threadIdx.x; s < a.segs; s += 64) ls += w[2 * s + 1] * expf(w[2 * s] - gmax);
+    const float gsum = wave_sum(ls);
+    if (threadIdx.x == 0) {
+      stat[0] = gmax;
+      stat[1] = logf(gsum);
+    }
+  }
+  __syncthreads();
+  const float gm = stat[0], lg = stat[1];
   const float* xr = a.x + row * a.ldx;
   float* orow = a.out + row * a.ldo;
   float v[4][4];
