@@ -371,9 +371,21 @@ static bool make_plan(int M, int N, int K, int leaf_k, Plan* pl) {
   const int64_t wide_tiles = (int64_t)((M + 127) / 128) * ((N + 255) / 256);
   int split = 1;
   bool wide = false;
-  if (M > 64) {
-    while (wide_tiles * split < 192 && split < max_split) split *= 2;
-    wide = wide_tiles * split >= 128;
+  if (M >= 64) {
+    // Estimated time of the wide kernel for each legal split: work-group rounds on 256 CUs times the K extent of
+    // one shard, plus the shard-combine pass over (split + 1) [M,N] arrays.  Constants are measured on MI355X
+    // (17 ns per k per round; 5 TB/s and 4 us for the combine).
+    double best = 0;
+    for (int sp = 1; sp <= max_split; sp *= 2) {
+      const double rounds = (double)((wide_tiles * sp + 255) / 256);
+      double t = rounds * ((double)K / sp) * 0.0173;
+      if (sp > 1) t += 4.0 + (double)(sp + 1) * M * N * 2.0 / 5.0e6;
+      if (sp == 1 || t < best) {
+        best = t;
+        split = sp;
+      }
+    }
+    wide = wide_tiles * split >= 64;
   }
   if (!wide) {
     const int bm = M <= 16 ? 16 : (M <= 64 ? 64 : 128), bn = M <= 16 ? 64 : 128;
