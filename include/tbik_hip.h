@@ -170,6 +170,29 @@ int bi_attention_bf16(const void* q, const void* k_cache, const void* vt_cache, 
                       float scale, tbik_stream_t stream);
 
 /*
+ * fp16 counterparts of tbik_gemm_bf16 / tbik_gemm_workspace_bytes / tbik_tree_combine_bf16 / bi_gemm_bf16: same
+ * arguments and contract, elements are IEEE half, leaves are chains of v_mfma_f32_16x16x32_f16 rounded once to
+ * fp16, every tree node is one fp16 addition (round to nearest even).
+ * Replaces: the float16 branch of the reference's dtype-keyed configuration,
+ *           src/tbik/tree_based_matmul.py:206-238 and src/bio/batch_invariant_ops.py:138-170.
+ */
+size_t tbik_gemm_f16_workspace_bytes(int M, int N, int K, int leaf_k);
+int tbik_gemm_f16(const void* A, int64_t lda,
+                  const void* B, int64_t ldb_k, int64_t ldb_n,
+                  void* C, int64_t ldc,
+                  int M, int N, int K, int leaf_k,
+                  const void* bias_or_null,
+                  void* workspace, size_t workspace_bytes,
+                  tbik_stream_t stream);
+int tbik_tree_combine_f16(const void* const* parts, int nparts, void* out, int64_t numel, tbik_stream_t stream);
+int bi_gemm_f16(const void* A, int64_t lda,
+                const void* B, int64_t ldb_k, int64_t ldb_n,
+                void* C, int64_t ldc,
+                int M, int N, int K,
+                const void* bias_or_null,
+                tbik_stream_t stream);
+
+/*
  * Gated activation in front of the row-split down projection:
  *   out[r, i] = bf16( bf16(silu(gate_up[r, i])) * gate_up[r, inter + i] ),  i < inter,  silu in fp32.
  * gate_up [rows, >= 2*inter] with row stride ld_in, out [rows, inter] with row stride ld_out (elements);

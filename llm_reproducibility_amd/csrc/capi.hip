@@ -3,11 +3,11 @@
 #include "common.h"
 
 namespace tbik {
-int gemm_dispatch(bool tree, const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C,
+int gemm_dispatch(bool tree, bool f16, const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C,
                   int64_t ldc, int M, int N, int K, int leaf_k, const void* bias, void* ws, size_t ws_bytes,
                   hipStream_t stream);
-size_t gemm_workspace_bytes(int M, int N, int K, int leaf_k);
-int tree_combine_dispatch(const void* const* parts, int nparts, void* out, int64_t numel, hipStream_t stream);
+size_t gemm_workspace_bytes(int M, int N, int K, int leaf_k, bool f16);
+int tree_combine_dispatch(const void* const* parts, int nparts, void* out, int64_t numel, bool f16, hipStream_t stream);
 int rmsnorm_dispatch(const void* x, int64_t ldx, const void* res, int64_t ldr, const void* w, void* out, int64_t ldo,
                      void* res_out, int64_t ldro, int64_t rows, int hidden, float eps, hipStream_t stream);
 size_t lsm_workspace_bytes(int64_t rows, int64_t cols);
@@ -23,7 +23,7 @@ int silu_mul_dispatch(const void* gate_up, int64_t ld_in, void* out, int64_t ld_
 
 extern "C" {
 
-int tbik_abi_version(void) { return 4; }
+int tbik_abi_version(void) { return 5; }
 
 const char* tbik_error_string(int code) {
   switch (code) {
@@ -49,22 +49,40 @@ int tbik_tree_params(int K, int leaf_k, int* T, int* flb, int* level_k) {
   return TBIK_OK;
 }
 
-size_t tbik_gemm_workspace_bytes(int M, int N, int K, int leaf_k) { return tbik::gemm_workspace_bytes(M, N, K, leaf_k); }
+size_t tbik_gemm_workspace_bytes(int M, int N, int K, int leaf_k) { return tbik::gemm_workspace_bytes(M, N, K, leaf_k, false); }
+size_t tbik_gemm_f16_workspace_bytes(int M, int N, int K, int leaf_k) { return tbik::gemm_workspace_bytes(M, N, K, leaf_k, true); }
 
 int tbik_gemm_bf16(const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C, int64_t ldc, int M,
                    int N, int K, int leaf_k, const void* bias_or_null, void* workspace, size_t workspace_bytes,
                    tbik_stream_t stream) {
-  return tbik::gemm_dispatch(true, A, lda, B, ldb_k, ldb_n, C, ldc, M, N, K, leaf_k, bias_or_null, workspace,
+  return tbik::gemm_dispatch(true, false, A, lda, B, ldb_k, ldb_n, C, ldc, M, N, K, leaf_k, bias_or_null, workspace,
                              workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
 int tbik_tree_combine_bf16(const void* const* parts, int nparts, void* out, int64_t numel, tbik_stream_t stream) {
-  return tbik::tree_combine_dispatch(parts, nparts, out, numel, static_cast<hipStream_t>(stream));
+  return tbik::tree_combine_dispatch(parts, nparts, out, numel, false, static_cast<hipStream_t>(stream));
+}
+
+int tbik_gemm_f16(const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C, int64_t ldc, int M,
+                  int N, int K, int leaf_k, const void* bias_or_null, void* workspace, size_t workspace_bytes,
+                  tbik_stream_t stream) {
+  return tbik::gemm_dispatch(true, true, A, lda, B, ldb_k, ldb_n, C, ldc, M, N, K, leaf_k, bias_or_null, workspace,
+                             workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+int tbik_tree_combine_f16(const void* const* parts, int nparts, void* out, int64_t numel, tbik_stream_t stream) {
+  return tbik::tree_combine_dispatch(parts, nparts, out, numel, true, static_cast<hipStream_t>(stream));
+}
+
+int bi_gemm_f16(const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C, int64_t ldc, int M,
+                int N, int K, const void* bias_or_null, tbik_stream_t stream) {
+  return tbik::gemm_dispatch(false, true, A, lda, B, ldb_k, ldb_n, C, ldc, M, N, K, 0, bias_or_null, nullptr, 0,
+                             static_cast<hipStream_t>(stream));
 }
 
 int bi_gemm_bf16(const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C, int64_t ldc, int M,
                  int N, int K, const void* bias_or_null, tbik_stream_t stream) {
-  return tbik::gemm_dispatch(false, A, lda, B, ldb_k, ldb_n, C, ldc, M, N, K, 0, bias_or_null, nullptr, 0,
+  return tbik::gemm_dispatch(false, false, A, lda, B, ldb_k, ldb_n, C, ldc, M, N, K, 0, bias_or_null, nullptr, 0,
                              static_cast<hipStream_t>(stream));
 }
 

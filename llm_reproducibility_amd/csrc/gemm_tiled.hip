@@ -42,8 +42,9 @@ constexpr int BK = 64;  // K elements per LDS stage (8 chunks of 16 bytes per ro
 // The XOR spreads the 16 rows an MFMA fragment read touches over all banks.
 __device__ __forceinline__ int lds_off(int r, int c) { return r * BK + ((c ^ (r & 7)) << 3); }
 
-template <int WAVES_M, int WAVES_N, int TM, int TN, int LS, int LBMAX, bool TREE>
+template <int WAVES_M, int WAVES_N, int TM, int TN, int LS, int LBMAX, bool TREE, bool F16>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmArgs p) {
+  using Num = Num16<F16>;
   constexpr int NT = WAVES_M * WAVES_N * 64;
   constexpr int BM = WAVES_M * TM * 16;
   constexpr int BN = WAVES_N * TN * 16;
@@ -181,7 +182,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
 #pragma unroll
             for (int b = 0; b < TN; b++) {
               const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-              acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[b], fx[a], fresh ? zero : acc[a][b], 0, 0, 0);
+              acc[a][b] = Num::mfma(fw[b], fx[a], fresh ? zero : acc[a][b]);
             }
         }
         store_stage((s + 1) & 1);
@@ -194,16 +195,16 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
       for (int a = 0; a < TM; a++)
 #pragma unroll
         for (int b = 0; b < TN; b++) {
-          t[a][b][0] = pack_bf16x2(acc[a][b][0], acc[a][b][1]);
-          t[a][b][1] = pack_bf16x2(acc[a][b][2], acc[a][b][3]);
+          t[a][b][0] = Num::pack(acc[a][b][0], acc[a][b][1]);
+          t[a][b][1] = Num::pack(acc[a][b][2], acc[a][b][3]);
         }
       if (c0 != 0) {
 #pragma unroll
         for (int a = 0; a < TM; a++)
 #pragma unroll
           for (int b = 0; b < TN; b++) {
-            t[a][b][0] = add_bf16x2(s0[a][b][0], t[a][b][0]);
-            t[a][b][1] = add_bf16x2(s0[a][b][1], t[a][b][1]);
+            t[a][b][0] = Num::add(s0[a][b][0], t[a][b][0]);
+            t[a][b][1] = Num::add(s0[a][b][1], t[a][b][1]);
           }
       }
       c0++;
@@ -218,8 +219,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
               for (int a = 0; a < TM; a++)
 #pragma unroll
                 for (int b = 0; b < TN; b++) {
-                  t[a][b][0] = add_bf16x2(sb[l][a][b][0], t[a][b][0]);
-                  t[a][b][1] = add_bf16x2(sb[l][a][b][1], t[a][b][1]);
+                  t[a][b][0] = Num::add(sb[l][a][b][0], t[a][b][0]);
+                  t[a][b][1] = Num::add(sb[l][a][b][1], t[a][b][1]);
                 }
             } else {
 #pragma unroll
@@ -259,18 +260,18 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
       if (p.bias) {
 #pragma unroll
         for (int e = 0; e < 4; e++)
-          if (n + e < p.N) bv[e] = bf16_bits_to_f32(p.bias[n + e]);
+          if (n + e < p.N) bv[e] = Num::to_f32(p.bias[n + e]);
       }
       if (TREE) {
         lo = t[a][b][0];
         hi = t[a][b][1];
         if (p.bias) {
-          lo = add_bf16x2(lo, pack_bf16x2(bv[0], bv[1]));
-          hi = add_bf16x2(hi, pack_bf16x2(bv[2], bv[3]));
+          lo = Num::add(lo, Num::pack(bv[0], bv[1]));
+          hi = Num::add(hi, Num::pack(bv[2], bv[3]));
         }
       } else {
-        lo = pack_bf16x2(acc[a][b][0] + bv[0], acc[a][b][1] + bv[1]);
-        hi = pack_bf16x2(acc[a][b][2] + bv[2], acc[a][b][3] + bv[3]);
+        lo = Num::pack(acc[a][b][0] + bv[0], acc[a][b][1] + bv[1]);
+        hi = Num::pack(acc[a][b][2] + bv[2], acc[a][b][3] + bv[3]);
       }
       uint16_t* dst = Cs + (int64_t)m * p.ldc + n;
       if (p.vec_store && n + 3 < p.N) {
@@ -288,13 +289,13 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
 // ------------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------------
-template <int WAVES_M, int WAVES_N, int TM, int TN, int LS, int LBMAX, bool TREE>
+template <int WAVES_M, int WAVES_N, int TM, int TN, int LS, int LBMAX, bool TREE, bool F16>
 static int launch(const GemmArgs& a, int split, hipStream_t stream) {
   constexpr int NT = WAVES_M * WAVES_N * 64;
   constexpr int BM = WAVES_M * TM * 16;
   constexpr int BN = WAVES_N * TN * 16;
   constexpr size_t smem = (size_t)2 * (BM + BN) * BK * sizeof(uint16_t);
-  auto kern = gemm_kernel<WAVES_M, WAVES_N, TM, TN, LS, LBMAX, TREE>;
+  auto kern = gemm_kernel<WAVES_M, WAVES_N, TM, TN, LS, LBMAX, TREE, F16>;
   if (smem > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
@@ -306,18 +307,18 @@ static int launch(const GemmArgs& a, int split, hipStream_t stream) {
   return hip_code(hipGetLastError());
 }
 
-template <int LS, int LBMAX, bool TREE>
+template <int LS, int LBMAX, bool TREE, bool F16>
 static int launch_by_m(const GemmArgs& a, int split, hipStream_t stream) {
-  if (a.M <= 16) return launch<1, 4, 1, 1, LS, LBMAX, TREE>(a, split, stream);
-  if (a.M <= 64) return launch<1, 4, 4, 2, LS, LBMAX, TREE>(a, split, stream);
-  return launch<2, 2, 4, 4, LS, LBMAX, TREE>(a, split, stream);
+  if (a.M <= 16) return launch<1, 4, 1, 1, LS, LBMAX, TREE, F16>(a, split, stream);
+  if (a.M <= 64) return launch<1, 4, 4, 2, LS, LBMAX, TREE, F16>(a, split, stream);
+  return launch<2, 2, 4, 4, LS, LBMAX, TREE, F16>(a, split, stream);
 }
 
-template <int LS>
+template <int LS, bool F16>
 static int launch_tree(const GemmArgs& a, int split, hipStream_t stream) {
-  if (a.lb <= 2) return launch_by_m<LS, 2, true>(a, split, stream);
-  if (a.lb <= 4) return launch_by_m<LS, 4, true>(a, split, stream);
-  if (a.lb <= 6) return launch_by_m<LS, 6, true>(a, split, stream);
+  if (a.lb <= 2) return launch_by_m<LS, 2, true, F16>(a, split, stream);
+  if (a.lb <= 4) return launch_by_m<LS, 4, true, F16>(a, split, stream);
+  if (a.lb <= 6) return launch_by_m<LS, 6, true, F16>(a, split, stream);
   return TBIK_ERR_UNSUPPORTED;
 }
 
@@ -339,7 +340,7 @@ struct WideArgs {
 size_t wide_workspace_bytes(int M, int N, int lb, int split);
 int gemm_tree_wide_launch(const WideArgs& a, int leaf_k, int split, hipStream_t stream);
 int tree_combine_bias_dispatch(const void* const* parts, int nparts, void* out, int64_t numel, const void* bias, int N,
-                               hipStream_t stream);
+                               bool f16, hipStream_t stream);
 
 // one-wave-per-SIMD single-accumulator kernel (gemm_single_acc_quad.hip)
 struct QuadArgs {
@@ -363,7 +364,7 @@ struct Plan {
   size_t partial_bytes, parked_bytes;
 };
 
-static bool make_plan(int M, int N, int K, int leaf_k, Plan* pl) {
+static bool make_plan(int M, int N, int K, int leaf_k, bool f16, Plan* pl) {
   int T, flb, level_k;
   if (M <= 0 || N <= 0 || tbik_tree_params(K, leaf_k, &T, &flb, &level_k) != TBIK_OK) return false;
   const int lb = level_k - 1;
@@ -371,7 +372,7 @@ static bool make_plan(int M, int N, int K, int leaf_k, Plan* pl) {
   const int64_t wide_tiles = (int64_t)((M + 127) / 128) * ((N + 255) / 256);
   int split = 1;
   bool wide = false;
-  if (M >= 64) {
+  if (M >= 64 && !f16) {  // the wide kernel exists for bf16 only
     // Estimated time of the wide kernel for each legal split: work-group rounds on 256 CUs times the K extent of
     // one shard, plus the shard-combine pass over (split + 1) [M,N] arrays.  Constants are measured on MI355X
     // (17 ns per k per round; 5 TB/s and 4 us for the combine).
@@ -406,13 +407,13 @@ static bool make_plan(int M, int N, int K, int leaf_k, Plan* pl) {
   return true;
 }
 
-size_t gemm_workspace_bytes(int M, int N, int K, int leaf_k) {
+size_t gemm_workspace_bytes(int M, int N, int K, int leaf_k, bool f16) {
   Plan pl;
-  if (!make_plan(M, N, K, leaf_k, &pl)) return 0;
+  if (!make_plan(M, N, K, leaf_k, f16, &pl)) return 0;
   return pl.partial_bytes + pl.parked_bytes;
 }
 
-int gemm_dispatch(bool tree, const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C,
+int gemm_dispatch(bool tree, bool f16, const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C,
                   int64_t ldc, int M, int N, int K, int leaf_k, const void* bias, void* ws, size_t ws_bytes,
                   hipStream_t stream) {
   if (!A || !B || !C || M < 0 || N < 0 || K <= 0) return TBIK_ERR_INVALID;
@@ -443,16 +444,16 @@ int gemm_dispatch(bool tree, const void* A, int64_t lda, const void* B, int64_t 
     // large problems whose K is a whole number of 64-wide slices take the one-wave-per-SIMD pipeline (same MFMA
     // chain per element, so the same bits as the tiled kernel)
     const int64_t wide_tiles = (int64_t)((M + 127) / 128) * ((N + 255) / 256);
-    if (M > 64 && wide_tiles >= 128 && (K & 63) == 0 && lda < (1 << 22) && ldb_n < (1 << 22)) {
+    if (!f16 && M > 64 && wide_tiles >= 128 && (K & 63) == 0 && lda < (1 << 22) && ldb_n < (1 << 22)) {
       QuadArgs qa{a.X, a.W, a.C, a.bias, a.ldx, a.ldw, a.ldc, M, N, K, a.vec_store};
       return gemm_single_acc_quad_launch(qa, stream);
     }
-    return launch_by_m<4, 0, false>(a, 1, stream);
+    return f16 ? launch_by_m<4, 0, false, true>(a, 1, stream) : launch_by_m<4, 0, false, false>(a, 1, stream);
   }
 
   if (leaf_k != 256 && leaf_k != 128) return TBIK_ERR_UNSUPPORTED;
   Plan pl;
-  if (!make_plan(M, N, K, leaf_k, &pl)) return TBIK_ERR_INVALID;
+  if (!make_plan(M, N, K, leaf_k, f16, &pl)) return TBIK_ERR_INVALID;
   const size_t need = pl.partial_bytes + pl.parked_bytes;
   if (need > 0 && (!ws || ws_bytes < need || !aligned16(ws))) return TBIK_ERR_WORKSPACE;
   uint8_t* wsb = static_cast<uint8_t*>(ws);
@@ -475,16 +476,17 @@ int gemm_dispatch(bool tree, const void* A, int64_t lda, const void* B, int64_t 
                a.T, a.flb, a.lb, a.vec_store, a.k_shard, a.c_shard};
     rc = gemm_tree_wide_launch(w, leaf_k, pl.split, stream);
   } else {
-    rc = leaf_k == 256 ? launch_tree<4>(a, pl.split, stream) : launch_tree<2>(a, pl.split, stream);
+    if (f16) rc = leaf_k == 256 ? launch_tree<4, true>(a, pl.split, stream) : launch_tree<2, true>(a, pl.split, stream);
+    else rc = leaf_k == 256 ? launch_tree<4, false>(a, pl.split, stream) : launch_tree<2, false>(a, pl.split, stream);
   }
   if (rc != TBIK_OK || pl.split == 1) return rc;
   const void* parts[8];
   for (int i = 0; i < pl.split; i++) parts[i] = wsb + (size_t)i * M * N * sizeof(uint16_t);
-  if (ldc == N) return tree_combine_bias_dispatch(parts, pl.split, C, (int64_t)M * N, bias, N, stream);
+  if (ldc == N) return tree_combine_bias_dispatch(parts, pl.split, C, (int64_t)M * N, bias, N, f16, stream);
   for (int m = 0; m < M && rc == TBIK_OK; m++) {  // strided C (rare): row by row
     const void* rp[8];
     for (int i = 0; i < pl.split; i++) rp[i] = static_cast<const uint8_t*>(parts[i]) + (size_t)m * N * sizeof(uint16_t);
-    rc = tree_combine_bias_dispatch(rp, pl.split, static_cast<uint16_t*>(C) + (int64_t)m * ldc, N, bias, N, stream);
+    rc = tree_combine_bias_dispatch(rp, pl.split, static_cast<uint16_t*>(C) + (int64_t)m * ldc, N, bias, N, f16, stream);
   }
   return rc;
 }

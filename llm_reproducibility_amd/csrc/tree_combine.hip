@@ -1,5 +1,5 @@
-// Shard combine: out[i] = adjacent-pair binary tree over up to 8 bf16 partials, every node rounded to
-// bf16.  This is the arithmetic of the reference's cross-GPU tree all-reduce
+// Shard combine: out[i] = adjacent-pair binary tree over up to 8 bf16 (or fp16) partials, every node rounded to
+// the element type.  This is the arithmetic of the reference's cross-GPU tree all-reduce
 // (src/tbik/tree_based_all_reduce.py:32-37; packed_tree_reduce,
 // mini_allreduce/tbik_kernel/csrc/allreduce/custom_all_reduce.cuh:203-234) applied to partials that
 // already sit in one GPU's memory.  HBM bound: (nparts + 1) * numel * 2 bytes.
@@ -15,7 +15,7 @@ struct CombineArgs {
   int ncols;
 };
 
-template <int NP>
+template <int NP, bool F16>
 __device__ __forceinline__ uint32_t tree_node(const uint32_t (&v)[8]) {
   uint32_t w[8];
 #pragma unroll
@@ -23,12 +23,12 @@ __device__ __forceinline__ uint32_t tree_node(const uint32_t (&v)[8]) {
 #pragma unroll
   for (int step = 1; step < NP; step <<= 1)
 #pragma unroll
-    for (int left = 0; left < NP; left += 2 * step) w[left] = add_bf16x2(w[left], w[left + step]);
+    for (int left = 0; left < NP; left += 2 * step) w[left] = Num16<F16>::add(w[left], w[left + step]);
   return w[0];
 }
 
 // One thread per 16-byte pack (8 bf16); grid-stride so any numel fits one launch.
-template <int NP>
+template <int NP, bool F16>
 __global__ __launch_bounds__(256) void combine_vec_kernel(const CombineArgs a, int64_t npacks) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < npacks; i += stride) {
@@ -39,61 +39,61 @@ __global__ __launch_bounds__(256) void combine_vec_kernel(const CombineArgs a, i
     uint32_t v[8];
 #pragma unroll
     for (int p = 0; p < NP; p++) v[p] = in[p].x;
-    o.x = tree_node<NP>(v);
+    o.x = tree_node<NP, F16>(v);
 #pragma unroll
     for (int p = 0; p < NP; p++) v[p] = in[p].y;
-    o.y = tree_node<NP>(v);
+    o.y = tree_node<NP, F16>(v);
 #pragma unroll
     for (int p = 0; p < NP; p++) v[p] = in[p].z;
-    o.z = tree_node<NP>(v);
+    o.z = tree_node<NP, F16>(v);
 #pragma unroll
     for (int p = 0; p < NP; p++) v[p] = in[p].w;
-    o.w = tree_node<NP>(v);
+    o.w = tree_node<NP, F16>(v);
     if (a.bias) {  // ncols % 8 == 0 on this path: the pack stays inside one row
       const uint4 bq = *reinterpret_cast<const uint4*>(a.bias + (i * 8) % a.ncols);
-      o.x = add_bf16x2(o.x, bq.x);
-      o.y = add_bf16x2(o.y, bq.y);
-      o.z = add_bf16x2(o.z, bq.z);
-      o.w = add_bf16x2(o.w, bq.w);
+      o.x = Num16<F16>::add(o.x, bq.x);
+      o.y = Num16<F16>::add(o.y, bq.y);
+      o.z = Num16<F16>::add(o.z, bq.z);
+      o.w = Num16<F16>::add(o.w, bq.w);
     }
     reinterpret_cast<uint4*>(a.out)[i] = o;
   }
 }
 
 // Scalar path for the tail and for buffers that are not 16-byte aligned.
-template <int NP>
+template <int NP, bool F16>
 __global__ __launch_bounds__(256) void combine_scalar_kernel(const CombineArgs a, int64_t begin) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = begin + (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < a.numel; i += stride) {
     uint32_t v[8];
 #pragma unroll
     for (int p = 0; p < NP; p++) v[p] = a.parts[p][i];
-    uint32_t r = tree_node<NP>(v);
-    if (a.bias) r = add_bf16x2(r, a.bias[i % a.ncols]);
+    uint32_t r = tree_node<NP, F16>(v);
+    if (a.bias) r = Num16<F16>::add(r, a.bias[i % a.ncols]);
     a.out[i] = (uint16_t)(r & 0xffffu);
   }
 }
 
-template <int NP>
+template <int NP, bool F16>
 static int launch_combine(const CombineArgs& a, bool vec_ok, hipStream_t stream) {
   const int64_t npacks = vec_ok ? a.numel / 8 : 0;
   if (npacks > 0) {
     const int64_t blocks = (npacks + 255) / 256;
     const unsigned grid = (unsigned)(blocks < 8192 ? blocks : 8192);
-    hipLaunchKernelGGL(combine_vec_kernel<NP>, dim3(grid), dim3(256), 0, stream, a, npacks);
+    hipLaunchKernelGGL((combine_vec_kernel<NP, F16>), dim3(grid), dim3(256), 0, stream, a, npacks);
   }
   const int64_t begin = npacks * 8;
   if (begin < a.numel) {
     const int64_t rest = a.numel - begin;
     const int64_t blocks = (rest + 255) / 256;
     const unsigned grid = (unsigned)(blocks < 8192 ? blocks : 8192);
-    hipLaunchKernelGGL(combine_scalar_kernel<NP>, dim3(grid), dim3(256), 0, stream, a, begin);
+    hipLaunchKernelGGL((combine_scalar_kernel<NP, F16>), dim3(grid), dim3(256), 0, stream, a, begin);
   }
   return hip_code(hipGetLastError());
 }
 
 int tree_combine_bias_dispatch(const void* const* parts, int nparts, void* out, int64_t numel, const void* bias, int N,
-                               hipStream_t stream) {
+                               bool f16, hipStream_t stream) {
   if (!parts || !out || numel < 0 || (bias && N <= 0)) return TBIK_ERR_INVALID;
   if (nparts != 1 && nparts != 2 && nparts != 4 && nparts != 8) return TBIK_ERR_INVALID;
   if (numel == 0) return TBIK_OK;
@@ -112,16 +112,24 @@ int tree_combine_bias_dispatch(const void* const* parts, int nparts, void* out, 
   a.bias = static_cast<const uint16_t*>(bias);
   a.ncols = N;
   if (bias) vec_ok = vec_ok && (N & 7) == 0 && (reinterpret_cast<uintptr_t>(bias) & 15) == 0;
+  if (f16) {
+    switch (nparts) {
+      case 1: return launch_combine<1, true>(a, vec_ok, stream);
+      case 2: return launch_combine<2, true>(a, vec_ok, stream);
+      case 4: return launch_combine<4, true>(a, vec_ok, stream);
+      default: return launch_combine<8, true>(a, vec_ok, stream);
+    }
+  }
   switch (nparts) {
-    case 1: return launch_combine<1>(a, vec_ok, stream);
-    case 2: return launch_combine<2>(a, vec_ok, stream);
-    case 4: return launch_combine<4>(a, vec_ok, stream);
-    default: return launch_combine<8>(a, vec_ok, stream);
+    case 1: return launch_combine<1, false>(a, vec_ok, stream);
+    case 2: return launch_combine<2, false>(a, vec_ok, stream);
+    case 4: return launch_combine<4, false>(a, vec_ok, stream);
+    default: return launch_combine<8, false>(a, vec_ok, stream);
   }
 }
 
-int tree_combine_dispatch(const void* const* parts, int nparts, void* out, int64_t numel, hipStream_t stream) {
-  return tree_combine_bias_dispatch(parts, nparts, out, numel, nullptr, 0, stream);
+int tree_combine_dispatch(const void* const* parts, int nparts, void* out, int64_t numel, bool f16, hipStream_t stream) {
+  return tree_combine_bias_dispatch(parts, nparts, out, numel, nullptr, 0, f16, stream);
 }
 
 }  // namespace tbik

@@ -34,6 +34,14 @@ def _aligned16(t: torch.Tensor) -> bool:
     return t.data_ptr() % 16 == 0
 
 
+def _is_f16(*tensors) -> bool:
+    """True for float16 operands, False for bfloat16; every operand must have the same one of the two."""
+    dts = {t.dtype for t in tensors if t is not None}
+    if len(dts) != 1 or not dts <= {torch.bfloat16, torch.float16}:
+        raise NotImplementedError(f"16-bit GEMM kernels take all-bfloat16 or all-float16 operands, got {sorted(map(str, dts))}")
+    return dts == {torch.float16}
+
+
 def _rows16(t: torch.Tensor):
     """(tensor, leading dimension) with a contiguous last dim and 16-byte aligned rows; copies if needed."""
     ok = t.stride(1) == 1 and _aligned16(t) and t.shape[1] % 8 == 0
@@ -63,11 +71,12 @@ def _gemm_tree_bf16_impl(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.
     a, lda = _rows16(A)
     w, ldw = _weight_nk(B)
     b = None if bias is None else bias.contiguous()
-    C = torch.empty((M, N), device=A.device, dtype=torch.bfloat16)
+    f16 = _is_f16(A, B, bias)
+    C = torch.empty((M, N), device=A.device, dtype=A.dtype)
     L = _lib.lib()
-    ws_bytes = L.tbik_gemm_workspace_bytes(M, N, K, leaf_k)
+    ws_bytes = (L.tbik_gemm_f16_workspace_bytes if f16 else L.tbik_gemm_workspace_bytes)(M, N, K, leaf_k)
     ws = torch.empty(ws_bytes, device=A.device, dtype=torch.uint8) if ws_bytes else None
-    rc = L.tbik_gemm_bf16(a.data_ptr(), lda, w.data_ptr(), 1, ldw, C.data_ptr(), C.stride(0),
+    rc = (L.tbik_gemm_f16 if f16 else L.tbik_gemm_bf16)(a.data_ptr(), lda, w.data_ptr(), 1, ldw, C.data_ptr(), C.stride(0),
                           M, N, K, leaf_k, None if b is None else b.data_ptr(),
                           None if ws is None else ws.data_ptr(), ws_bytes, _stream(A))
     _lib.check(rc, "tbik_gemm_bf16")
@@ -93,7 +102,8 @@ def _tree_combine_bf16_impl(parts: List[torch.Tensor]) -> torch.Tensor:
     ps = [p.contiguous() for p in parts]
     out = torch.empty_like(ps[0])
     arr = (ctypes.c_void_p * len(ps))(*[p.data_ptr() for p in ps])
-    rc = _lib.lib().tbik_tree_combine_bf16(arr, len(ps), out.data_ptr(), out.numel(), _stream(out))
+    L = _lib.lib()
+    rc = (L.tbik_tree_combine_f16 if _is_f16(*ps) else L.tbik_tree_combine_bf16)(arr, len(ps), out.data_ptr(), out.numel(), _stream(out))
     _lib.check(rc, "tbik_tree_combine_bf16")
     return out
 
@@ -128,8 +138,9 @@ def _bi_gemm_bf16_impl(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.Te
     a, lda = _rows16(A)
     w, ldw = _weight_nk(B)
     b = None if bias is None else bias.contiguous()
-    C = torch.empty((M, N), device=A.device, dtype=torch.bfloat16)
-    rc = _lib.lib().bi_gemm_bf16(a.data_ptr(), lda, w.data_ptr(), 1, ldw, C.data_ptr(), C.stride(0),
+    C = torch.empty((M, N), device=A.device, dtype=A.dtype)
+    L = _lib.lib()
+    rc = (L.bi_gemm_f16 if _is_f16(A, B, bias) else L.bi_gemm_bf16)(a.data_ptr(), lda, w.data_ptr(), 1, ldw, C.data_ptr(), C.stride(0),
                                  M, N, K, None if b is None else b.data_ptr(), _stream(A))
     _lib.check(rc, "bi_gemm_bf16")
     return C

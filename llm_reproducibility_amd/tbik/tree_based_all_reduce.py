@@ -24,8 +24,8 @@ def tree_combine(parts: Sequence[torch.Tensor]) -> torch.Tensor:
     if n > 8:
         # wider worlds: reduce groups of 8 first; adjacent-pair trees compose
         return tree_combine([tree_combine(parts[i:i + 8]) for i in range(0, n, 8)])
-    if any(p.dtype != torch.bfloat16 for p in parts):
-        raise NotImplementedError("tree_combine is implemented for bfloat16 partials")
+    if parts[0].dtype not in (torch.bfloat16, torch.float16) or any(p.dtype != parts[0].dtype for p in parts):
+        raise NotImplementedError("tree_combine is implemented for bfloat16 or float16 partials of one dtype")
     if any(p.shape != parts[0].shape for p in parts):
         raise ValueError("partials must have the same shape")
     return ops.tree_combine_bf16(list(parts))

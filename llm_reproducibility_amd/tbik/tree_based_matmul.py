@@ -39,8 +39,8 @@ def matmul_tp_persistent(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.
     """
     assert A.shape[-1] == B.shape[-2], "Dim doesn't match"
     assert A.dim() == 2 and B.dim() == 2, "2-D operands only"
-    if A.dtype != torch.bfloat16 or B.dtype != torch.bfloat16:
-        raise NotImplementedError("the gfx950 tree matmul is implemented for bfloat16 operands")
+    if A.dtype != B.dtype or A.dtype not in (torch.bfloat16, torch.float16):
+        raise NotImplementedError("the gfx950 tree matmul is implemented for bfloat16 and float16 operands of one dtype")
     K = A.shape[1]
     assert K % leaf_k == 0, f"K={K} must be a multiple of the leaf size {leaf_k}"
     if bias is not None:

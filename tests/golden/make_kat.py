@@ -17,8 +17,9 @@ import numpy as np
 HERE = os.path.dirname(os.path.abspath(__file__))
 
 
-def rn_bf16(x: Fraction) -> Fraction:
-    """Round a rational to the nearest bf16 value (8 significant bits), ties to even; no overflow handling."""
+def rn(x: Fraction, sig_bits: int) -> Fraction:
+    """Round a rational to `sig_bits` significant bits (8: bf16, 11: fp16), ties to even; no overflow or
+    subnormal handling (the callers check the range)."""
     if x == 0:
         return Fraction(0)
     s = -1 if x < 0 else 1
@@ -28,7 +29,7 @@ def rn_bf16(x: Fraction) -> Fraction:
         e += 1
     while a < 2 ** e:
         e -= 1
-    ulp = Fraction(2) ** (e - 7)
+    ulp = Fraction(2) ** (e - (sig_bits - 1))
     q = a / ulp
     fl = q.numerator // q.denominator
     rem = q - fl
@@ -45,7 +46,7 @@ def tree_params(T):
     return flb, lev
 
 
-def brute_force(A, B, leaf):
+def brute_force(A, B, leaf, sig_bits):
     M, K = A.shape
     N = B.shape[1]
     T = K // leaf
@@ -53,16 +54,16 @@ def brute_force(A, B, leaf):
     out = np.zeros((M, N), dtype=np.float64)
     for m in range(M):
         for n in range(N):
-            leaves = [rn_bf16(Fraction(int(np.dot(A[m, j * leaf:(j + 1) * leaf], B[j * leaf:(j + 1) * leaf, n]))))
+            leaves = [rn(Fraction(int(np.dot(A[m, j * leaf:(j + 1) * leaf], B[j * leaf:(j + 1) * leaf, n]))), sig_bits)
                       for j in range(T)]
             groups = []
             for g in range(0, T, flb):
                 s = leaves[g]
                 for j in range(1, flb):
-                    s = rn_bf16(s + leaves[g + j])
+                    s = rn(s + leaves[g + j], sig_bits)
                 groups.append(s)
             while len(groups) > 1:
-                groups = [rn_bf16(groups[i] + groups[i + 1]) for i in range(0, len(groups), 2)]
+                groups = [rn(groups[i] + groups[i + 1], sig_bits) for i in range(0, len(groups), 2)]
             out[m, n] = float(groups[0])
     return out
 
@@ -73,6 +74,13 @@ def to_bf16_bits(x: np.ndarray) -> np.ndarray:
     u = f.view(np.uint32)
     assert np.all((u & 0xFFFF) == 0), "value not exact in bf16"
     return (u >> 16).astype(np.uint16)
+
+
+def to_f16_bits(x: np.ndarray) -> np.ndarray:
+    assert np.abs(x).max() < 65504, "fp16 overflow: outside what the brute force models"
+    h = x.astype(np.float16)
+    assert np.array_equal(h.astype(np.float64), x), "value not exact in fp16"
+    return h.view(np.uint16)
 
 
 CASES = [  # name, M, N, K, leaf, amax, bmax, seed
@@ -94,12 +102,15 @@ def main():
         rng = np.random.default_rng(seed)
         A = rng.integers(-amax, amax + 1, size=(M, K)).astype(np.int64)
         B = rng.integers(-bmax, bmax + 1, size=(K, N)).astype(np.int64)
-        C = brute_force(A, B, leaf)
+        C = brute_force(A, B, leaf, 8)
+        C16 = brute_force(A, B, leaf, 11)
         out[name + "_A"] = A.astype(np.int8)
         out[name + "_B"] = B.astype(np.int8)
         out[name + "_C"] = to_bf16_bits(C)
+        out[name + "_C16"] = to_f16_bits(C16)   # the same product with fp16 leaves and nodes
         out[name + "_leaf"] = np.array(leaf, dtype=np.int32)
-        print(name, "max |C| =", np.abs(C).max(), "rounded nodes matter:", bool(np.abs(C).max() > 256))
+        print(name, "max |C| =", np.abs(C).max(), "rounded nodes matter:", bool(np.abs(C).max() > 256),
+              "| fp16:", bool(np.abs(C16).max() > 2048), "differs from bf16:", bool((C != C16).any()))
     np.savez_compressed(os.path.join(HERE, "kat_tree_matmul.npz"), **out)
 
 

@@ -127,6 +127,24 @@ def test_single_accumulator_mm_large_and_small_kernels_agree_bitwise(dev):
     assert torch.equal(bio.matmul_persistent(ai.to(dev), wi.to(dev).t()).cpu(), O.matmul_single_acc(ai, wi.t()))
 
 
+def test_single_accumulator_mm_fp16(dev):
+    a = O.gaussian_bf16((300, 1000), 1.0, 0).to(torch.float16)
+    w = O.gaussian_bf16((200, 1000), 0.05, 1).to(torch.float16)
+    b = O.gaussian_bf16((200,), 1.0, 2).to(torch.float16)
+    got = bio.matmul_persistent(a.to(dev), w.to(dev).t(), bias=b.to(dev))
+    want = O.matmul_single_acc(a, w.t(), b)
+    assert got.dtype == torch.float16
+    d = (got.cpu().float() - want.float()).abs()
+    assert (d <= 2.0 ** -10 * want.float().abs().clamp_min(2.0 ** -6)).all()   # one fp16 ulp (fp32 order differs)
+    for rows in (1, 7, 64):
+        assert torch.equal(bio.matmul_persistent(a[:rows].to(dev), w.to(dev).t(), bias=b.to(dev)), got[:rows])
+    ai = O.integer_bf16((70, 512), -9, 9, 8).to(torch.float16)
+    wi = O.integer_bf16((96, 512), -7, 7, 9).to(torch.float16)
+    assert torch.equal(bio.matmul_persistent(ai.to(dev), wi.to(dev).t()).cpu(), O.matmul_single_acc(ai, wi.t()))
+    with bio.set_batch_invariant_mode(True):
+        assert torch.equal(torch.mm(ai.to(dev), wi.to(dev).t()).cpu(), O.matmul_single_acc(ai, wi.t()))
+
+
 def test_silu_mul_parity_and_batch_invariance(dev):
     from llm_reproducibility_amd import ops
     g = torch.Generator().manual_seed(11)

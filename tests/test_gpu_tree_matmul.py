@@ -165,3 +165,58 @@ def test_tree_combine_matches_oracle_bitwise(dev):
     flat = big.to(dev).reshape(-1)
     shifted = [flat[1 + i * 1001: 1 + i * 1001 + 999] for i in range(4)]
     assert_bitwise(tree_combine(shifted), O.tree_combine([s.cpu() for s in shifted]), "shifted views")
+
+
+# ---------------------------------------------------------------------------------------------
+# float16: the other 16-bit branch of the reference's dtype-keyed configuration
+# (src/tbik/tree_based_matmul.py:206-222): same tree, leaves and nodes rounded to fp16
+# ---------------------------------------------------------------------------------------------
+def f16_ulp_distance(a, b):
+    def ordered(t):
+        i = t.contiguous().view(torch.int16).to(torch.int32)
+        return torch.where(i < 0, -(i & 0x7FFF), i)
+    return (ordered(a) - ordered(b)).abs()
+
+
+def test_fp16_rational_known_answers(dev):
+    z = np.load(GOLDEN)
+    for n in sorted({k[:-2] for k in z.files if k.endswith("_A")}):
+        A = torch.from_numpy(z[n + "_A"].astype(np.float32)).to(torch.float16).to(dev)
+        B = torch.from_numpy(z[n + "_B"].astype(np.float32)).to(torch.float16).to(dev)
+        C = torch.from_numpy(z[n + "_C16"].view(np.int16).copy()).view(torch.float16)
+        leaf = int(z[n + "_leaf"])
+        print("fp16 case", n, tuple(A.shape), tuple(B.shape), leaf, flush=True)
+        got = matmul_tp_persistent(A, B, leaf_k=leaf)
+        assert got.dtype == torch.float16
+        assert_bitwise(got, C, n)
+        assert_bitwise(matmul_tp_persistent(A, B.t().contiguous().t(), leaf_k=leaf), C, n + " (weight.t())")
+
+
+@pytest.mark.parametrize("M,N,K,leaf", [(1, 64, 512, 256), (17, 200, 1536, 256), (70, 136, 2048, 256), (300, 520, 3072, 256),
+                                        (33, 72, 3200, 128)])
+def test_fp16_integer_inputs_match_oracle_bitwise(dev, M, N, K, leaf):
+    A = O.integer_bf16((M, K), -9, 9, 3).to(torch.float16)
+    W = O.integer_bf16((N, K), -7, 7, 4).to(torch.float16)
+    bias = O.integer_bf16((N,), -50, 50, 5).to(torch.float16)
+    print("fp16 ints", M, N, K, leaf, flush=True)
+    want = O.matmul_tree(A, W.t(), bias, leaf=leaf)
+    assert_bitwise(matmul_tp_persistent(A.to(dev), W.to(dev).t(), bias.to(dev), leaf_k=leaf), want, "vs oracle")
+
+
+def test_fp16_gaussian_tolerance_and_invariance(dev):
+    M, K, N = 2048, 4096, 4096
+    X = O.gaussian_bf16((M, K), 1.0, 0).to(torch.float16).to(dev)
+    W = O.gaussian_bf16((N, K), 0.02, 1).to(torch.float16).to(dev)
+    full = matmul_tp_persistent(X, W.t())
+    want = O.matmul_tree(X[:64].cpu(), W.cpu().t())
+    ulp = f16_ulp_distance(full[:64].cpu(), want)
+    diff = (full[:64].cpu().float() - want.float()).abs()
+    scale = want.float().abs().max().item()
+    bad = (ulp > 1) & (diff > 2.0 ** -11 * scale)   # <= 1 fp16 ulp, or 2^-11 of the output scale
+    assert not bad.any(), f"{int(bad.sum())} elements off, max ulp {int(ulp.max())}"
+    for p in (2, 4, 8):
+        assert_bitwise(sim_tp(X, W.t(), p, 256), full, f"fp16 TP={p}")
+    for m in (1, 16, 64, 300):
+        assert_bitwise(matmul_tp_persistent(X[:m], W.t()), full[:m], f"fp16 rows {m}")
+    parts = [O.gaussian_bf16((33, 257), 1.0, s).to(torch.float16) for s in range(4)]
+    assert_bitwise(tree_combine([q.to(dev) for q in parts]), O.tree_combine(parts), "fp16 tree_combine")

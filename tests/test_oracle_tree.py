@@ -109,6 +109,23 @@ def test_oracles_reproduce_rational_known_answers(case):
     assert torch.equal(c_oracle.matmul_tree(A, B, leaf=leaf).view(torch.int16), C.view(torch.int16))
 
 
+def _load_kat_f16():
+    z = np.load(GOLDEN)
+    for n in sorted({k[:-2] for k in z.files if k.endswith("_A")}):
+        A = torch.from_numpy(z[n + "_A"].astype(np.float32)).to(torch.float16)
+        B = torch.from_numpy(z[n + "_B"].astype(np.float32)).to(torch.float16)
+        C = torch.from_numpy(z[n + "_C16"].view(np.int16).copy()).view(torch.float16)
+        yield n, A, B, C, int(z[n + "_leaf"])
+
+
+@pytest.mark.parametrize("case", list(_load_kat_f16()), ids=lambda c: c[0])
+def test_oracle_reproduces_rational_known_answers_in_fp16(case):
+    # the float16 branch of the reference's dtype-keyed configuration (src/tbik/tree_based_matmul.py:206-222):
+    # same tree, leaves and nodes rounded to 11 significant bits
+    _, A, B, C, leaf = case
+    assert torch.equal(O.matmul_tree(A, B, leaf=leaf).view(torch.int16), C.view(torch.int16))
+
+
 def test_known_answers_discriminate_other_orders():
     # a sequential (left-to-right over all leaves) order or an fp32 tree must NOT reproduce the fixtures
     differs_seq = differs_f32 = 0
