@@ -193,6 +193,28 @@ int bi_gemm_f16(const void* A, int64_t lda,
                 tbik_stream_t stream);
 
 /*
+ * fp32 variants: C[M,N] = A[M,K] x B[K,N] (+ bias), all float.  tbik_gemm_f32 is tree-ordered with leaves of 128
+ * (leaf_k must be 128, K a multiple of it): a leaf is the fp32 sum of its products, every tree node one fp32
+ * addition; no workspace.  bi_gemm_f32 runs one fp32 accumulator over K (K a multiple of 16; callers pad with
+ * zeros).  Products are full-precision fp32 MFMAs in an order that depends on K only.  16-byte aligned A and B,
+ * leading dimensions multiples of 4, ldb_k == 1.
+ * Replaces: the float32 branch of the reference's dtype-keyed configurations,
+ *           src/tbik/tree_based_matmul.py:223-231 and src/bio/batch_invariant_ops.py:160-170.
+ */
+int tbik_gemm_f32(const void* A, int64_t lda,
+                  const void* B, int64_t ldb_k, int64_t ldb_n,
+                  void* C, int64_t ldc,
+                  int M, int N, int K, int leaf_k,
+                  const void* bias_or_null,
+                  tbik_stream_t stream);
+int bi_gemm_f32(const void* A, int64_t lda,
+                const void* B, int64_t ldb_k, int64_t ldb_n,
+                void* C, int64_t ldc,
+                int M, int N, int K,
+                const void* bias_or_null,
+                tbik_stream_t stream);
+
+/*
  * Gated activation in front of the row-split down projection:
  *   out[r, i] = bf16( bf16(silu(gate_up[r, i])) * gate_up[r, inter + i] ),  i < inter,  silu in fp32.
  * gate_up [rows, >= 2*inter] with row stride ld_in, out [rows, inter] with row stride ld_out (elements);

@@ -31,8 +31,8 @@ def matmul_persistent(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Ten
     assert a.shape[1] == b.shape[0], "Incompatible dimensions"
     assert a.dtype == b.dtype, "Incompatible dtypes"
     assert bias is None or bias.dim() == 1, "Currently assuming bias is 1D"
-    if a.dtype not in (torch.bfloat16, torch.float16):
-        raise NotImplementedError(f"batch-invariant mm on gfx950 is implemented for bfloat16 and float16, got {a.dtype}")
+    if a.dtype not in (torch.bfloat16, torch.float16, torch.float32):
+        raise NotImplementedError(f"batch-invariant mm on gfx950 takes bfloat16, float16 or float32, got {a.dtype}")
     if bias is not None and bias.dtype != a.dtype:
         bias = bias.to(a.dtype)
     return ops.bi_gemm_bf16(a, b, bias)

@@ -17,13 +17,15 @@ int attention_dispatch(const void* q, const void* k_cache, const void* vt_cache,
                        const int* q_len, const int* ctx_len, int batch, int max_q_len, int q_heads, int kv_heads,
                        int head_dim, int max_len, float scale, hipStream_t stream);
 int mean_dispatch(const void* x, void* out, int64_t outer, int64_t n, int64_t inner, int dtype_code, hipStream_t stream);
+int gemm_f32_dispatch(bool tree, const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C,
+                      int64_t ldc, int M, int N, int K, int leaf_k, const void* bias, hipStream_t stream);
 int silu_mul_dispatch(const void* gate_up, int64_t ld_in, void* out, int64_t ld_out, int64_t rows, int inter,
                       hipStream_t stream);
 }  // namespace tbik
 
 extern "C" {
 
-int tbik_abi_version(void) { return 5; }
+int tbik_abi_version(void) { return 6; }
 
 const char* tbik_error_string(int code) {
   switch (code) {
@@ -110,6 +112,18 @@ int bi_attention_bf16(const void* q, const void* k_cache, const void* vt_cache, 
                       int head_dim, int max_len, float scale, tbik_stream_t stream) {
   return tbik::attention_dispatch(q, k_cache, vt_cache, out, q_start, q_len, ctx_len, batch, max_q_len, q_heads, kv_heads,
                                   head_dim, max_len, scale, static_cast<hipStream_t>(stream));
+}
+
+int tbik_gemm_f32(const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C, int64_t ldc, int M,
+                  int N, int K, int leaf_k, const void* bias_or_null, tbik_stream_t stream) {
+  return tbik::gemm_f32_dispatch(true, A, lda, B, ldb_k, ldb_n, C, ldc, M, N, K, leaf_k, bias_or_null,
+                                 static_cast<hipStream_t>(stream));
+}
+
+int bi_gemm_f32(const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C, int64_t ldc, int M,
+                int N, int K, const void* bias_or_null, tbik_stream_t stream) {
+  return tbik::gemm_f32_dispatch(false, A, lda, B, ldb_k, ldb_n, C, ldc, M, N, K, 0, bias_or_null,
+                                 static_cast<hipStream_t>(stream));
 }
 
 int bi_silu_mul_bf16(const void* gate_up, int64_t ld_in, void* out, int64_t ld_out, int64_t rows, int inter,

@@ -42,6 +42,40 @@ def _is_f16(*tensors) -> bool:
     return dts == {torch.float16}
 
 
+def _rows_f32(t: torch.Tensor):
+    """fp32 operand with a contiguous last dim, 16-byte aligned rows (leading dimension a multiple of 4)."""
+    ok = t.stride(1) == 1 and _aligned16(t) and (t.shape[0] == 1 or (t.stride(0) >= t.shape[1] and t.stride(0) % 4 == 0))
+    if ok:
+        return t, (t.shape[1] if t.shape[0] == 1 else t.stride(0))
+    c = t.contiguous()
+    if not _aligned16(c) or c.shape[1] % 4 != 0:
+        c = torch.nn.functional.pad(c, (0, (-c.shape[1]) % 4))[:, : t.shape[1]] if c.shape[1] % 4 else c.clone()
+    return c, c.stride(0)
+
+
+def _gemm_f32(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.Tensor], leaf_k: int, tree: bool) -> torch.Tensor:
+    M, K = A.shape
+    N = B.shape[1]
+    if K % 16 != 0:  # only the single-accumulator form gets here: zero columns do not change a sequential sum
+        pad = (-K) % 16
+        A = torch.nn.functional.pad(A, (0, pad))
+        B = torch.nn.functional.pad(B, (0, 0, 0, pad))
+        K += pad
+    a, lda = _rows_f32(A)
+    w, ldw = _rows_f32(B.t())
+    b = None if bias is None else bias.contiguous()
+    C = torch.empty((M, N), device=A.device, dtype=torch.float32)
+    L = _lib.lib()
+    if tree:
+        rc = L.tbik_gemm_f32(a.data_ptr(), lda, w.data_ptr(), 1, ldw, C.data_ptr(), C.stride(0), M, N, K, leaf_k,
+                             None if b is None else b.data_ptr(), _stream(A))
+    else:
+        rc = L.bi_gemm_f32(a.data_ptr(), lda, w.data_ptr(), 1, ldw, C.data_ptr(), C.stride(0), M, N, K,
+                           None if b is None else b.data_ptr(), _stream(A))
+    _lib.check(rc, "tbik_gemm_f32" if tree else "bi_gemm_f32")
+    return C
+
+
 def _rows16(t: torch.Tensor):
     """(tensor, leading dimension) with a contiguous last dim and 16-byte aligned rows; copies if needed."""
     ok = t.stride(1) == 1 and _aligned16(t) and t.shape[1] % 8 == 0
@@ -66,6 +100,8 @@ def _weight_nk(B: torch.Tensor):
 # --------------------------------------------------------------------------------------------
 def _gemm_tree_bf16_impl(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.Tensor], leaf_k: int) -> torch.Tensor:
     _require_gpu(A, B, bias)
+    if A.dtype == torch.float32 and B.dtype == torch.float32 and (bias is None or bias.dtype == torch.float32):
+        return _gemm_f32(A, B, bias, leaf_k, True)
     M, K = A.shape
     N = B.shape[1]
     a, lda = _rows16(A)
@@ -127,6 +163,8 @@ def _(parts):
 # --------------------------------------------------------------------------------------------
 def _bi_gemm_bf16_impl(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
     _require_gpu(A, B, bias)
+    if A.dtype == torch.float32 and B.dtype == torch.float32 and (bias is None or bias.dtype == torch.float32):
+        return _gemm_f32(A, B, bias, 0, False)
     M, K = A.shape
     N = B.shape[1]
     if K % 8 != 0:

@@ -39,8 +39,10 @@ def matmul_tp_persistent(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.
     """
     assert A.shape[-1] == B.shape[-2], "Dim doesn't match"
     assert A.dim() == 2 and B.dim() == 2, "2-D operands only"
-    if A.dtype != B.dtype or A.dtype not in (torch.bfloat16, torch.float16):
-        raise NotImplementedError("the gfx950 tree matmul is implemented for bfloat16 and float16 operands of one dtype")
+    if A.dtype != B.dtype or A.dtype not in (torch.bfloat16, torch.float16, torch.float32):
+        raise NotImplementedError("the gfx950 tree matmul takes bfloat16, float16 or float32 operands of one dtype")
+    if A.dtype == torch.float32 and leaf_k == LEAF_K_DEFAULT:
+        leaf_k = 128  # the reference's float32 configuration cuts K into leaves of 128 (:223-231)
     K = A.shape[1]
     assert K % leaf_k == 0, f"K={K} must be a multiple of the leaf size {leaf_k}"
     if bias is not None:

@@ -96,8 +96,40 @@ CASES = [  # name, M, N, K, leaf, amax, bmax, seed
 ]
 
 
+# float32 (leaves of 128, 24 significant bits): ONE non-zero product per leaf, so every leaf is exact whatever the
+# order inside it, and products near 2^24 so that the nodes above do round: the result pins the tree order.
+CASES_F32 = [  # name, M, N, K, seed
+    ("f32_t6_flb3", 3, 4, 768, 11),
+    ("f32_t16_flb2", 3, 4, 2048, 12),
+    ("f32_t25_flb25", 2, 4, 3200, 13),
+    ("f32_t48_flb3", 2, 4, 6144, 14),
+]
+
+
 def main():
     out = {}
+    for name, M, N, K, seed in CASES_F32:
+        rng = np.random.default_rng(seed)
+        A = np.zeros((M, K), dtype=np.int64)
+        B = np.zeros((K, N), dtype=np.int64)
+        for j in range(K // 128):
+            pos = j * 128 + int(rng.integers(0, 128))
+            A[:, pos] = rng.integers(1, 4096, size=M) * rng.choice([-1, 1], size=M)
+            B[pos, :] = rng.integers(1, 4096, size=N) * rng.choice([-1, 1], size=N)
+        C = brute_force(A, B, 128, 24)
+        seq = np.zeros_like(C)
+        for m in range(M):
+            for n in range(N):
+                acc = Fraction(0)
+                for j in range(K // 128):
+                    acc = rn(acc + int(np.dot(A[m, j * 128:(j + 1) * 128], B[j * 128:(j + 1) * 128, n])), 24)
+                seq[m, n] = float(acc)
+        assert np.array_equal(C.astype(np.float32).astype(np.float64), C)
+        out[name + "_A32"] = A.astype(np.int16)
+        out[name + "_B32"] = B.astype(np.int16)
+        out[name + "_C32"] = C.astype(np.float32)
+        print(name, "max |C| =", np.abs(C).max(), "nodes round:", bool(np.abs(C).max() > 2 ** 24),
+              "differs from a sequential fp32 sum:", bool((C != seq).any()))
     for name, M, N, K, leaf, amax, bmax, seed in CASES:
         rng = np.random.default_rng(seed)
         A = rng.integers(-amax, amax + 1, size=(M, K)).astype(np.int64)

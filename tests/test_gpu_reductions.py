@@ -145,6 +145,24 @@ def test_single_accumulator_mm_fp16(dev):
         assert torch.equal(torch.mm(ai.to(dev), wi.to(dev).t()).cpu(), O.matmul_single_acc(ai, wi.t()))
 
 
+def test_single_accumulator_mm_fp32(dev):
+    g = torch.Generator().manual_seed(4)
+    a = torch.randn((130, 1001), generator=g)
+    w = torch.randn((77, 1001), generator=g) * 0.05
+    b = torch.randn((77,), generator=g)
+    got = bio.matmul_persistent(a.to(dev), w.to(dev).t(), bias=b.to(dev))
+    want = (a.double() @ w.double().t() + b.double()).float()
+    assert got.dtype == torch.float32 and got.shape == (130, 77)
+    assert torch.allclose(got.cpu(), want, rtol=1e-5, atol=1e-5 * want.abs().max().item())
+    for rows in (1, 7, 64):
+        assert torch.equal(bio.matmul_persistent(a[:rows].to(dev), w.to(dev).t(), bias=b.to(dev)), got[:rows])
+    ai = O.integer_bf16((70, 512), -9, 9, 8).float()
+    wi = O.integer_bf16((96, 512), -7, 7, 9).float()
+    with bio.set_batch_invariant_mode(True):
+        assert torch.equal(torch.mm(ai.to(dev), wi.to(dev).t()).cpu(), ai @ wi.t())
+        assert torch.equal(torch.addmm(b[:1].to(dev).expand(96), ai.to(dev), wi.to(dev).t()).cpu(), ai @ wi.t() + b[0])
+
+
 def test_silu_mul_parity_and_batch_invariance(dev):
     from llm_reproducibility_amd import ops
     g = torch.Generator().manual_seed(11)

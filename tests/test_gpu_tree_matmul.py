@@ -220,3 +220,33 @@ def test_fp16_gaussian_tolerance_and_invariance(dev):
         assert_bitwise(matmul_tp_persistent(X[:m], W.t()), full[:m], f"fp16 rows {m}")
     parts = [O.gaussian_bf16((33, 257), 1.0, s).to(torch.float16) for s in range(4)]
     assert_bitwise(tree_combine([q.to(dev) for q in parts]), O.tree_combine(parts), "fp16 tree_combine")
+
+
+# ---------------------------------------------------------------------------------------------
+# float32 (leaves of 128, src/tbik/tree_based_matmul.py:223-231)
+# ---------------------------------------------------------------------------------------------
+def test_fp32_rational_known_answers_and_invariance(dev):
+    z = np.load(GOLDEN)
+    for n in sorted({k[:-4] for k in z.files if k.endswith("_A32")}):
+        A = torch.from_numpy(z[n + "_A32"].astype(np.float32)).to(dev)
+        B = torch.from_numpy(z[n + "_B32"].astype(np.float32)).to(dev)
+        C = torch.from_numpy(z[n + "_C32"])
+        print("fp32 case", n, tuple(A.shape), tuple(B.shape), flush=True)
+        got = matmul_tp_persistent(A, B)   # leaf 128 is the float32 default
+        assert got.dtype == torch.float32
+        assert torch.equal(got.cpu().view(torch.int32), C.view(torch.int32)), n
+    M, K, N = 300, 2048, 520
+    g = torch.Generator().manual_seed(3)
+    X = torch.randn((M, K), generator=g).to(dev)
+    W = (torch.randn((N, K), generator=g) * 0.02).to(dev)
+    bias = torch.randn((N,), generator=g).to(dev)
+    full = matmul_tp_persistent(X, W.t(), bias)
+    want = O.matmul_tree(X.cpu(), W.cpu().t(), bias.cpu(), leaf=128)
+    assert torch.allclose(full.cpu(), want, rtol=2e-5, atol=2e-5 * want.abs().max().item())
+    nb = matmul_tp_persistent(X, W.t())
+    for p in (2, 4, 8):
+        ks = K // p
+        parts = [matmul_tp_persistent(X[:, r * ks:(r + 1) * ks], W[:, r * ks:(r + 1) * ks].t()) for r in range(p)]
+        assert torch.equal(tree_combine(parts), nb), f"fp32 TP={p}"
+    for m in (1, 17, 64):
+        assert torch.equal(matmul_tp_persistent(X[:m], W.t(), bias), full[:m]), f"fp32 rows {m}"

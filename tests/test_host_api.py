@@ -138,7 +138,7 @@ def test_operator_errors_match_the_reference_contract():
     with pytest.raises(AssertionError):
         matmul_tp_persistent(torch.zeros((4, 384), dtype=torch.bfloat16), torch.zeros((384, 8), dtype=torch.bfloat16))
     with pytest.raises(NotImplementedError):
-        matmul_tp_persistent(a.float(), torch.zeros((512, 8)))
+        matmul_tp_persistent(a.double(), torch.zeros((512, 8), dtype=torch.float64))
     with pytest.raises(ValueError):
         tree_combine([a, a, a])
     # there is no CPU path: CPU tensors fail loudly instead of falling back
@@ -146,6 +146,10 @@ def test_operator_errors_match_the_reference_contract():
         matmul_tp_persistent(a, torch.zeros((512, 8), dtype=torch.bfloat16))
     with pytest.raises((NotImplementedError, RuntimeError)):
         tree_combine([a, a])
+    with pytest.raises(RuntimeError):
+        tree_combine([a.float(), a.float()])
+    with pytest.raises(RuntimeError):
+        matmul_tp_persistent(a.float(), torch.zeros((512, 8)))
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

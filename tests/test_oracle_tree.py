@@ -126,6 +126,21 @@ def test_oracle_reproduces_rational_known_answers_in_fp16(case):
     assert torch.equal(O.matmul_tree(A, B, leaf=leaf).view(torch.int16), C.view(torch.int16))
 
 
+def _load_kat_f32():
+    z = np.load(GOLDEN)
+    for n in sorted({k[:-4] for k in z.files if k.endswith("_A32")}):
+        yield (n, torch.from_numpy(z[n + "_A32"].astype(np.float32)), torch.from_numpy(z[n + "_B32"].astype(np.float32)),
+               torch.from_numpy(z[n + "_C32"]))
+
+
+@pytest.mark.parametrize("case", list(_load_kat_f32()), ids=lambda c: c[0])
+def test_oracle_reproduces_rational_known_answers_in_fp32(case):
+    # float32 branch (leaves of 128, src/tbik/tree_based_matmul.py:223-231): one exact product per leaf, sums
+    # beyond 2^24, so only the tree order and fp32 rounding decide the bits
+    _, A, B, C = case
+    assert torch.equal(O.matmul_tree(A, B, leaf=128).view(torch.int32), C.view(torch.int32))
+
+
 def test_known_answers_discriminate_other_orders():
     # a sequential (left-to-right over all leaves) order or an fp32 tree must NOT reproduce the fixtures
     differs_seq = differs_f32 = 0
