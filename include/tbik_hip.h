@@ -193,6 +193,22 @@ int bi_gemm_f16(const void* A, int64_t lda,
                 tbik_stream_t stream);
 
 /*
+ * fp16 counterparts of bi_rmsnorm_bf16 and bi_silu_mul_bf16: same arguments, IEEE half elements, the same places
+ * where a value is rounded to the element type.
+ */
+int bi_rmsnorm_f16(const void* x, int64_t ldx,
+                   const void* residual_or_null, int64_t ldr,
+                   const void* weight_or_null,
+                   void* out, int64_t ldo,
+                   void* residual_out_or_null, int64_t ldro,
+                   int64_t rows, int hidden, float eps,
+                   tbik_stream_t stream);
+int bi_silu_mul_f16(const void* gate_up, int64_t ld_in,
+                    void* out, int64_t ld_out,
+                    int64_t rows, int inter,
+                    tbik_stream_t stream);
+
+/*
  * fp32 variants: C[M,N] = A[M,K] x B[K,N] (+ bias), all float.  tbik_gemm_f32 is tree-ordered with leaves of 128
  * (leaf_k must be 128, K a multiple of it): a leaf is the fp32 sum of its products, every tree node one fp32
  * addition; no workspace.  bi_gemm_f32 runs one fp32 accumulator over K (K a multiple of 16; callers pad with

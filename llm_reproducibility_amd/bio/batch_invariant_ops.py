@@ -66,8 +66,8 @@ def rms_norm(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, residu
     """Fused RMSNorm (optionally add-residual first) with the arithmetic of vLLM's forward_native, which is
     what the reference routes RMSNorm to (src/patch/patch_batch_invariant.py:9-16).  Returns `out`, or
     `(out, new_residual)` when a residual is given."""
-    if x.dtype != torch.bfloat16:
-        raise NotImplementedError("rms_norm on gfx950 is implemented for bfloat16")
+    if x.dtype not in (torch.bfloat16, torch.float16):
+        raise NotImplementedError("rms_norm on gfx950 is implemented for bfloat16 and float16")
     if residual is None:
         return ops.bi_rmsnorm_bf16(x, weight, eps)
     out, new_res = ops.bi_add_rmsnorm_bf16(x, residual, weight, eps)

@@ -9,7 +9,7 @@ int gemm_dispatch(bool tree, bool f16, const void* A, int64_t lda, const void* B
 size_t gemm_workspace_bytes(int M, int N, int K, int leaf_k, bool f16);
 int tree_combine_dispatch(const void* const* parts, int nparts, void* out, int64_t numel, bool f16, hipStream_t stream);
 int rmsnorm_dispatch(const void* x, int64_t ldx, const void* res, int64_t ldr, const void* w, void* out, int64_t ldo,
-                     void* res_out, int64_t ldro, int64_t rows, int hidden, float eps, hipStream_t stream);
+                     void* res_out, int64_t ldro, int64_t rows, int hidden, float eps, bool f16, hipStream_t stream);
 size_t lsm_workspace_bytes(int64_t rows, int64_t cols);
 int log_softmax_dispatch(const void* x, int64_t ldx, void* out, int64_t ldo, int64_t rows, int64_t cols, void* ws,
                          size_t ws_bytes, int write_softmax, hipStream_t stream);
@@ -19,13 +19,13 @@ int attention_dispatch(const void* q, const void* k_cache, const void* vt_cache,
 int mean_dispatch(const void* x, void* out, int64_t outer, int64_t n, int64_t inner, int dtype_code, hipStream_t stream);
 int gemm_f32_dispatch(bool tree, const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C,
                       int64_t ldc, int M, int N, int K, int leaf_k, const void* bias, hipStream_t stream);
-int silu_mul_dispatch(const void* gate_up, int64_t ld_in, void* out, int64_t ld_out, int64_t rows, int inter,
+int silu_mul_dispatch(const void* gate_up, int64_t ld_in, void* out, int64_t ld_out, int64_t rows, int inter, bool f16,
                       hipStream_t stream);
 }  // namespace tbik
 
 extern "C" {
 
-int tbik_abi_version(void) { return 6; }
+int tbik_abi_version(void) { return 7; }
 
 const char* tbik_error_string(int code) {
   switch (code) {
@@ -92,7 +92,14 @@ int bi_rmsnorm_bf16(const void* x, int64_t ldx, const void* residual_or_null, in
                     void* out, int64_t ldo, void* residual_out_or_null, int64_t ldro, int64_t rows, int hidden, float eps,
                     tbik_stream_t stream) {
   return tbik::rmsnorm_dispatch(x, ldx, residual_or_null, ldr, weight_or_null, out, ldo, residual_out_or_null, ldro, rows,
-                                hidden, eps, static_cast<hipStream_t>(stream));
+                                hidden, eps, false, static_cast<hipStream_t>(stream));
+}
+
+int bi_rmsnorm_f16(const void* x, int64_t ldx, const void* residual_or_null, int64_t ldr, const void* weight_or_null,
+                   void* out, int64_t ldo, void* residual_out_or_null, int64_t ldro, int64_t rows, int hidden, float eps,
+                   tbik_stream_t stream) {
+  return tbik::rmsnorm_dispatch(x, ldx, residual_or_null, ldr, weight_or_null, out, ldo, residual_out_or_null, ldro, rows,
+                                hidden, eps, true, static_cast<hipStream_t>(stream));
 }
 
 size_t bi_log_softmax_workspace_bytes(int64_t rows, int64_t cols) { return tbik::lsm_workspace_bytes(rows, cols); }
@@ -128,7 +135,12 @@ int bi_gemm_f32(const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_
 
 int bi_silu_mul_bf16(const void* gate_up, int64_t ld_in, void* out, int64_t ld_out, int64_t rows, int inter,
                      tbik_stream_t stream) {
-  return tbik::silu_mul_dispatch(gate_up, ld_in, out, ld_out, rows, inter, static_cast<hipStream_t>(stream));
+  return tbik::silu_mul_dispatch(gate_up, ld_in, out, ld_out, rows, inter, false, static_cast<hipStream_t>(stream));
+}
+
+int bi_silu_mul_f16(const void* gate_up, int64_t ld_in, void* out, int64_t ld_out, int64_t rows, int inter,
+                    tbik_stream_t stream) {
+  return tbik::silu_mul_dispatch(gate_up, ld_in, out, ld_out, rows, inter, true, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

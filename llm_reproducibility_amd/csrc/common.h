@@ -59,6 +59,8 @@ struct Num16<false> {
   static __device__ __forceinline__ uint32_t pack(float lo, float hi) { return pack_bf16x2(lo, hi); }
   static __device__ __forceinline__ uint32_t add(uint32_t a, uint32_t b) { return add_bf16x2(a, b); }
   static __device__ __forceinline__ float to_f32(uint16_t h) { return bf16_bits_to_f32(h); }
+  static __device__ __forceinline__ float lo(uint32_t p) { return bf16_lo(p); }
+  static __device__ __forceinline__ float hi(uint32_t p) { return bf16_hi(p); }
 };
 template <>
 struct Num16<true> {
@@ -68,6 +70,8 @@ struct Num16<true> {
   static __device__ __forceinline__ uint32_t pack(float lo, float hi) { return pack_f16x2(lo, hi); }
   static __device__ __forceinline__ uint32_t add(uint32_t a, uint32_t b) { return add_f16x2(a, b); }
   static __device__ __forceinline__ float to_f32(uint16_t h) { return f16_bits_to_f32(h); }
+  static __device__ __forceinline__ float lo(uint32_t p) { return (float)__builtin_bit_cast(f16x2, p)[0]; }
+  static __device__ __forceinline__ float hi(uint32_t p) { return (float)__builtin_bit_cast(f16x2, p)[1]; }
 };
 
 // Butterfly reductions over the 64 lanes of a wavefront.  The exchange pattern is fixed, so the

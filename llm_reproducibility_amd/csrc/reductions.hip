@@ -1,4 +1,4 @@
-// Batch-invariant row reductions for gfx950: RMSNorm (bf16), log_softmax / softmax (fp32), mean.
+// Batch-invariant row reductions for gfx950: RMSNorm (bf16 or fp16), log_softmax / softmax (fp32), mean.
 //
 // Rule shared by all kernels here: the decomposition of a row into lanes, wavefronts and segments,
 // and the order in which partial sums meet, is a function of the ROW LENGTH only.  The number of rows
@@ -27,8 +27,9 @@ struct RmsArgs {
   float eps;
 };
 
-template <int CPL>  // chunks (8 bf16) per lane kept in registers
+template <int CPL, bool F16>  // chunks (8 elements) per lane kept in registers; bf16 or fp16 elements
 __global__ __launch_bounds__(256) void rmsnorm_kernel(const RmsArgs a) {
+  using Num = Num16<F16>;
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= a.rows) return;
@@ -46,8 +47,8 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const RmsArgs a) {
       const uint32_t u[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
       for (int e = 0; e < 4; e++) {
-        v[i][2 * e] = bf16_lo(u[e]);
-        v[i][2 * e + 1] = bf16_hi(u[e]);
+        v[i][2 * e] = Num::lo(u[e]);
+        v[i][2 * e + 1] = Num::hi(u[e]);
       }
       if (rr) {
         const uint4 r = rr[c];
@@ -55,9 +56,9 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const RmsArgs a) {
         uint32_t so[4];
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-          v[i][2 * e] += bf16_lo(ru[e]);
-          v[i][2 * e + 1] += bf16_hi(ru[e]);
-          so[e] = pack_bf16x2(v[i][2 * e], v[i][2 * e + 1]);
+          v[i][2 * e] += Num::lo(ru[e]);
+          v[i][2 * e + 1] += Num::hi(ru[e]);
+          so[e] = Num::pack(v[i][2 * e], v[i][2 * e + 1]);
         }
         if (a.res_out) reinterpret_cast<uint4*>(a.res_out + row * a.ldro)[c] = make_uint4(so[0], so[1], so[2], so[3]);
       }
@@ -76,21 +77,31 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const RmsArgs a) {
     if (c < nchunks) {
       uint32_t o[4];
 #pragma unroll
-      for (int e = 0; e < 4; e++) o[e] = pack_bf16x2(v[i][2 * e] * rs, v[i][2 * e + 1] * rs);
+      for (int e = 0; e < 4; e++) o[e] = Num::pack(v[i][2 * e] * rs, v[i][2 * e + 1] * rs);
       if (wr) {
         const uint4 wq = wr[c];
         const uint32_t wu[4] = {wq.x, wq.y, wq.z, wq.w};
 #pragma unroll
         for (int e = 0; e < 4; e++)
-          o[e] = pack_bf16x2(bf16_lo(o[e]) * bf16_lo(wu[e]), bf16_hi(o[e]) * bf16_hi(wu[e]));
+          o[e] = Num::pack(Num::lo(o[e]) * Num::lo(wu[e]), Num::hi(o[e]) * Num::hi(wu[e]));
       }
       orow[c] = make_uint4(o[0], o[1], o[2], o[3]);
     }
   }
 }
 
+template <bool F16>
+static void rmsnorm_launch(const RmsArgs& a, int cpl, dim3 grid, hipStream_t stream) {
+  const dim3 block(256);
+  if (cpl <= 1) hipLaunchKernelGGL((rmsnorm_kernel<1, F16>), grid, block, 0, stream, a);
+  else if (cpl <= 2) hipLaunchKernelGGL((rmsnorm_kernel<2, F16>), grid, block, 0, stream, a);
+  else if (cpl <= 4) hipLaunchKernelGGL((rmsnorm_kernel<4, F16>), grid, block, 0, stream, a);
+  else if (cpl <= 8) hipLaunchKernelGGL((rmsnorm_kernel<8, F16>), grid, block, 0, stream, a);
+  else hipLaunchKernelGGL((rmsnorm_kernel<16, F16>), grid, block, 0, stream, a);
+}
+
 int rmsnorm_dispatch(const void* x, int64_t ldx, const void* res, int64_t ldr, const void* w, void* out, int64_t ldo,
-                     void* res_out, int64_t ldro, int64_t rows, int hidden, float eps, hipStream_t stream) {
+                     void* res_out, int64_t ldro, int64_t rows, int hidden, float eps, bool f16, hipStream_t stream) {
   if (!x || !out || rows < 0 || hidden <= 0) return TBIK_ERR_INVALID;
   if (res && !res_out) return TBIK_ERR_INVALID;
   if (rows == 0) return TBIK_OK;
@@ -103,13 +114,10 @@ int rmsnorm_dispatch(const void* x, int64_t ldx, const void* res, int64_t ldr, c
             static_cast<uint16_t*>(out), static_cast<uint16_t*>(res_out), ldx, ldr, ldo, ldro, rows, hidden, eps};
   const int64_t blocks = (rows + 3) / 4;
   if (blocks > 0x7fffffff) return TBIK_ERR_INVALID;
-  const dim3 grid((unsigned)blocks), block(256);
+  const dim3 grid((unsigned)blocks);
   const int cpl = (hidden + 511) / 512;  // a function of the row length only
-  if (cpl <= 1) hipLaunchKernelGGL(rmsnorm_kernel<1>, grid, block, 0, stream, a);
-  else if (cpl <= 2) hipLaunchKernelGGL(rmsnorm_kernel<2>, grid, block, 0, stream, a);
-  else if (cpl <= 4) hipLaunchKernelGGL(rmsnorm_kernel<4>, grid, block, 0, stream, a);
-  else if (cpl <= 8) hipLaunchKernelGGL(rmsnorm_kernel<8>, grid, block, 0, stream, a);
-  else hipLaunchKernelGGL(rmsnorm_kernel<16>, grid, block, 0, stream, a);
+  if (f16) rmsnorm_launch<true>(a, cpl, grid, stream);
+  else rmsnorm_launch<false>(a, cpl, grid, stream);
   return hip_code(hipGetLastError());
 }
 

@@ -202,9 +202,10 @@ def _bi_rmsnorm_bf16_impl(x: torch.Tensor, weight: Optional[torch.Tensor], eps: 
     _require_gpu(x, weight)
     hidden = x.shape[-1]
     x2, ldx = _rows16(x.reshape(-1, hidden))
-    out = torch.empty((x2.shape[0], hidden), device=x.device, dtype=torch.bfloat16)
+    out = torch.empty((x2.shape[0], hidden), device=x.device, dtype=x.dtype)
     w = None if weight is None else weight.contiguous()
-    rc = _lib.lib().bi_rmsnorm_bf16(x2.data_ptr(), ldx, None, 0, None if w is None else w.data_ptr(),
+    L = _lib.lib()
+    rc = (L.bi_rmsnorm_f16 if _is_f16(x, weight) else L.bi_rmsnorm_bf16)(x2.data_ptr(), ldx, None, 0, None if w is None else w.data_ptr(),
                                     out.data_ptr(), out.stride(0), None, 0, x2.shape[0], hidden, eps, _stream(x))
     _lib.check(rc, "bi_rmsnorm_bf16")
     return out.reshape(x.shape)
@@ -230,10 +231,11 @@ def _bi_add_rmsnorm_bf16_impl(x: torch.Tensor, residual: torch.Tensor, weight: O
     hidden = x.shape[-1]
     x2, ldx = _rows16(x.reshape(-1, hidden))
     r2, ldr = _rows16(residual.reshape(-1, hidden))
-    out = torch.empty((x2.shape[0], hidden), device=x.device, dtype=torch.bfloat16)
+    out = torch.empty((x2.shape[0], hidden), device=x.device, dtype=x.dtype)
     rout = torch.empty_like(out)
     w = None if weight is None else weight.contiguous()
-    rc = _lib.lib().bi_rmsnorm_bf16(x2.data_ptr(), ldx, r2.data_ptr(), ldr,
+    L = _lib.lib()
+    rc = (L.bi_rmsnorm_f16 if _is_f16(x, residual, weight) else L.bi_rmsnorm_bf16)(x2.data_ptr(), ldx, r2.data_ptr(), ldr,
                                     None if w is None else w.data_ptr(), out.data_ptr(), out.stride(0),
                                     rout.data_ptr(), rout.stride(0), x2.shape[0], hidden, eps, _stream(x))
     _lib.check(rc, "bi_rmsnorm_bf16")
@@ -365,15 +367,15 @@ def _(q, k_cache, vt_cache, q_start, q_len, ctx_len, max_q_len, scale):
 # --------------------------------------------------------------------------------------------
 def _bi_silu_mul_bf16_impl(gate_up: torch.Tensor) -> torch.Tensor:
     _require_gpu(gate_up)
-    if gate_up.dtype != torch.bfloat16:
-        raise NotImplementedError(f"bi_silu_mul_bf16: unsupported dtype {gate_up.dtype}")
+    f16 = _is_f16(gate_up)
     two_i = gate_up.shape[-1]
     if two_i % 16 != 0:
         raise ValueError(f"bi_silu_mul_bf16: last dimension {two_i} must be a multiple of 16")
     inter = two_i // 2
     g2, ld = _rows16(gate_up.reshape(-1, two_i))
-    out = torch.empty((g2.shape[0], inter), device=gate_up.device, dtype=torch.bfloat16)
-    rc = _lib.lib().bi_silu_mul_bf16(g2.data_ptr(), ld, out.data_ptr(), out.stride(0), g2.shape[0], inter, _stream(gate_up))
+    out = torch.empty((g2.shape[0], inter), device=gate_up.device, dtype=gate_up.dtype)
+    L = _lib.lib()
+    rc = (L.bi_silu_mul_f16 if f16 else L.bi_silu_mul_bf16)(g2.data_ptr(), ld, out.data_ptr(), out.stride(0), g2.shape[0], inter, _stream(gate_up))
     _lib.check(rc, "bi_silu_mul_bf16")
     return out.reshape(*gate_up.shape[:-1], inter)
 

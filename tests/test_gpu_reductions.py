@@ -28,6 +28,29 @@ def test_rmsnorm_parity_and_batch_invariance(dev):
     assert torch.equal(bio.rms_norm(s.to(dev), torch.ones(4096, dtype=torch.bfloat16, device=dev), 1e-6).cpu(), s)
 
 
+def test_fp16_rmsnorm_and_silu_mul(dev):
+    from llm_reproducibility_amd import ops
+    x = O.gaussian_bf16((300, 4096), 1.0, 0).to(torch.float16)
+    r = O.gaussian_bf16((300, 4096), 1.0, 3).to(torch.float16)
+    w = (1.0 + 0.1 * torch.randn(4096, generator=torch.Generator().manual_seed(1))).to(torch.float16)
+    got = bio.rms_norm(x.to(dev), w.to(dev), 1e-6)
+    want = O.rmsnorm(x, w, 1e-6)
+    assert got.dtype == torch.float16
+    assert ((got.cpu().float() - want.float()).abs() <= 2.0 ** -9 * want.float().abs().clamp_min(2.0 ** -4)).all()
+    g2, res2 = bio.rms_norm(x.to(dev), w.to(dev), 1e-6, residual=r.to(dev))
+    w2, wres = O.rmsnorm(x, w, 1e-6, residual=r)
+    assert torch.equal(res2.cpu(), wres)
+    assert ((g2.cpu().float() - w2.float()).abs() <= 2.0 ** -9 * w2.float().abs().clamp_min(2.0 ** -4)).all()
+    for rows in (1, 7, 64):
+        assert torch.equal(bio.rms_norm(x[:rows].to(dev), w.to(dev), 1e-6), got[:rows])
+    gu = (torch.randn((65, 2 * 1024), generator=torch.Generator().manual_seed(2)) * 2).to(torch.float16)
+    act = ops.bi_silu_mul_bf16(gu.to(dev))
+    wa = O.silu_mul(gu)
+    assert act.dtype == torch.float16
+    assert ((act.cpu().float() - wa.float()).abs() <= 2.0 ** -9 * wa.float().abs().clamp_min(2.0 ** -6)).all()
+    assert torch.equal(ops.bi_silu_mul_bf16(gu[:3].to(dev)), act[:3])
+
+
 def test_add_rmsnorm_parity(dev):
     x = O.gaussian_bf16((64, 4096), 1.0, 2)
     res = O.gaussian_bf16((64, 4096), 1.0, 3)
