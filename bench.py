@@ -119,6 +119,21 @@ def table(steps, warmup):
         x = torch.randn((r, 2 * 12288), device=dev).to(torch.bfloat16)
         ms, _ = hip_time_ms(lambda: ops.bi_silu_mul_bf16(x), steps, warmup)
         rows.append((f"silu_mul rows={r} inter=12288 (6 B/elem)", ms * 1e3, 0.0, r * 12288 * 6 / ms / 1e6))
+    # fixed-order attention (Qwen3-8B heads: 32 query, 8 key/value, head_dim 128)
+    Hq, Hkv, D = 32, 8, 128
+    def i32(v):
+        return torch.tensor(v, dtype=torch.int32, device=dev)
+    for name, B, qlen, ctx in (("prefill 8 x 512", 8, 512, 512), ("prefill 1 x 4096", 1, 4096, 4096),
+                               ("decode 128 seqs ctx 768", 128, 1, 768), ("decode 8 seqs ctx 4096", 8, 1, 4096)):
+        L = ((ctx + 31) // 32) * 32
+        q = torch.randn((B * qlen, Hq, D), device=dev).to(torch.bfloat16)
+        kc = torch.randn((B, Hkv, L, D), device=dev).to(torch.bfloat16)
+        vt = torch.randn((B, Hkv, D, L), device=dev).to(torch.bfloat16)
+        qs, ql, cl = i32([b * qlen for b in range(B)]), i32([qlen] * B), i32([ctx] * B)
+        ms, _ = hip_time_ms(lambda: ops.bi_attention_bf16(q, kc, vt, qs, ql, cl, qlen, D ** -0.5), max(steps // 2, 3), warmup)
+        pairs = B * Hq * (qlen * (2 * ctx - qlen + 1) // 2)          # causal (query, key) pairs
+        byts = 2.0 * (2 * B * Hkv * ctx * D + 2 * B * qlen * Hq * D)   # K, V once; q and out
+        rows.append((f"attention {name}", ms * 1e3, 4.0 * pairs * D / ms / 1e9, byts / ms / 1e6))
     print(f"{'case':52s} {'us':>10s} {'TFLOP/s':>9s} {'%MFMA':>6s} {'GB/s':>9s} {'%HBM':>6s}", file=sys.stderr)
     for name, us, tf, gbs in rows:
         print(f"{name:52s} {us:10.1f} {tf:9.1f} {100 * tf / PEAK_BF16_TFLOPS:6.1f} {gbs:9.1f} {100 * gbs / PEAK_HBM_GBS:6.1f}",

@@ -135,6 +135,148 @@ __global__ __launch_bounds__(64) void attention_kernel(const AttnArgs a) {
   }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Grouped variant: one work-group per (16 consecutive queries, KV head, sequence); its G wavefronts are the G query
+// heads that share the KV head.  Each 32-key tile of K and of V^T is fetched from global memory ONCE per group with
+// coalesced 16-byte loads, staged in LDS (double buffered, XOR-swizzled against bank conflicts) and read from there
+// by every wave.  A row's arithmetic -- the lanes that own it, the MFMA chain, the order of the softmax updates --
+// is exactly that of attention_kernel above, so both kernels produce the same bits; this one just moves 1/G of
+// the bytes and hides the load latency behind the previous tile.
+// ------------------------------------------------------------------------------------------------
+template <int G>
+__global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs a) {
+  __shared__ __attribute__((aligned(16))) uint8_t lds[2][16384];  // per buffer: K tile [32][128] (8 KiB), V^T tile [128][32] (8 KiB)
+  const int b = blockIdx.z;
+  const int kvh = blockIdx.y;
+  const int qb = blockIdx.x;
+  const int qlen = a.q_len[b];
+  if (qb * 16 >= qlen) return;  // uniform over the work-group
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int h = kvh * G + (tid >> 6);
+  const int j = lane & 15;
+  const int g = lane >> 4;
+  const int ctx = a.ctx_len[b];
+  const int qrow = qb * 16 + j;
+  const bool qvalid = qrow < qlen;
+  const int qpos = ctx - qlen + min(qrow, qlen - 1);
+  const int last_pos = ctx - qlen + min(qb * 16 + 15, qlen - 1);
+
+  const uint16_t* qp = a.q + ((int64_t)(a.q_start[b] + min(qrow, qlen - 1)) * a.q_heads + h) * HD;
+  bf16x8 qf[4];
+#pragma unroll
+  for (int c = 0; c < 4; c++) qf[c] = *reinterpret_cast<const bf16x8*>(qp + c * 32 + g * 8);
+
+  const uint8_t* kbase = reinterpret_cast<const uint8_t*>(a.k_cache + ((int64_t)b * a.kv_heads + kvh) * a.max_len * HD);
+  const uint8_t* vbase = reinterpret_cast<const uint8_t*>(a.vt_cache + ((int64_t)b * a.kv_heads + kvh) * (int64_t)HD * a.max_len);
+
+  // cooperative staging: 512 16-byte chunks per tile and operand, NCH per thread
+  constexpr int NT = 64 * G;
+  constexpr int NCH = (512 + NT - 1) / NT;
+  u32x4 kreg[NCH], vreg[NCH];
+  auto load_tile = [&](int tile) __attribute__((always_inline)) {
+    const int k0 = min(tile * 32, a.max_len - 32);  // max_len is a multiple of 32: never past the cache
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+      const int ch = tid + i * NT;
+      if (512 % NT == 0 || ch < 512) {
+        kreg[i] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)(k0 + (ch >> 4)) * (HD * 2) + (ch & 15) * 16);
+        vreg[i] = *reinterpret_cast<const u32x4*>(vbase + ((int64_t)(ch >> 2) * a.max_len + k0) * 2 + (ch & 3) * 16);
+      }
+    }
+  };
+  auto store_tile = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+      const int ch = tid + i * NT;
+      if (512 % NT == 0 || ch < 512) {
+        const int kr = ch >> 4, kc = ch & 15;   // key row, 16-byte chunk of its 256 bytes
+        *reinterpret_cast<u32x4*>(&lds[buf][kr * 256 + ((kc ^ (2 * (kr & 7))) << 4)]) = kreg[i];
+        const int vr = ch >> 2, vc = ch & 3;    // channel row, 16-byte chunk of its 64 bytes
+        *reinterpret_cast<u32x4*>(&lds[buf][8192 + vr * 64 + ((vc ^ ((vr >> 2) & 3)) << 4)]) = vreg[i];
+      }
+    }
+  };
+
+  f32x4 o[8];
+#pragma unroll
+  for (int t = 0; t < 8; t++) o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY;
+  float l = 0.f;
+
+  const int ntiles = last_pos / 32 + 1;
+  load_tile(0);
+  store_tile(0);
+  __syncthreads();
+  for (int tile = 0; tile < ntiles; tile++) {
+    const int cur = tile & 1;
+    if (tile + 1 < ntiles) load_tile(tile + 1);
+    const int k0 = tile * 32;
+    f32x4 s[2];
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+      const int kr = 16 * u + j;
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(&lds[cur][kr * 256 + (((c * 4 + g) ^ (2 * (kr & 7))) << 4)]);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[c], acc, 0, 0, 0);
+      }
+      s[u] = acc;
+    }
+    float sv[8];
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < 2; u++)
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const int key = k0 + 16 * u + 4 * g + i;
+        const float v = (key <= qpos) ? s[u][i] * a.scale_log2 : -INFINITY;
+        sv[4 * u + i] = v;
+        tmax = fmaxf(tmax, v);
+      }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_new = fmaxf(m, tmax);
+    const float alpha = exp2f(m - m_new);
+    float psum = 0.f;
+    float pv[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      pv[e] = exp2f(sv[e] - m_new);
+      psum += pv[e];
+    }
+    psum += __shfl_xor(psum, 16, 64);
+    psum += __shfl_xor(psum, 32, 64);
+    l = l * alpha + psum;
+    m = m_new;
+    const uint32_t p0 = pack_bf16x2(pv[0], pv[1]), p1 = pack_bf16x2(pv[2], pv[3]);
+    const uint32_t p2 = pack_bf16x2(pv[4], pv[5]), p3 = pack_bf16x2(pv[6], pv[7]);
+    const bf16x8 pf = __builtin_bit_cast(bf16x8, u32x4{p0, p1, p2, p3});
+#pragma unroll
+    for (int t = 0; t < 8; t++) {
+      const int vr = 16 * t + j;
+      const int sw = 2 * ((vr >> 2) & 3);  // 8-byte slots: keys 4g.. sit in slot g, keys 16+4g.. in slot 4+g
+      const uint2 va = *reinterpret_cast<const uint2*>(&lds[cur][8192 + vr * 64 + ((g ^ sw) << 3)]);
+      const uint2 vb = *reinterpret_cast<const uint2*>(&lds[cur][8192 + vr * 64 + (((4 + g) ^ sw) << 3)]);
+      const bf16x8 vf = __builtin_bit_cast(bf16x8, u32x4{va.x, va.y, vb.x, vb.y});
+      f32x4 scaled = {o[t][0] * alpha, o[t][1] * alpha, o[t][2] * alpha, o[t][3] * alpha};
+      o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, scaled, 0, 0, 0);
+    }
+    if (tile + 1 < ntiles) store_tile(cur ^ 1);
+    __syncthreads();
+  }
+  if (!qvalid) return;
+  const float inv = 1.0f / l;
+  uint16_t* op = a.out + ((int64_t)(a.q_start[b] + qrow) * a.q_heads + h) * HD;
+#pragma unroll
+  for (int t = 0; t < 8; t++) {
+    const uint32_t lo = pack_bf16x2(o[t][0] * inv, o[t][1] * inv);
+    const uint32_t hi = pack_bf16x2(o[t][2] * inv, o[t][3] * inv);
+    *reinterpret_cast<uint2*>(op + 16 * t + 4 * g) = make_uint2(lo, hi);
+  }
+}
+
 int attention_dispatch(const void* q, const void* k_cache, const void* vt_cache, void* out, const int* q_start,
                        const int* q_len, const int* ctx_len, int batch, int max_q_len, int q_heads, int kv_heads,
                        int head_dim, int max_len, float scale, hipStream_t stream) {
@@ -147,8 +289,19 @@ int attention_dispatch(const void* q, const void* k_cache, const void* vt_cache,
   if (batch > 65535 || q_heads > 65535) return TBIK_ERR_INVALID;
   AttnArgs a{static_cast<const uint16_t*>(q), static_cast<const uint16_t*>(k_cache), static_cast<const uint16_t*>(vt_cache),
              static_cast<uint16_t*>(out), q_start, q_len, ctx_len, q_heads, kv_heads, max_len, scale * 1.4426950408889634f};
-  const dim3 grid((unsigned)((max_q_len + 15) / 16), (unsigned)q_heads, (unsigned)batch);
-  hipLaunchKernelGGL(attention_kernel, grid, dim3(64), 0, stream, a);
+  // the grouped kernel needs whole 32-key tiles in the caches and at most 8 query heads per KV head
+  const int G = q_heads / kv_heads;
+  const bool grouped = (max_len & 31) == 0 && (G == 1 || G == 2 || G == 4 || G == 8) && kv_heads <= 65535;
+  if (grouped) {
+    const dim3 grid((unsigned)((max_q_len + 15) / 16), (unsigned)kv_heads, (unsigned)batch);
+    if (G == 1) hipLaunchKernelGGL(attention_group_kernel<1>, grid, dim3(64), 0, stream, a);
+    else if (G == 2) hipLaunchKernelGGL(attention_group_kernel<2>, grid, dim3(128), 0, stream, a);
+    else if (G == 4) hipLaunchKernelGGL(attention_group_kernel<4>, grid, dim3(256), 0, stream, a);
+    else hipLaunchKernelGGL(attention_group_kernel<8>, grid, dim3(512), 0, stream, a);
+  } else {
+    const dim3 grid((unsigned)((max_q_len + 15) / 16), (unsigned)q_heads, (unsigned)batch);
+    hipLaunchKernelGGL(attention_kernel, grid, dim3(64), 0, stream, a);
+  }
   return hip_code(hipGetLastError());
 }
 

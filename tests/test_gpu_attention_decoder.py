@@ -65,6 +65,22 @@ def test_attention_matches_fp32_reference_and_is_batch_and_phase_invariant(dev):
     # chunked prefill: the last 5 tokens of sequence 0 against the cache == the same rows of the full prefill
     tail = ops.bi_attention_bf16(qs[0][-5:], kc[:1], vt[:1], i32([0]), i32([5]), i32([lens[0]]), 5, scale)
     assert torch.equal(tail, out[starts[0] + lens[0] - 5: starts[0] + lens[0]])
+    # a cache length that is not a whole number of 32-key tiles takes the one-wave-per-head kernel instead of the
+    # grouped one (K/V tiles staged in LDS once per KV head): same per-row arithmetic, same bits
+    kc2, vt2 = _make_cache(ks, vs, 164, dev)
+    out2 = ops.bi_attention_bf16(torch.cat(qs), kc2, vt2, i32(starts), i32(lens), i32(lens), max(lens), scale)
+    assert torch.equal(out2, out)
+    # other group sizes (query heads per KV head): 1, 2, 8
+    for hq, hkv in ((2, 2), (4, 2), (16, 2)):
+        k1 = [torch.randn((n, hkv, D), device=dev).to(torch.bfloat16) for n in lens[:3]]
+        v1 = [torch.randn((n, hkv, D), device=dev).to(torch.bfloat16) for n in lens[:3]]
+        q1 = [torch.randn((n, hq, D), device=dev).to(torch.bfloat16) for n in lens[:3]]
+        st = [sum(lens[:i]) for i in range(3)]
+        ca, va = _make_cache(k1, v1, 96, dev)
+        cb, vb = _make_cache(k1, v1, 100, dev)
+        oa = ops.bi_attention_bf16(torch.cat(q1), ca, va, i32(st), i32(lens[:3]), i32(lens[:3]), max(lens[:3]), scale)
+        ob = ops.bi_attention_bf16(torch.cat(q1), cb, vb, i32(st), i32(lens[:3]), i32(lens[:3]), max(lens[:3]), scale)
+        assert torch.equal(oa, ob), (hq, hkv)
 
 
 SMALL = DecoderConfig(vocab_size=3000, hidden_size=1024, num_layers=2, num_q_heads=16, num_kv_heads=4, head_dim=128,
