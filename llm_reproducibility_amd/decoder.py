@@ -53,9 +53,12 @@ class _Layer:
 
 
 class Qwen3Decoder:
-    def __init__(self, cfg: DecoderConfig, tp_size: int = 1, seed: int = 0, device="cuda:0"):
+    def __init__(self, cfg: DecoderConfig, tp_size: int = 1, seed: int = 0, device="cuda:0", use_graphs: bool = False):
         assert cfg.head_dim == 128, "the attention kernel is built for head_dim 128"
         self.cfg, self.tp_size, self.device = cfg, tp_size, torch.device(device)
+        # decode steps replayed from one captured HIP graph (same kernels, same order, same bits as eager; the
+        # per-step host work shrinks to one graph launch, which is what bounds small batches)
+        self.use_graphs = use_graphs
         gen = torch.Generator().manual_seed(seed)
         emb = lambda *shape: (torch.randn(shape, generator=gen, dtype=torch.float32) * 0.02).to(torch.bfloat16).to(self.device)  # noqa: E731
         self.embed = emb(cfg.vocab_size, cfg.hidden_size)
@@ -141,14 +144,40 @@ class Qwen3Decoder:
         q_start = torch.arange(B, dtype=torch.int32, device=dev)
         q_len = torch.ones(B, dtype=torch.int32, device=dev)
         seq = torch.arange(B, dtype=torch.long, device=dev)
-        cur = torch.tensor(lens, dtype=torch.long, device=dev)
-        for _ in range(max_new_tokens - 1):
-            ctx = (cur + 1).to(torch.int32)
-            h = self._forward(out_ids[-1], cur, seq, q_start, q_len, ctx, 1, cache)
+        # the step works on static tensors, so that it can be captured once and replayed
+        tok_s = out_ids[-1].clone()
+        pos_s = torch.tensor(lens, dtype=torch.long, device=dev)
+        ctx_s = (pos_s + 1).to(torch.int32)
+
+        def step():
+            h = self._forward(tok_s, pos_s, seq, q_start, q_len, ctx_s, 1, cache)
             logits = matmul_persistent(h, self.lm_head.t())
-            out_ids.append(self._greedy(logits))
+            nxt = self._greedy(logits)
+            tok_s.copy_(nxt)
+            pos_s.add_(1)
+            ctx_s.add_(1)
+            return nxt, logits
+
+        def record(nxt, logits):
+            out_ids.append(nxt.clone())
             if return_logits:
-                all_logits.append(logits)
-            cur = cur + 1
+                all_logits.append(logits.clone())
+
+        steps = max_new_tokens - 1
+        if self.use_graphs and steps >= 3:
+            side = torch.cuda.Stream(device=dev)
+            side.wait_stream(torch.cuda.current_stream(dev))
+            with torch.cuda.stream(side):
+                record(*step())          # first step eagerly on the capture stream (also warms every kernel up)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                static_next, static_logits = step()
+            torch.cuda.current_stream(dev).wait_stream(side)
+            for _ in range(steps - 1):
+                graph.replay()
+                record(static_next, static_logits)
+        else:
+            for _ in range(steps):
+                record(*step())
         ids = torch.stack(out_ids, dim=1)
         return (ids, torch.stack(all_logits, dim=1)) if return_logits else ids

@@ -119,6 +119,23 @@ def test_greedy_decode_is_identical_across_tp_and_batch(dev):
         del m
 
 
+def test_graph_replayed_decode_steps_equal_eager_steps(dev):
+    """Every replay of the captured decode step must give the eager step's bits (token ids and logits)."""
+    prompts = _prompts(5, seed=7)
+    eager = Qwen3Decoder(SMALL, tp_size=2, seed=0, device=dev)
+    graphed = Qwen3Decoder(SMALL, tp_size=2, seed=0, device=dev, use_graphs=True)
+    ids_e, log_e = eager.generate(prompts, 9, return_logits=True)
+    torch.cuda.synchronize()
+    ids_g, log_g = graphed.generate(prompts, 9, return_logits=True)
+    torch.cuda.synchronize()
+    assert torch.equal(ids_g, ids_e)
+    for step in range(log_e.shape[1]):
+        assert torch.equal(log_g[:, step], log_e[:, step]), step
+    # a second generation on the same object (new capture, new caches) and another batch size
+    ids_g2 = graphed.generate(prompts[:2], 6)
+    assert torch.equal(ids_g2, eager.generate(prompts[:2], 6))
+
+
 def test_decoder_logits_agree_with_plain_pytorch_math(dev):
     """Tolerance check of the whole stack against a straightforward fp32 PyTorch forward of the same weights."""
     cfg = DecoderConfig(vocab_size=512, hidden_size=512, num_layers=2, num_q_heads=8, num_kv_heads=2, head_dim=128,
