@@ -117,7 +117,7 @@ def table(steps, warmup):
     from llm_reproducibility_amd import ops
     for r in (1, 256, 4096):
         x = torch.randn((r, 2 * 12288), device=dev).to(torch.bfloat16)
-        ms, _ = hip_time_ms(lambda: ops.bi_silu_mul_bf16(x), steps, warmup)
+        ms, _ = hip_time_ms(lambda: ops.bi_silu_mul(x), steps, warmup)
         rows.append((f"silu_mul rows={r} inter=12288 (6 B/elem)", ms * 1e3, 0.0, r * 12288 * 6 / ms / 1e6))
     # fixed-order attention (Qwen3-8B heads: 32 query, 8 key/value, head_dim 128)
     Hq, Hkv, D = 32, 8, 128

@@ -35,7 +35,7 @@ def matmul_persistent(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Ten
         raise NotImplementedError(f"batch-invariant mm on gfx950 takes bfloat16, float16 or float32, got {a.dtype}")
     if bias is not None and bias.dtype != a.dtype:
         bias = bias.to(a.dtype)
-    return ops.bi_gemm_bf16(a, b, bias)
+    return ops.bi_gemm(a, b, bias)
 
 
 def log_softmax(input: torch.Tensor, dim: int = -1) -> torch.Tensor:
@@ -69,8 +69,8 @@ def rms_norm(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, residu
     if x.dtype not in (torch.bfloat16, torch.float16):
         raise NotImplementedError("rms_norm on gfx950 is implemented for bfloat16 and float16")
     if residual is None:
-        return ops.bi_rmsnorm_bf16(x, weight, eps)
-    out, new_res = ops.bi_add_rmsnorm_bf16(x, residual, weight, eps)
+        return ops.bi_rmsnorm(x, weight, eps)
+    out, new_res = ops.bi_add_rmsnorm(x, residual, weight, eps)
     return out, new_res
 
 

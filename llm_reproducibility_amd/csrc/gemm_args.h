@@ -1,0 +1,40 @@
+// Argument blocks and entry points of the large-M GEMM kernels, shared by the kernels' own files and by the
+// dispatcher in gemm_tiled.hip.
+#pragma once
+#include "common.h"
+
+namespace tbik {
+
+// gemm_tree_wide.hip: tree-ordered bf16 GEMM, 128x256 tiles
+struct WideArgs {
+  const uint16_t* X;   // [M,K], row stride ldx
+  const uint16_t* W;   // [N,K], row stride ldw
+  uint16_t* C;         // [M,N], row stride ldc
+  const uint16_t* bias;
+  u32x4* ws;           // parked tree levels: [level][shard * tile][wave][chunk 0..7][lane]
+  int64_t ldx, ldw, ldc;
+  int M, N, K;
+  int T, flb, lb;
+  int vec_store;
+  int64_t k_shard, c_shard;  // K split over gridDim.y shards: operand column offset and partial-output offset per shard
+};
+size_t wide_workspace_bytes(int M, int N, int lb, int split);
+int gemm_tree_wide_launch(const WideArgs& a, int leaf_k, int split, hipStream_t stream);
+
+// gemm_single_acc_quad.hip: single-accumulator bf16 GEMM, one wave per SIMD
+struct QuadArgs {
+  const uint16_t* X;   // [M,K], row stride ldx
+  const uint16_t* W;   // [N,K], row stride ldw
+  uint16_t* C;         // [M,N], row stride ldc
+  const uint16_t* bias;
+  int64_t ldx, ldw, ldc;
+  int M, N, K;
+  int vec_store;
+};
+int gemm_single_acc_quad_launch(const QuadArgs& a, hipStream_t stream);
+
+// tree_combine.hip
+int tree_combine_bias_dispatch(const void* const* parts, int nparts, void* out, int64_t numel, const void* bias, int N,
+                               bool f16, hipStream_t stream);
+
+}  // namespace tbik

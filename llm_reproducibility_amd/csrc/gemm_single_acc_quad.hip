@@ -13,18 +13,9 @@
 //   * one barrier per slice, placed BETWEEN its two 32-wide k steps, so fragment reads always run one k step
 //     ahead of the MFMAs, also across the barrier; scheduling fences keep that order in the generated code.
 #include "common.h"
+#include "gemm_args.h"
 
 namespace tbik {
-
-struct QuadArgs {
-  const uint16_t* X;   // [M,K], row stride ldx
-  const uint16_t* W;   // [N,K], row stride ldw
-  uint16_t* C;         // [M,N], row stride ldc
-  const uint16_t* bias;
-  int64_t ldx, ldw, ldc;
-  int M, N, K;
-  int vec_store;
-};
 
 namespace quad {
 constexpr int BM = 128, BN = 256, BK = 64, NT = 256, NWAVE = 4, TM = 4, TN = 8;

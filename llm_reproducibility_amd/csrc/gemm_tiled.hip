@@ -17,6 +17,7 @@
 // Operand roles: W ([N,K], K contiguous) feeds the MFMA "A" port and X ([M,K]) the "B" port, so an
 // output lane holds 4 consecutive n of one m and stores them as one 8-byte word.
 #include "common.h"
+#include "gemm_args.h"
 
 namespace tbik {
 
@@ -323,36 +324,6 @@ static int launch_tree(const GemmArgs& a, int split, hipStream_t stream) {
 }
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
-
-// large-M kernel (gemm_tree_wide.hip)
-struct WideArgs {
-  const uint16_t* X;
-  const uint16_t* W;
-  uint16_t* C;
-  const uint16_t* bias;
-  u32x4* ws;
-  int64_t ldx, ldw, ldc;
-  int M, N, K;
-  int T, flb, lb;
-  int vec_store;
-  int64_t k_shard, c_shard;
-};
-size_t wide_workspace_bytes(int M, int N, int lb, int split);
-int gemm_tree_wide_launch(const WideArgs& a, int leaf_k, int split, hipStream_t stream);
-int tree_combine_bias_dispatch(const void* const* parts, int nparts, void* out, int64_t numel, const void* bias, int N,
-                               bool f16, hipStream_t stream);
-
-// one-wave-per-SIMD single-accumulator kernel (gemm_single_acc_quad.hip)
-struct QuadArgs {
-  const uint16_t* X;
-  const uint16_t* W;
-  uint16_t* C;
-  const uint16_t* bias;
-  int64_t ldx, ldw, ldc;
-  int M, N, K;
-  int vec_store;
-};
-int gemm_single_acc_quad_launch(const QuadArgs& a, hipStream_t stream);
 
 // How one problem is run.  Small grids are filled by cutting K into `split` aligned subtrees (one grid.y slice
 // each) whose bf16 partials meet in the shard tree afterwards -- the same arithmetic as tensor-parallel shards, so

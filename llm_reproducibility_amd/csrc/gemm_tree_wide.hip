@@ -21,21 +21,9 @@
 #include <type_traits>
 
 #include "common.h"
+#include "gemm_args.h"
 
 namespace tbik {
-
-struct WideArgs {
-  const uint16_t* X;   // [M,K], row stride ldx
-  const uint16_t* W;   // [N,K], row stride ldw
-  uint16_t* C;         // [M,N], row stride ldc
-  const uint16_t* bias;
-  u32x4* ws;           // parked tree levels: [level][tile][wave][chunk 0..7][lane]
-  int64_t ldx, ldw, ldc;
-  int M, N, K;
-  int T, flb, lb;
-  int vec_store;
-  int64_t k_shard, c_shard;  // K split over gridDim.y shards: operand column offset and partial-output offset per shard
-};
 
 namespace wide {
 constexpr int BM = 128, BN = 256, BK = 64;

@@ -102,7 +102,7 @@ class Qwen3Decoder:
             x = layer.o_proj(attn.reshape(-1, Hq * D))
             h, residual = rms_norm(x, layer.post_norm, cfg.rms_eps, residual=residual)
             gu = matmul_persistent(h, layer.gate_up_w.t())
-            act = ops.bi_silu_mul_bf16(gu)
+            act = ops.bi_silu_mul(gu)
             x = layer.down_proj(act)
         h, _ = rms_norm(x, self.final_norm, cfg.rms_eps, residual=residual)
         return h

@@ -98,7 +98,7 @@ def _weight_nk(B: torch.Tensor):
 # --------------------------------------------------------------------------------------------
 # tree-ordered GEMM
 # --------------------------------------------------------------------------------------------
-def _gemm_tree_bf16_impl(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.Tensor], leaf_k: int) -> torch.Tensor:
+def _gemm_tree_impl(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.Tensor], leaf_k: int) -> torch.Tensor:
     _require_gpu(A, B, bias)
     if A.dtype == torch.float32 and B.dtype == torch.float32 and (bias is None or bias.dtype == torch.float32):
         return _gemm_f32(A, B, bias, leaf_k, True)
@@ -119,21 +119,21 @@ def _gemm_tree_bf16_impl(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.
     return C
 
 
-_gemm_tree_bf16_op = torch.library.custom_op("tbik::gemm_tree_bf16", _gemm_tree_bf16_impl, mutates_args=(), device_types="cuda")
+_gemm_tree_op = torch.library.custom_op("tbik::gemm_tree", _gemm_tree_impl, mutates_args=(), device_types="cuda")
 
 
-def gemm_tree_bf16(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.Tensor], leaf_k: int) -> torch.Tensor:
+def gemm_tree(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.Tensor], leaf_k: int) -> torch.Tensor:
     if torch.compiler.is_compiling():
-        return _gemm_tree_bf16_op(A, B, bias, leaf_k)
-    return _gemm_tree_bf16_impl(A, B, bias, leaf_k)
+        return _gemm_tree_op(A, B, bias, leaf_k)
+    return _gemm_tree_impl(A, B, bias, leaf_k)
 
 
-@_gemm_tree_bf16_op.register_fake
+@_gemm_tree_op.register_fake
 def _(A, B, bias, leaf_k):
     return A.new_empty((A.shape[0], B.shape[1]))
 
 
-def _tree_combine_bf16_impl(parts: List[torch.Tensor]) -> torch.Tensor:
+def _tree_combine_impl(parts: List[torch.Tensor]) -> torch.Tensor:
     _require_gpu(*parts)
     ps = [p.contiguous() for p in parts]
     out = torch.empty_like(ps[0])
@@ -144,16 +144,16 @@ def _tree_combine_bf16_impl(parts: List[torch.Tensor]) -> torch.Tensor:
     return out
 
 
-_tree_combine_bf16_op = torch.library.custom_op("tbik::tree_combine_bf16", _tree_combine_bf16_impl, mutates_args=(), device_types="cuda")
+_tree_combine_op = torch.library.custom_op("tbik::tree_combine", _tree_combine_impl, mutates_args=(), device_types="cuda")
 
 
-def tree_combine_bf16(parts: List[torch.Tensor]) -> torch.Tensor:
+def tree_combine(parts: List[torch.Tensor]) -> torch.Tensor:
     if torch.compiler.is_compiling():
-        return _tree_combine_bf16_op(parts)
-    return _tree_combine_bf16_impl(parts)
+        return _tree_combine_op(parts)
+    return _tree_combine_impl(parts)
 
 
-@_tree_combine_bf16_op.register_fake
+@_tree_combine_op.register_fake
 def _(parts):
     return torch.empty_like(parts[0])
 
@@ -161,7 +161,7 @@ def _(parts):
 # --------------------------------------------------------------------------------------------
 # batch-invariant ops
 # --------------------------------------------------------------------------------------------
-def _bi_gemm_bf16_impl(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
+def _bi_gemm_impl(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
     _require_gpu(A, B, bias)
     if A.dtype == torch.float32 and B.dtype == torch.float32 and (bias is None or bias.dtype == torch.float32):
         return _gemm_f32(A, B, bias, 0, False)
@@ -180,25 +180,25 @@ def _bi_gemm_bf16_impl(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.Te
     L = _lib.lib()
     rc = (L.bi_gemm_f16 if _is_f16(A, B, bias) else L.bi_gemm_bf16)(a.data_ptr(), lda, w.data_ptr(), 1, ldw, C.data_ptr(), C.stride(0),
                                  M, N, K, None if b is None else b.data_ptr(), _stream(A))
-    _lib.check(rc, "bi_gemm_bf16")
+    _lib.check(rc, "bi_gemm")
     return C
 
 
-_bi_gemm_bf16_op = torch.library.custom_op("tbik::bi_gemm_bf16", _bi_gemm_bf16_impl, mutates_args=(), device_types="cuda")
+_bi_gemm_op = torch.library.custom_op("tbik::bi_gemm", _bi_gemm_impl, mutates_args=(), device_types="cuda")
 
 
-def bi_gemm_bf16(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
+def bi_gemm(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.Tensor]) -> torch.Tensor:
     if torch.compiler.is_compiling():
-        return _bi_gemm_bf16_op(A, B, bias)
-    return _bi_gemm_bf16_impl(A, B, bias)
+        return _bi_gemm_op(A, B, bias)
+    return _bi_gemm_impl(A, B, bias)
 
 
-@_bi_gemm_bf16_op.register_fake
+@_bi_gemm_op.register_fake
 def _(A, B, bias):
     return A.new_empty((A.shape[0], B.shape[1]))
 
 
-def _bi_rmsnorm_bf16_impl(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float) -> torch.Tensor:
+def _bi_rmsnorm_impl(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float) -> torch.Tensor:
     _require_gpu(x, weight)
     hidden = x.shape[-1]
     x2, ldx = _rows16(x.reshape(-1, hidden))
@@ -207,25 +207,25 @@ def _bi_rmsnorm_bf16_impl(x: torch.Tensor, weight: Optional[torch.Tensor], eps: 
     L = _lib.lib()
     rc = (L.bi_rmsnorm_f16 if _is_f16(x, weight) else L.bi_rmsnorm_bf16)(x2.data_ptr(), ldx, None, 0, None if w is None else w.data_ptr(),
                                     out.data_ptr(), out.stride(0), None, 0, x2.shape[0], hidden, eps, _stream(x))
-    _lib.check(rc, "bi_rmsnorm_bf16")
+    _lib.check(rc, "bi_rmsnorm")
     return out.reshape(x.shape)
 
 
-_bi_rmsnorm_bf16_op = torch.library.custom_op("tbik::bi_rmsnorm_bf16", _bi_rmsnorm_bf16_impl, mutates_args=(), device_types="cuda")
+_bi_rmsnorm_op = torch.library.custom_op("tbik::bi_rmsnorm", _bi_rmsnorm_impl, mutates_args=(), device_types="cuda")
 
 
-def bi_rmsnorm_bf16(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float) -> torch.Tensor:
+def bi_rmsnorm(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float) -> torch.Tensor:
     if torch.compiler.is_compiling():
-        return _bi_rmsnorm_bf16_op(x, weight, eps)
-    return _bi_rmsnorm_bf16_impl(x, weight, eps)
+        return _bi_rmsnorm_op(x, weight, eps)
+    return _bi_rmsnorm_impl(x, weight, eps)
 
 
-@_bi_rmsnorm_bf16_op.register_fake
+@_bi_rmsnorm_op.register_fake
 def _(x, weight, eps):
     return torch.empty_like(x)
 
 
-def _bi_add_rmsnorm_bf16_impl(x: torch.Tensor, residual: torch.Tensor, weight: Optional[torch.Tensor],
+def _bi_add_rmsnorm_impl(x: torch.Tensor, residual: torch.Tensor, weight: Optional[torch.Tensor],
                         eps: float) -> List[torch.Tensor]:
     _require_gpu(x, residual, weight)
     hidden = x.shape[-1]
@@ -238,21 +238,21 @@ def _bi_add_rmsnorm_bf16_impl(x: torch.Tensor, residual: torch.Tensor, weight: O
     rc = (L.bi_rmsnorm_f16 if _is_f16(x, residual, weight) else L.bi_rmsnorm_bf16)(x2.data_ptr(), ldx, r2.data_ptr(), ldr,
                                     None if w is None else w.data_ptr(), out.data_ptr(), out.stride(0),
                                     rout.data_ptr(), rout.stride(0), x2.shape[0], hidden, eps, _stream(x))
-    _lib.check(rc, "bi_rmsnorm_bf16")
+    _lib.check(rc, "bi_rmsnorm")
     return [out.reshape(x.shape), rout.reshape(x.shape)]
 
 
-_bi_add_rmsnorm_bf16_op = torch.library.custom_op("tbik::bi_add_rmsnorm_bf16", _bi_add_rmsnorm_bf16_impl, mutates_args=(), device_types="cuda")
+_bi_add_rmsnorm_op = torch.library.custom_op("tbik::bi_add_rmsnorm", _bi_add_rmsnorm_impl, mutates_args=(), device_types="cuda")
 
 
-def bi_add_rmsnorm_bf16(x: torch.Tensor, residual: torch.Tensor, weight: Optional[torch.Tensor],
+def bi_add_rmsnorm(x: torch.Tensor, residual: torch.Tensor, weight: Optional[torch.Tensor],
                         eps: float) -> List[torch.Tensor]:
     if torch.compiler.is_compiling():
-        return _bi_add_rmsnorm_bf16_op(x, residual, weight, eps)
-    return _bi_add_rmsnorm_bf16_impl(x, residual, weight, eps)
+        return _bi_add_rmsnorm_op(x, residual, weight, eps)
+    return _bi_add_rmsnorm_impl(x, residual, weight, eps)
 
 
-@_bi_add_rmsnorm_bf16_op.register_fake
+@_bi_add_rmsnorm_op.register_fake
 def _(x, residual, weight, eps):
     return [torch.empty_like(x), torch.empty_like(x)]
 
@@ -365,31 +365,31 @@ def _(q, k_cache, vt_cache, q_start, q_len, ctx_len, max_q_len, scale):
 # --------------------------------------------------------------------------------------------
 # gated activation in front of down_proj
 # --------------------------------------------------------------------------------------------
-def _bi_silu_mul_bf16_impl(gate_up: torch.Tensor) -> torch.Tensor:
+def _bi_silu_mul_impl(gate_up: torch.Tensor) -> torch.Tensor:
     _require_gpu(gate_up)
     f16 = _is_f16(gate_up)
     two_i = gate_up.shape[-1]
     if two_i % 16 != 0:
-        raise ValueError(f"bi_silu_mul_bf16: last dimension {two_i} must be a multiple of 16")
+        raise ValueError(f"bi_silu_mul: last dimension {two_i} must be a multiple of 16")
     inter = two_i // 2
     g2, ld = _rows16(gate_up.reshape(-1, two_i))
     out = torch.empty((g2.shape[0], inter), device=gate_up.device, dtype=gate_up.dtype)
     L = _lib.lib()
     rc = (L.bi_silu_mul_f16 if f16 else L.bi_silu_mul_bf16)(g2.data_ptr(), ld, out.data_ptr(), out.stride(0), g2.shape[0], inter, _stream(gate_up))
-    _lib.check(rc, "bi_silu_mul_bf16")
+    _lib.check(rc, "bi_silu_mul")
     return out.reshape(*gate_up.shape[:-1], inter)
 
 
-_bi_silu_mul_bf16_op = torch.library.custom_op("tbik::bi_silu_mul_bf16", _bi_silu_mul_bf16_impl, mutates_args=(), device_types="cuda")
+_bi_silu_mul_op = torch.library.custom_op("tbik::bi_silu_mul", _bi_silu_mul_impl, mutates_args=(), device_types="cuda")
 
 
-def bi_silu_mul_bf16(gate_up: torch.Tensor) -> torch.Tensor:
+def bi_silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
     """act = silu(gate_up[..., :I]) * gate_up[..., I:] (I = half the last dimension), fused, bf16."""
     if torch.compiler.is_compiling():
-        return _bi_silu_mul_bf16_op(gate_up)
-    return _bi_silu_mul_bf16_impl(gate_up)
+        return _bi_silu_mul_op(gate_up)
+    return _bi_silu_mul_impl(gate_up)
 
 
-@_bi_silu_mul_bf16_op.register_fake
+@_bi_silu_mul_op.register_fake
 def _(gate_up):
     return gate_up.new_empty((*gate_up.shape[:-1], gate_up.shape[-1] // 2))

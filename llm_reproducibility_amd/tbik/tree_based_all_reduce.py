@@ -40,7 +40,7 @@ def tree_combine(parts: Sequence[torch.Tensor]) -> torch.Tensor:
         return result[0] if n > 1 else result[0].clone()
     if parts[0].dtype not in (torch.bfloat16, torch.float16):
         raise NotImplementedError("tree_combine is implemented for bfloat16, float16 and float32 partials")
-    return ops.tree_combine_bf16(list(parts))
+    return ops.tree_combine(list(parts))
 
 
 def tree_all_reduce_sum_native(x: torch.Tensor, device_group=None) -> torch.Tensor:

@@ -47,4 +47,4 @@ def matmul_tp_persistent(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.
     assert K % leaf_k == 0, f"K={K} must be a multiple of the leaf size {leaf_k}"
     if bias is not None:
         assert bias.dim() == 1 and bias.shape[0] == B.shape[1] and bias.dtype == A.dtype
-    return ops.gemm_tree_bf16(A, B, bias, leaf_k)
+    return ops.gemm_tree(A, B, bias, leaf_k)

@@ -44,11 +44,11 @@ def test_fp16_rmsnorm_and_silu_mul(dev):
     for rows in (1, 7, 64):
         assert torch.equal(bio.rms_norm(x[:rows].to(dev), w.to(dev), 1e-6), got[:rows])
     gu = (torch.randn((65, 2 * 1024), generator=torch.Generator().manual_seed(2)) * 2).to(torch.float16)
-    act = ops.bi_silu_mul_bf16(gu.to(dev))
+    act = ops.bi_silu_mul(gu.to(dev))
     wa = O.silu_mul(gu)
     assert act.dtype == torch.float16
     assert ((act.cpu().float() - wa.float()).abs() <= 2.0 ** -9 * wa.float().abs().clamp_min(2.0 ** -6)).all()
-    assert torch.equal(ops.bi_silu_mul_bf16(gu[:3].to(dev)), act[:3])
+    assert torch.equal(ops.bi_silu_mul(gu[:3].to(dev)), act[:3])
 
 
 def test_add_rmsnorm_parity(dev):
@@ -191,21 +191,21 @@ def test_silu_mul_parity_and_batch_invariance(dev):
     g = torch.Generator().manual_seed(11)
     gu = (torch.randn((300, 2 * 12288), generator=g) * 2).to(torch.bfloat16)
     want = O.silu_mul(gu)
-    got = ops.bi_silu_mul_bf16(gu.to(dev))
+    got = ops.bi_silu_mul(gu.to(dev))
     assert got.shape == want.shape
     assert O.bf16_ulp_distance(got.cpu(), want).max().item() <= 1   # device exp vs host exp: at most one rounding flip
     for rows in (1, 7, 256):
-        assert torch.equal(ops.bi_silu_mul_bf16(gu[:rows].to(dev)), got[:rows])
+        assert torch.equal(ops.bi_silu_mul(gu[:rows].to(dev)), got[:rows])
     # a strided view (row stride larger than the row) and a 3-D input
     wide = torch.zeros((16, 2 * 256 + 64), dtype=torch.bfloat16)
     wide[:, :512] = gu[:16, :512]
-    assert torch.equal(ops.bi_silu_mul_bf16(wide.to(dev)[:, :512]).cpu(), ops.bi_silu_mul_bf16(gu[:16, :512].contiguous().to(dev)).cpu())
-    assert ops.bi_silu_mul_bf16(gu[:12, :64].reshape(3, 4, 64).to(dev)).shape == (3, 4, 32)
+    assert torch.equal(ops.bi_silu_mul(wide.to(dev)[:, :512]).cpu(), ops.bi_silu_mul(gu[:16, :512].contiguous().to(dev)).cpu())
+    assert ops.bi_silu_mul(gu[:12, :64].reshape(3, 4, 64).to(dev)).shape == (3, 4, 32)
     # exact cases: silu(0) * u = 0, silu(40) = 40
     z = torch.zeros((1, 16), dtype=torch.bfloat16)
     z[0, 1] = 40.0
     z[0, 8:] = 2.0
-    assert ops.bi_silu_mul_bf16(z.to(dev)).cpu().tolist() == [[0.0, 80.0, 0, 0, 0, 0, 0, 0]]
+    assert ops.bi_silu_mul(z.to(dev)).cpu().tolist() == [[0.0, 80.0, 0, 0, 0, 0, 0, 0]]
 
 
 def test_aten_overrides_route_to_the_hip_kernels(dev):
