@@ -243,6 +243,25 @@ int bi_silu_mul_bf16(const void* gate_up, int64_t ld_in,
                      int64_t rows, int inter,
                      tbik_stream_t stream);
 
+/*
+ * Caller side of bi_attention_bf16 for a Qwen3-style block: per-head RMSNorm of q and k (weights [128]), rotary
+ * embedding (rotate-half, angle = position * inv_freq[i], fp32), and the KV-cache write, for the fused projection
+ * output qkv [tokens, (q_heads + 2*kv_heads) * 128] (row stride ld):
+ *   q_out    [tokens, q_heads, 128]
+ *   k_cache  [batch, kv_heads, max_len, 128]   row (seq_of_token[t], h, positions[t]) is written
+ *   vt_cache [batch, kv_heads, 128, max_len]   column positions[t] is written
+ * positions / seq_of_token: device int64 [tokens].  One wavefront per (token, head): batch invariant.
+ * Replaces: the rotary-embedding patch of the alignment mode and the engine code around it,
+ *           src/patch/patch_training_inference_align.py:35-44; model wiring simple_rl.py:320-338 (qk_norm, head_dim 128).
+ */
+int bi_qk_norm_rope_cache_bf16(const void* qkv, int64_t ld,
+                               const void* q_weight, const void* k_weight,
+                               const float* inv_freq,
+                               const int64_t* positions, const int64_t* seq_of_token,
+                               void* q_out, void* k_cache, void* vt_cache,
+                               int64_t tokens, int q_heads, int kv_heads, int head_dim, int max_len, int batch,
+                               float eps, tbik_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -19,13 +19,17 @@ int attention_dispatch(const void* q, const void* k_cache, const void* vt_cache,
 int mean_dispatch(const void* x, void* out, int64_t outer, int64_t n, int64_t inner, int dtype_code, hipStream_t stream);
 int gemm_f32_dispatch(bool tree, const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C,
                       int64_t ldc, int M, int N, int K, int leaf_k, const void* bias, hipStream_t stream);
+int qk_norm_rope_cache_dispatch(const void* qkv, int64_t ld, const void* q_weight, const void* k_weight,
+                                const float* inv_freq, const int64_t* positions, const int64_t* seq_of_token, void* q_out,
+                                void* k_cache, void* vt_cache, int64_t tokens, int q_heads, int kv_heads, int head_dim,
+                                int max_len, int batch, float eps, hipStream_t stream);
 int silu_mul_dispatch(const void* gate_up, int64_t ld_in, void* out, int64_t ld_out, int64_t rows, int inter, bool f16,
                       hipStream_t stream);
 }  // namespace tbik
 
 extern "C" {
 
-int tbik_abi_version(void) { return 7; }
+int tbik_abi_version(void) { return 8; }
 
 const char* tbik_error_string(int code) {
   switch (code) {
@@ -141,6 +145,15 @@ int bi_silu_mul_bf16(const void* gate_up, int64_t ld_in, void* out, int64_t ld_o
 int bi_silu_mul_f16(const void* gate_up, int64_t ld_in, void* out, int64_t ld_out, int64_t rows, int inter,
                     tbik_stream_t stream) {
   return tbik::silu_mul_dispatch(gate_up, ld_in, out, ld_out, rows, inter, true, static_cast<hipStream_t>(stream));
+}
+
+int bi_qk_norm_rope_cache_bf16(const void* qkv, int64_t ld, const void* q_weight, const void* k_weight,
+                                const float* inv_freq, const int64_t* positions, const int64_t* seq_of_token, void* q_out,
+                                void* k_cache, void* vt_cache, int64_t tokens, int q_heads, int kv_heads, int head_dim,
+                                int max_len, int batch, float eps, tbik_stream_t stream) {
+  return tbik::qk_norm_rope_cache_dispatch(qkv, ld, q_weight, k_weight, inv_freq, positions, seq_of_token, q_out, k_cache,
+                                           vt_cache, tokens, q_heads, kv_heads, head_dim, max_len, batch, eps,
+                                           static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

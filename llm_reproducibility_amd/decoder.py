@@ -53,12 +53,14 @@ class _Layer:
 
 
 class Qwen3Decoder:
-    def __init__(self, cfg: DecoderConfig, tp_size: int = 1, seed: int = 0, device="cuda:0", use_graphs: bool = False):
+    def __init__(self, cfg: DecoderConfig, tp_size: int = 1, seed: int = 0, device="cuda:0", use_graphs: bool = False,
+                 fused_rope: bool = True):
         assert cfg.head_dim == 128, "the attention kernel is built for head_dim 128"
         self.cfg, self.tp_size, self.device = cfg, tp_size, torch.device(device)
         # decode steps replayed from one captured HIP graph (same kernels, same order, same bits as eager; the
         # per-step host work shrinks to one graph launch, which is what bounds small batches)
         self.use_graphs = use_graphs
+        self.fused_rope = fused_rope
         gen = torch.Generator().manual_seed(seed)
         emb = lambda *shape: (torch.randn(shape, generator=gen, dtype=torch.float32) * 0.02).to(torch.bfloat16).to(self.device)  # noqa: E731
         self.embed = emb(cfg.vocab_size, cfg.hidden_size)
@@ -90,14 +92,19 @@ class Qwen3Decoder:
             else:
                 h, residual = rms_norm(x, layer.input_norm, cfg.rms_eps, residual=residual)
             qkv = matmul_persistent(h, layer.qkv_w.t())
-            q = qkv[:, : Hq * D].reshape(-1, Hq, D)
-            k = qkv[:, Hq * D: (Hq + Hkv) * D].reshape(-1, Hkv, D)
-            v = qkv[:, (Hq + Hkv) * D:].reshape(-1, Hkv, D)
-            q = self._rope(rms_norm(q.contiguous(), layer.q_norm, cfg.rms_eps), positions)
-            k = self._rope(rms_norm(k.contiguous(), layer.k_norm, cfg.rms_eps), positions)
             k_cache, vt_cache = cache[li]
-            k_cache[seq_of_token, :, positions] = k                 # [tokens, Hkv, D] -> [B, Hkv, L, D]
-            vt_cache[seq_of_token, :, :, positions] = v             # stored transposed: [B, Hkv, D, L]
+            if self.fused_rope:
+                # per-head q/k norm, rotary embedding and the cache write in one kernel
+                q = ops.bi_qk_norm_rope_cache_bf16(qkv, layer.q_norm, layer.k_norm, self.inv_freq, positions, seq_of_token,
+                                                   k_cache, vt_cache, Hq, Hkv, cfg.rms_eps)
+            else:
+                q = qkv[:, : Hq * D].reshape(-1, Hq, D)
+                k = qkv[:, Hq * D: (Hq + Hkv) * D].reshape(-1, Hkv, D)
+                v = qkv[:, (Hq + Hkv) * D:].reshape(-1, Hkv, D)
+                q = self._rope(rms_norm(q.contiguous(), layer.q_norm, cfg.rms_eps), positions)
+                k = self._rope(rms_norm(k.contiguous(), layer.k_norm, cfg.rms_eps), positions)
+                k_cache[seq_of_token, :, positions] = k             # [tokens, Hkv, D] -> [B, Hkv, L, D]
+                vt_cache[seq_of_token, :, :, positions] = v         # stored transposed: [B, Hkv, D, L]
             attn = ops.bi_attention_bf16(q, k_cache, vt_cache, q_start, q_len, ctx_len, max_q_len, self.scale)
             x = layer.o_proj(attn.reshape(-1, Hq * D))
             h, residual = rms_norm(x, layer.post_norm, cfg.rms_eps, residual=residual)

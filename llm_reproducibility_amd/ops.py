@@ -393,3 +393,27 @@ def bi_silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
 @_bi_silu_mul_op.register_fake
 def _(gate_up):
     return gate_up.new_empty((*gate_up.shape[:-1], gate_up.shape[-1] // 2))
+
+
+# --------------------------------------------------------------------------------------------
+# q/k norm + rotary embedding + KV-cache write in front of the attention
+# --------------------------------------------------------------------------------------------
+def bi_qk_norm_rope_cache_bf16(qkv: torch.Tensor, q_weight: torch.Tensor, k_weight: torch.Tensor, inv_freq: torch.Tensor,
+                               positions: torch.Tensor, seq_of_token: torch.Tensor, k_cache: torch.Tensor,
+                               vt_cache: torch.Tensor, q_heads: int, kv_heads: int, eps: float) -> torch.Tensor:
+    """Writes this step's keys and values into the caches (in place) and returns the normed, rotated queries
+    [tokens, q_heads, 128]."""
+    _require_gpu(qkv, q_weight, k_weight, inv_freq, positions, seq_of_token, k_cache, vt_cache)
+    tokens = qkv.shape[0]
+    assert qkv.dtype == torch.bfloat16 and qkv.stride(1) == 1 and qkv.shape[1] == (q_heads + 2 * kv_heads) * 128
+    assert k_cache.is_contiguous() and vt_cache.is_contiguous() and k_cache.shape[1] == kv_heads and k_cache.shape[3] == 128
+    assert positions.dtype == torch.int64 and seq_of_token.dtype == torch.int64 and inv_freq.dtype == torch.float32
+    assert positions.numel() == tokens and seq_of_token.numel() == tokens and inv_freq.numel() == 64
+    q_out = torch.empty((tokens, q_heads, 128), device=qkv.device, dtype=torch.bfloat16)
+    rc = _lib.lib().bi_qk_norm_rope_cache_bf16(
+        qkv.data_ptr(), qkv.stride(0), q_weight.contiguous().data_ptr(), k_weight.contiguous().data_ptr(),
+        inv_freq.contiguous().data_ptr(), positions.contiguous().data_ptr(), seq_of_token.contiguous().data_ptr(),
+        q_out.data_ptr(), k_cache.data_ptr(), vt_cache.data_ptr(), tokens, q_heads, kv_heads, 128,
+        k_cache.shape[2], k_cache.shape[0], eps, _stream(qkv))
+    _lib.check(rc, "bi_qk_norm_rope_cache_bf16")
+    return q_out

@@ -119,6 +119,50 @@ def test_greedy_decode_is_identical_across_tp_and_batch(dev):
         del m
 
 
+def test_fused_qk_norm_rope_cache_matches_the_unfused_composition(dev):
+    from llm_reproducibility_amd.bio.batch_invariant_ops import rms_norm
+    from llm_reproducibility_amd.patch.patch_training_inference_align import compute_inv_freq
+    torch.manual_seed(2)
+    Hq, Hkv, D, B, L, T = 8, 2, 128, 3, 64, 37
+    qkv = torch.randn((T, (Hq + 2 * Hkv) * D), device=dev).to(torch.bfloat16)
+    qw = (1 + 0.1 * torch.randn(D, device=dev)).to(torch.bfloat16)
+    kw = (1 + 0.1 * torch.randn(D, device=dev)).to(torch.bfloat16)
+    inv = compute_inv_freq(D, 1e6, dev)
+    seq = torch.randint(0, B, (T,), device=dev)
+    pos = torch.stack([torch.randperm(L, device=dev)[:T] for _ in range(1)])[0]   # distinct positions: no write races
+    kc = torch.zeros((B, Hkv, L, D), dtype=torch.bfloat16, device=dev)
+    vt = torch.zeros((B, Hkv, D, L), dtype=torch.bfloat16, device=dev)
+    q = ops.bi_qk_norm_rope_cache_bf16(qkv, qw, kw, inv, pos, seq, kc, vt, Hq, Hkv, 1e-6)
+
+    def rope(x):
+        ang = pos.float()[:, None] * inv[None, :]
+        cos, sin = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+        xf = x.float()
+        a, b = xf[..., :64], xf[..., 64:]
+        return torch.cat((a * cos - b * sin, b * cos + a * sin), -1).to(torch.bfloat16)
+
+    q_ref = rope(rms_norm(qkv[:, : Hq * D].reshape(T, Hq, D).contiguous(), qw, 1e-6))
+    k_ref = rope(rms_norm(qkv[:, Hq * D: (Hq + Hkv) * D].reshape(T, Hkv, D).contiguous(), kw, 1e-6))
+    v_ref = qkv[:, (Hq + Hkv) * D:].reshape(T, Hkv, D)
+    tol = lambda got, want: ((got.float() - want.float()).abs() <= 2.0 ** -7 * want.float().abs().clamp_min(2.0 ** -5)).all()  # noqa: E731
+    assert tol(q, q_ref)
+    assert tol(kc[seq, :, pos], k_ref)
+    assert torch.equal(vt[seq, :, :, pos], v_ref)
+    # nothing else in the caches was touched
+    mask = torch.zeros((B, L), dtype=torch.bool, device=dev)
+    mask[seq, pos] = True
+    assert (kc.permute(0, 2, 1, 3)[~mask] == 0).all() and (vt.permute(0, 3, 1, 2)[~mask] == 0).all()
+    # row i alone == row i in the batch
+    kc1, vt1 = torch.zeros_like(kc), torch.zeros_like(vt)
+    q1 = ops.bi_qk_norm_rope_cache_bf16(qkv[5:6], qw, kw, inv, pos[5:6], seq[5:6], kc1, vt1, Hq, Hkv, 1e-6)
+    assert torch.equal(q1[0], q[5]) and torch.equal(kc1[seq[5], :, pos[5]], kc[seq[5], :, pos[5]])
+    # the decoder with and without the fused kernel: same tokens on a short run, logits within tolerance
+    prompts = _prompts(3, seed=9)
+    a = Qwen3Decoder(SMALL, tp_size=1, seed=0, device=dev, fused_rope=True).generate(prompts, 3, return_logits=True)
+    b = Qwen3Decoder(SMALL, tp_size=1, seed=0, device=dev, fused_rope=False).generate(prompts, 3, return_logits=True)
+    assert (a[1].float() - b[1].float()).abs().max() < 0.05 * b[1].float().abs().max()
+
+
 def test_graph_replayed_decode_steps_equal_eager_steps(dev):
     """Every replay of the captured decode step must give the eager step's bits (token ids and logits)."""
     prompts = _prompts(5, seed=7)
