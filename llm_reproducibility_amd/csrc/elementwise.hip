@@ -42,7 +42,9 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t* __restric
 
 int silu_mul_dispatch(const void* gate_up, int64_t ld_in, void* out, int64_t ld_out, int64_t rows, int inter, bool f16,
                       hipStream_t stream) {
-  if (!gate_up || !out || rows < 0 || inter <= 0 || ld_in < 2 * (int64_t)inter || ld_out < inter) return TBIK_ERR_INVALID;
+  if (rows < 0 || inter <= 0 || ld_in < 2 * (int64_t)inter || ld_out < inter) return TBIK_ERR_INVALID;
+  if (rows == 0 && !(inter & 7)) return TBIK_OK;
+  if (!gate_up || !out) return TBIK_ERR_INVALID;
   if ((inter & 7) || (ld_in & 7) || (ld_out & 7)) return TBIK_ERR_ALIGNMENT;
   if ((reinterpret_cast<uintptr_t>(gate_up) & 15) || (reinterpret_cast<uintptr_t>(out) & 15)) return TBIK_ERR_ALIGNMENT;
   if (rows == 0) return TBIK_OK;

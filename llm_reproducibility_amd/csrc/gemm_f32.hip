@@ -134,8 +134,9 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmF32Args p) {
 
 int gemm_f32_dispatch(bool tree, const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C,
                       int64_t ldc, int M, int N, int K, int leaf_k, const void* bias, hipStream_t stream) {
-  if (!A || !B || !C || M < 0 || N < 0 || K <= 0) return TBIK_ERR_INVALID;
+  if (M < 0 || N < 0 || K <= 0) return TBIK_ERR_INVALID;
   if (M == 0 || N == 0) return TBIK_OK;
+  if (!A || !B || !C) return TBIK_ERR_INVALID;
   if (ldb_k != 1) return TBIK_ERR_UNSUPPORTED;  // row-major [K,N] weights are repacked by the caller
   if (lda < K || ldb_n < K || ldc < N) return TBIK_ERR_INVALID;
   auto mis = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) != 0; };

@@ -387,8 +387,9 @@ size_t gemm_workspace_bytes(int M, int N, int K, int leaf_k, bool f16) {
 int gemm_dispatch(bool tree, bool f16, const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C,
                   int64_t ldc, int M, int N, int K, int leaf_k, const void* bias, void* ws, size_t ws_bytes,
                   hipStream_t stream) {
-  if (!A || !B || !C || M < 0 || N < 0 || K <= 0) return TBIK_ERR_INVALID;
-  if (M == 0 || N == 0) return TBIK_OK;
+  if (M < 0 || N < 0 || K <= 0) return TBIK_ERR_INVALID;
+  if (M == 0 || N == 0) return TBIK_OK;  // nothing to do (empty tensors may come with null pointers)
+  if (!A || !B || !C) return TBIK_ERR_INVALID;
   if (ldb_k != 1) return TBIK_ERR_UNSUPPORTED;  // row-major [K,N] weights are repacked by the caller
   if (lda < K || ldb_n < K || ldc < N) return TBIK_ERR_INVALID;
   if (!aligned16(A) || !aligned16(B) || (lda & 7) || (ldb_n & 7) || (K & 7)) return TBIK_ERR_ALIGNMENT;

@@ -102,7 +102,9 @@ static void rmsnorm_launch(const RmsArgs& a, int cpl, dim3 grid, hipStream_t str
 
 int rmsnorm_dispatch(const void* x, int64_t ldx, const void* res, int64_t ldr, const void* w, void* out, int64_t ldo,
                      void* res_out, int64_t ldro, int64_t rows, int hidden, float eps, bool f16, hipStream_t stream) {
-  if (!x || !out || rows < 0 || hidden <= 0) return TBIK_ERR_INVALID;
+  if (rows < 0 || hidden <= 0) return TBIK_ERR_INVALID;
+  if (rows == 0) return TBIK_OK;
+  if (!x || !out) return TBIK_ERR_INVALID;
   if (res && !res_out) return TBIK_ERR_INVALID;
   if (rows == 0) return TBIK_OK;
   if (hidden & 7) return TBIK_ERR_ALIGNMENT;
@@ -245,8 +247,9 @@ size_t lsm_workspace_bytes(int64_t rows, int64_t cols) {
 
 int log_softmax_dispatch(const void* x, int64_t ldx, void* out, int64_t ldo, int64_t rows, int64_t cols, void* ws,
                          size_t ws_bytes, int write_softmax, hipStream_t stream) {
-  if (!x || !out || rows < 0 || cols <= 0 || ldx < cols || ldo < cols) return TBIK_ERR_INVALID;
+  if (rows < 0 || cols <= 0 || ldx < cols || ldo < cols) return TBIK_ERR_INVALID;
   if (rows == 0) return TBIK_OK;
+  if (!x || !out) return TBIK_ERR_INVALID;
   if ((reinterpret_cast<uintptr_t>(x) & 3) || (reinterpret_cast<uintptr_t>(out) & 3)) return TBIK_ERR_ALIGNMENT;
   if (!ws || ws_bytes < lsm_workspace_bytes(rows, cols) || (reinterpret_cast<uintptr_t>(ws) & 3)) return TBIK_ERR_WORKSPACE;
   const int64_t segs = (cols + kSeg - 1) / kSeg;
@@ -363,8 +366,9 @@ static int mean_launch(const void* x, void* out, int64_t outer, int64_t n, int64
 }
 
 int mean_dispatch(const void* x, void* out, int64_t outer, int64_t n, int64_t inner, int dtype_code, hipStream_t stream) {
-  if (!x || !out || outer < 0 || n <= 0 || inner <= 0) return TBIK_ERR_INVALID;
+  if (outer < 0 || n <= 0 || inner <= 0) return TBIK_ERR_INVALID;
   if (outer == 0) return TBIK_OK;
+  if (!x || !out) return TBIK_ERR_INVALID;
   switch (dtype_code) {
     case 0: return mean_launch<float>(x, out, outer, n, inner, stream);
     case 1: return mean_launch<uint16_t>(x, out, outer, n, inner, stream);

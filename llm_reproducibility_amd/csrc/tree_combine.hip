@@ -94,9 +94,10 @@ static int launch_combine(const CombineArgs& a, bool vec_ok, hipStream_t stream)
 
 int tree_combine_bias_dispatch(const void* const* parts, int nparts, void* out, int64_t numel, const void* bias, int N,
                                bool f16, hipStream_t stream) {
-  if (!parts || !out || numel < 0 || (bias && N <= 0)) return TBIK_ERR_INVALID;
+  if (numel < 0 || (bias && N <= 0)) return TBIK_ERR_INVALID;
   if (nparts != 1 && nparts != 2 && nparts != 4 && nparts != 8) return TBIK_ERR_INVALID;
   if (numel == 0) return TBIK_OK;
+  if (!parts || !out) return TBIK_ERR_INVALID;
   CombineArgs a;
   bool vec_ok = (reinterpret_cast<uintptr_t>(out) & 15) == 0;
   if (reinterpret_cast<uintptr_t>(out) & 1) return TBIK_ERR_ALIGNMENT;

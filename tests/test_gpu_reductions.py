@@ -225,3 +225,19 @@ def test_aten_overrides_route_to_the_hip_kernels(dev):
     assert not bio.is_batch_invariant_mode_enabled()
     ref = torch.log_softmax(logits, -1)              # stock kernel again after leaving the mode
     assert (ref - bio.log_softmax(logits)).abs().max() < 1e-5
+
+
+def test_empty_inputs_are_handled_without_a_launch(dev):
+    from llm_reproducibility_amd import ops
+    from llm_reproducibility_amd.tbik import matmul_tp_persistent, tree_combine
+    w = O.gaussian_bf16((64, 512), 0.1, 1).to(dev)
+    e = torch.empty((0, 512), dtype=torch.bfloat16, device=dev)
+    assert matmul_tp_persistent(e, w.t()).shape == (0, 64)
+    assert bio.matmul_persistent(e, w.t()).shape == (0, 64)
+    assert bio.rms_norm(e, torch.ones(512, dtype=torch.bfloat16, device=dev), 1e-6).shape == (0, 512)
+    assert bio.log_softmax(torch.empty((0, 100), device=dev)).shape == (0, 100)
+    assert bio.mean_dim(torch.empty((0, 16), device=dev), -1).shape == (0,)
+    assert ops.bi_silu_mul(torch.empty((0, 64), dtype=torch.bfloat16, device=dev)).shape == (0, 32)
+    z = torch.empty((0, 8), dtype=torch.bfloat16, device=dev)
+    assert tree_combine([z, z]).shape == (0, 8)
+    torch.cuda.synchronize()
