@@ -33,6 +33,18 @@ struct QuadArgs {
 };
 int gemm_single_acc_quad_launch(const QuadArgs& a, hipStream_t stream);
 
+// gemm_single_acc_stream.hip: single-accumulator 16-bit GEMM for at most 64 rows, weights streamed from global memory
+struct StreamArgs {
+  const uint16_t* X;   // [M,K], row stride ldx
+  const uint16_t* W;   // [N,K], row stride ldw
+  uint16_t* C;         // [M,N], row stride ldc
+  const uint16_t* bias;
+  int64_t ldx, ldw, ldc;
+  int M, N, K;
+  int vec_store;
+};
+int gemm_single_acc_stream_launch(const StreamArgs& a, bool f16, hipStream_t stream);
+
 // tree_combine.hip
 int tree_combine_bias_dispatch(const void* const* parts, int nparts, void* out, int64_t numel, const void* bias, int N,
                                bool f16, hipStream_t stream);

@@ -1,0 +1,284 @@
+// Single-accumulator 16-bit GEMM for gfx950, decode-sized M (at most 64 rows): the batch-invariant aten::mm /
+// aten::addmm of the reference (matmul_persistent, src/bio/batch_invariant_ops.py:127-197) when the batch is a
+// handful of tokens and the call is one pass over the weight matrix.
+//
+// The accumulation contract of the batch-invariant mm forbids a split over K (one fp32 accumulator per element,
+// k ascending), so the only parallelism is over N.  Every wave therefore owns ONE strip of 16 weight rows (16
+// output columns, all M rows) and streams it straight from global memory into MFMA fragments -- a lane's 16
+// bytes ARE its fragment: row lane%16, k = 8*(lane/16)..+7 of the 32-wide step -- a whole window of 16 or 32
+// steps ahead, so that a few hundred independent waves keep enough bytes in flight to load the memory system.  The
+// activations are small and shared: the waves of a work-group (2 or 4 strips) stage each window of X in LDS once
+// (double-buffered, one barrier per window), which keeps the vector-memory queue of every wave for the weights.
+// With a handful of rows all of X is staged up front and the waves never meet again; work-groups shrink to one
+// or two strips when N is small, so that every CU gets some.  Same MFMA chain per element as the tiled and the
+// quad kernels, hence the same bits.
+#include "common.h"
+#include "gemm_args.h"
+
+namespace tbik {
+
+namespace stream {
+// LDS bytes per X row of a window of `ws` steps: 16 bytes of padding spread the 16 rows of a fragment read over all banks
+constexpr int rowb(int ws) { return ws * 64 + 16; }
+}  // namespace stream
+
+// Epilogue shared by the two kernels: lane (m = r, g) holds C[16 b + r][n0 + 4g .. 4g+3]; the bias joins in fp32
+// before the single rounding.
+template <int MB, bool F16>
+__device__ __forceinline__ void stream_store(const StreamArgs& p, const f32x4* acc, int n0, int r, int g) {
+  using Num = Num16<F16>;
+  const int n = n0 + 4 * g;
+  if (n >= p.N) return;
+  float bv[4] = {0.f, 0.f, 0.f, 0.f};
+  if (p.bias) {
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+      if (n + e < p.N) bv[e] = Num::to_f32(p.bias[n + e]);
+  }
+#pragma unroll
+  for (int b = 0; b < MB; b++) {
+    const int m = b * 16 + r;
+    if (m >= p.M) continue;
+    const uint32_t lo = Num::pack(acc[b][0] + bv[0], acc[b][1] + bv[1]);
+    const uint32_t hi = Num::pack(acc[b][2] + bv[2], acc[b][3] + bv[3]);
+    uint16_t* dst = p.C + (int64_t)m * p.ldc + n;
+    if (p.vec_store && n + 3 < p.N) {
+      *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);
+    } else {
+      const uint16_t v[4] = {(uint16_t)(lo & 0xffff), (uint16_t)(lo >> 16), (uint16_t)(hi & 0xffff), (uint16_t)(hi >> 16)};
+#pragma unroll
+      for (int e = 0; e < 4; e++)
+        if (n + e < p.N) dst[e] = v[e];
+    }
+  }
+}
+
+// A few rows (M * K small enough for LDS): all of X is staged once, one barrier, and then every wave runs on its
+// own -- nothing couples a wave's stream of weight loads to its neighbours'.
+constexpr int ROWS_U = 16;        // steps per register chunk (two chunks in flight)
+constexpr int ROWS_MAX_ELEMS = 32768;  // M * K at most: two rounds of staging loads in a work-group of 4 waves
+template <int NWAVES, bool F16>   // strips per work-group: 1 when N is small, so that every CU gets some
+__global__ __launch_bounds__(NWAVES * 64) void gemm_single_acc_stream_rows_kernel(const StreamArgs p) {
+  using Num = Num16<F16>;
+  constexpr int NW = NWAVES, NT = NWAVES * 64;
+  constexpr int U = ROWS_U;
+  extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // M rows of 2K + 16 bytes
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int n0 = (blockIdx.x * NW + wave) * 16;
+  const int r = lane & 15, g = lane >> 4;
+  const uint16_t* wp = p.W + (int64_t)min(n0 + r, p.N - 1) * p.ldw + 8 * g;
+  const int nsteps = p.K / 32;
+  const int nchunks = nsteps / U;
+  const int rowb = p.K * 2 + 16;
+
+  bf16x8 wa[U], wb[U];
+  auto load = [&](bf16x8* w, int c) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < U; u++) w[u] = *reinterpret_cast<const bf16x8*>(wp + (int64_t)(c * U + u) * 32);
+  };
+  if (nchunks > 0) load(wa, 0);  // the weights start flowing before X is staged
+
+  {
+    const int kc = p.K / 8, total = p.M * kc;
+    for (int base = 0; base < total; base += NT * 8) {  // one or two rounds of 8 loads in flight per thread
+      u32x4 xr[8];
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        const int q = base + tid + NT * i;
+        if (q < total) xr[i] = *reinterpret_cast<const u32x4*>(p.X + (int64_t)(q / kc) * p.ldx + (q % kc) * 8);
+      }
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        const int q = base + tid + NT * i;
+        if (q < total) *reinterpret_cast<u32x4*>(xs + (q / kc) * rowb + (q % kc) * 16) = xr[i];
+      }
+    }
+  }
+  __syncthreads();
+
+  f32x4 acc[1] = {f32x4{0.f, 0.f, 0.f, 0.f}};
+  const uint8_t* xrow = xs + min(r, p.M - 1) * rowb + g * 16;
+  auto mma = [&](const bf16x8* w, int c) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const bf16x8 x = *reinterpret_cast<const bf16x8*>(xrow + (c * U + u) * 64);
+      acc[0] = Num::mfma(w[u], x, acc[0]);
+    }
+  };
+  int c = 0;
+  for (; c + 2 <= nchunks; c += 2) {
+    load(wb, c + 1);
+    mma(wa, c);
+    if (c + 2 < nchunks) load(wa, c + 2);
+    mma(wb, c + 1);
+  }
+  if (c < nchunks) mma(wa, c);  // odd number of chunks: the last one is already in registers
+  for (int s = nchunks * U; s < nsteps; s++) {
+    const bf16x8 w = *reinterpret_cast<const bf16x8*>(wp + (int64_t)s * 32);
+    const bf16x8 x = *reinterpret_cast<const bf16x8*>(xrow + s * 64);
+    acc[0] = Num::mfma(w, x, acc[0]);
+  }
+  stream_store<1, F16>(p, acc, n0, r, g);
+}
+
+template <int MB, int WS, int NWAVES, bool F16>  // MB blocks of 16 activation rows, windows of WS steps (32 k each)
+__global__ __launch_bounds__(NWAVES * 64) void gemm_single_acc_stream_kernel(const StreamArgs p) {
+  using namespace stream;
+  using Num = Num16<F16>;
+  constexpr int NW = NWAVES, NT = NWAVES * 64;
+  constexpr int KW = WS * 32;
+  constexpr int ROWB = rowb(WS);
+  constexpr int ROWS = MB * 16;
+  constexpr int XBUF = ROWS * ROWB;
+  constexpr int XLD = ROWS * (KW / 8) / NT;  // 16-byte loads per thread per window: 4 * MB
+  extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // two X windows of XBUF bytes
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int n0 = (blockIdx.x * NW + wave) * 16;
+  const int r = lane & 15, g = lane >> 4;
+
+  const uint16_t* wp = p.W + (int64_t)min(n0 + r, p.N - 1) * p.ldw + 8 * g;
+
+  // staging of X: thread t moves 16-byte chunk q % (KW/8) of row q / (KW/8), q = t + 256 i, i < XLD
+  const uint16_t* xsrc[XLD];
+  uint32_t xdst[XLD];
+  int xk[XLD];
+#pragma unroll
+  for (int i = 0; i < XLD; i++) {
+    const int q = tid + NT * i;
+    const int row = q / (KW / 8), c = q % (KW / 8);
+    xsrc[i] = p.X + (int64_t)min(row, p.M - 1) * p.ldx + c * 8;
+    xdst[i] = row * ROWB + c * 16;
+    xk[i] = c * 8;
+  }
+  const int nsteps = p.K / 32;
+  const int nwin = (nsteps + WS - 1) / WS;
+
+  u32x4 xr[XLD];
+  bf16x8 wa[WS], wb[WS];
+  auto load_x = [&](int w) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < XLD; i++)
+      xr[i] = w * KW + xk[i] < p.K ? *reinterpret_cast<const u32x4*>(xsrc[i] + (int64_t)w * KW) : u32x4{0, 0, 0, 0};
+  };
+  auto store_x = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < XLD; i++) *reinterpret_cast<u32x4*>(xs + buf * XBUF + xdst[i]) = xr[i];
+  };
+  auto load_w = [&](bf16x8* w, int win) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < WS; u++) {
+      const int s = min(win * WS + u, nsteps - 1);  // past the end: a valid address, the step is not used
+      w[u] = *reinterpret_cast<const bf16x8*>(wp + (int64_t)s * 32);
+    }
+  };
+
+  f32x4 acc[MB];
+#pragma unroll
+  for (int b = 0; b < MB; b++) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const uint32_t xfrag = r * ROWB + g * 16;
+  auto compute = [&](const bf16x8* w, int win, int buf) __attribute__((always_inline)) {
+    const int left = nsteps - win * WS;  // steps of this window that exist (uniform)
+#pragma unroll
+    for (int u = 0; u < WS; u++) {
+      if (u < left) {
+#pragma unroll
+        for (int b = 0; b < MB; b++) {
+          const bf16x8 x = *reinterpret_cast<const bf16x8*>(xs + buf * XBUF + xfrag + b * 16 * ROWB + u * 64);
+          acc[b] = Num::mfma(w[u], x, acc[b]);
+        }
+      }
+    }
+  };
+
+  load_x(0);
+  load_w(wa, 0);
+  store_x(0);
+  __syncthreads();
+  for (int win = 0; win < nwin; win += 2) {
+    // even window: weights in wa, X in buffer 0
+    if (win + 1 < nwin) {
+      load_x(win + 1);
+      load_w(wb, win + 1);
+    }
+    compute(wa, win, 0);
+    if (win + 1 < nwin) store_x(1);
+    __syncthreads();
+    if (win + 1 >= nwin) break;
+    // odd window: weights in wb, X in buffer 1
+    if (win + 2 < nwin) {
+      load_x(win + 2);
+      load_w(wa, win + 2);
+    }
+    compute(wb, win + 1, 1);
+    if (win + 2 < nwin) store_x(0);
+    __syncthreads();
+  }
+
+  stream_store<MB, F16>(p, acc, n0, r, g);
+}
+
+template <int MB, int WS, int NWAVES, bool F16>
+static int stream_launch_nw(const StreamArgs& a, hipStream_t stream) {
+  const int64_t groups = ((int64_t)a.N + 16 * NWAVES - 1) / (16 * NWAVES);
+  if (groups > 0x7fffffff) return TBIK_ERR_INVALID;
+  constexpr int smem = 2 * MB * 16 * stream::rowb(WS);
+  auto kern = gemm_single_acc_stream_kernel<MB, WS, NWAVES, F16>;
+  if (smem > 64 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return hip_code(e);
+  }
+  hipLaunchKernelGGL(kern, dim3((unsigned)groups), dim3(NWAVES * 64), smem, stream, a);
+  return hip_code(hipGetLastError());
+}
+
+template <int MB, int WS, bool F16>
+static int stream_launch(const StreamArgs& a, hipStream_t stream) {
+  // few strips and few rows: two strips per work-group, so that more CUs take part
+  if (MB <= 2 && a.N <= 16 * 1024) return stream_launch_nw<MB, WS, (MB <= 2 ? 2 : 4), F16>(a, stream);
+  return stream_launch_nw<MB, WS, 4, F16>(a, stream);
+}
+
+template <int NWAVES, bool F16>
+static int stream_rows_launch(const StreamArgs& a, hipStream_t stream) {
+  const int64_t groups = ((int64_t)a.N + 16 * NWAVES - 1) / (16 * NWAVES);
+  if (groups > 0x7fffffff) return TBIK_ERR_INVALID;
+  const int smem = a.M * (a.K * 2 + 16);
+  hipLaunchKernelGGL((gemm_single_acc_stream_rows_kernel<NWAVES, F16>), dim3((unsigned)groups), dim3(NWAVES * 64), smem, stream, a);
+  return hip_code(hipGetLastError());
+}
+
+// Requires 0 < M <= 64 and K a multiple of 32 (checked by the dispatcher).
+int gemm_single_acc_stream_launch(const StreamArgs& a, bool f16, hipStream_t stream) {
+  if (a.M <= 0 || a.M > 64 || (a.K & 31) != 0) return TBIK_ERR_UNSUPPORTED;
+  // one block of rows, and all of X fits the staging registers of one pass and 40 KiB of LDS (several work-groups
+  // per CU)
+  if (a.M <= 16 && (int64_t)a.M * a.K <= ROWS_MAX_ELEMS && (int64_t)a.M * (a.K * 2 + 16) <= 40 * 1024) {
+    if (a.N <= 16 * 1024)  // at most 1024 strips: one per work-group spreads them over all CUs
+      return a.M * a.K <= ROWS_MAX_ELEMS / 4 ? (f16 ? stream_rows_launch<1, true>(a, stream) : stream_rows_launch<1, false>(a, stream))
+                                             : (f16 ? stream_rows_launch<4, true>(a, stream) : stream_rows_launch<4, false>(a, stream));
+    return f16 ? stream_rows_launch<4, true>(a, stream) : stream_rows_launch<4, false>(a, stream);
+  }
+  const int mb = (a.M + 15) / 16;
+  if (f16) {
+    switch (mb) {
+      case 1: return stream_launch<1, 16, true>(a, stream);
+      case 2: return stream_launch<2, 16, true>(a, stream);
+      case 3: return stream_launch<3, 16, true>(a, stream);
+      default: return stream_launch<4, 16, true>(a, stream);
+    }
+  }
+  switch (mb) {
+    case 1: return stream_launch<1, 16, false>(a, stream);
+    case 2: return stream_launch<2, 16, false>(a, stream);
+    case 3: return stream_launch<3, 16, false>(a, stream);
+    default: return stream_launch<4, 16, false>(a, stream);
+  }
+}
+
+}  // namespace tbik

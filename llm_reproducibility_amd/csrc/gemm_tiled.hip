@@ -420,6 +420,11 @@ int gemm_dispatch(bool tree, bool f16, const void* A, int64_t lda, const void* B
       QuadArgs qa{a.X, a.W, a.C, a.bias, a.ldx, a.ldw, a.ldc, M, N, K, a.vec_store};
       return gemm_single_acc_quad_launch(qa, stream);
     }
+    // a handful of rows: one pass over the weights, every 16x16 tile its own wave (same chain per element again)
+    if (M <= 64 && (K & 31) == 0) {
+      StreamArgs sa{a.X, a.W, a.C, a.bias, a.ldx, a.ldw, a.ldc, M, N, K, a.vec_store};
+      return gemm_single_acc_stream_launch(sa, f16, stream);
+    }
     return f16 ? launch_by_m<4, 0, false, true>(a, 1, stream) : launch_by_m<4, 0, false, false>(a, 1, stream);
   }
 

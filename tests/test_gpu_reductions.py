@@ -141,13 +141,31 @@ def test_single_accumulator_mm_large_and_small_kernels_agree_bitwise(dev):
     bias = O.gaussian_bf16((4096,), 1.0, 7)
     ad, wd, bd = a.to(dev), w.to(dev), bias.to(dev)
     full = bio.matmul_persistent(ad, wd.t(), bd)
-    for m in (1, 16, 64, 300):
+    for m in (1, 3, 16, 17, 33, 48, 64, 300):          # every row-block count of the streaming kernels, then the tiled one
         assert torch.equal(bio.matmul_persistent(ad[:m], wd.t(), bd), full[:m]), m
     want = O.matmul_single_acc(a[:256], w.t(), bias)
     assert not O.outside_tolerance(full[:256], want).any()
     ai = O.integer_bf16((2048, 512), -9, 9, 8)
     wi = O.integer_bf16((4096, 512), -7, 7, 9)
     assert torch.equal(bio.matmul_persistent(ai.to(dev), wi.to(dev).t()).cpu(), O.matmul_single_acc(ai, wi.t()))
+
+
+def test_single_accumulator_mm_streaming_kernels_on_ragged_shapes(dev):
+    # K = 35 steps of 32 (two whole windows and a partial one), N ends inside a 16-wide strip, strided A, bias
+    ai = O.integer_bf16((40, 1200), -9, 9, 11)[:, :1120]
+    wi = O.integer_bf16((72 + 8, 1120), -7, 7, 12)[:72]
+    bi = O.integer_bf16((72,), -5, 5, 13)
+    want = O.matmul_single_acc(ai, wi.t(), bi)
+    for m in (1, 2, 5, 16, 23, 40):
+        got = bio.matmul_persistent(ai[:m].to(dev)[:, :], wi.to(dev).t(), bi.to(dev))
+        assert torch.equal(got.cpu(), want[:m]), m
+    a_strided = O.integer_bf16((40, 1200), -9, 9, 11).to(dev)[:, :1120]
+    assert not a_strided.is_contiguous()
+    assert torch.equal(bio.matmul_persistent(a_strided[:5], wi.to(dev).t(), bi.to(dev)).cpu(), want[:5])
+    # long K for a single row (the whole-X kernel stages up to 32768 activations)
+    a1 = O.integer_bf16((2, 16384), -3, 3, 14)
+    w1 = O.integer_bf16((48, 16384), -3, 3, 15)
+    assert torch.equal(bio.matmul_persistent(a1.to(dev), w1.to(dev).t()).cpu(), O.matmul_single_acc(a1, w1.t()))
 
 
 def test_single_accumulator_mm_fp16(dev):
