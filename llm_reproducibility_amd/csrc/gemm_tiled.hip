@@ -104,9 +104,15 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
     wptr[i] = Ws + (int64_t)gr * p.ldw + c * 8;
     wdst[i] = lds_off(r, c);
   }
-  u32x4 xreg[XCH], wreg[WCH];
+  // Staging registers.  The tree kernel loads one stage ahead; the single-accumulator mm (no K split, so often a
+  // small grid in which every work-group is a chain of memory round trips) loads two stages ahead into two
+  // register sets that alternate with the parity of the stage.
+  constexpr int NSET = TREE ? 1 : 2;
+  u32x4 xregs[NSET][XCH], wregs[NSET][WCH];
 
-  auto load_stage = [&](int s) __attribute__((always_inline)) {
+  auto load_stage = [&](int s, int set) __attribute__((always_inline)) {
+    u32x4* xreg = xregs[set];
+    u32x4* wreg = wregs[set];
     const int k0 = s * BK;
 #pragma unroll
     for (int i = 0; i < XCH; i++) {
@@ -127,7 +133,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
       }
     }
   };
-  auto store_stage = [&](int buf) __attribute__((always_inline)) {
+  auto store_stage = [&](int buf, int set) __attribute__((always_inline)) {
+    const u32x4* xreg = xregs[set];
+    const u32x4* wreg = wregs[set];
 #pragma unroll
     for (int i = 0; i < XCH; i++)
       if ((BM * 8) % NT == 0 || tid + i * NT < BM * 8) *reinterpret_cast<u32x4*>(smem + buf * STAGE + xdst[i]) = xreg[i];
@@ -150,8 +158,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
   const int nstages = TREE ? p.T * LS : (p.K + BK - 1) / BK;
   const int nouter = TREE ? p.T : (nstages + LS - 1) / LS;
 
-  load_stage(0);
-  store_stage(0);
+  load_stage(0, 0);
+  if (!TREE) load_stage(min(1, nstages - 1), 1);
+  store_stage(0, 0);
   __syncthreads();
 
   for (int j = 0; j < nouter; j++) {
@@ -161,7 +170,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
       if (TREE || s < nstages) {
         // the stage after the last one re-reads the last one into the idle buffer: harmless, and it
         // keeps the staging registers free of control flow
-        load_stage(min(s + 1, nstages - 1));
+        if (TREE) load_stage(min(s + 1, nstages - 1), 0);
+        else load_stage(min(s + 2, nstages - 1), i & 1);  // the set that held stage s, stored a stage ago
         const uint16_t* bx = smem + (s & 1) * STAGE;
         const uint16_t* bw = bx + BM * BK;
 #pragma unroll
@@ -186,7 +196,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
               acc[a][b] = Num::mfma(fw[b], fx[a], fresh ? zero : acc[a][b]);
             }
         }
-        store_stage((s + 1) & 1);
+        store_stage((s + 1) & 1, TREE ? 0 : (i + 1) & 1);
         __syncthreads();
       }
     }
@@ -312,6 +322,12 @@ template <int LS, int LBMAX, bool TREE, bool F16>
 static int launch_by_m(const GemmArgs& a, int split, hipStream_t stream) {
   if (a.M <= 16) return launch<1, 4, 1, 1, LS, LBMAX, TREE, F16>(a, split, stream);
   if (a.M <= 64) return launch<1, 4, 4, 2, LS, LBMAX, TREE, F16>(a, split, stream);
+  // without a split over K (the single-accumulator mm) a small grid of 128x128 tiles leaves CUs idle: 64x128 tiles
+  // double the work-groups (the choice cannot change any bit: the chain per element is the same)
+  if (!TREE && (int64_t)((a.M + 127) / 128) * ((a.N + 127) / 128) < 256) {
+    if ((int64_t)((a.M + 63) / 64) * ((a.N + 127) / 128) < 256) return launch<1, 4, 4, 1, LS, LBMAX, TREE, F16>(a, split, stream);
+    return launch<1, 4, 4, 2, LS, LBMAX, TREE, F16>(a, split, stream);
+  }
   return launch<2, 2, 4, 4, LS, LBMAX, TREE, F16>(a, split, stream);
 }
 

@@ -37,22 +37,43 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const RmsArgs a) {
   const uint4* xr = reinterpret_cast<const uint4*>(a.x + row * a.ldx);
   const uint4* rr = a.res ? reinterpret_cast<const uint4*>(a.res + row * a.ldr) : nullptr;
 
+  // the weights do not depend on the row: fetched together with it, not after the reduction (with a single row
+  // the kernel is nothing but memory round trips in a chain)
+  const uint4* wr = reinterpret_cast<const uint4*>(a.w);
+  uint4 wq[CPL];
+  if (wr) {
+#pragma unroll
+    for (int i = 0; i < CPL; i++) {
+      const int c = lane + 64 * i;
+      if (c < nchunks) wq[i] = wr[c];
+    }
+  }
+
+  // all loads of the row go out before the first store: the residual output may alias the inputs as far as the
+  // compiler knows, and loads issued behind a store would wait for one memory round trip per chunk
+  uint4 xq[CPL], rq[CPL];
+#pragma unroll
+  for (int i = 0; i < CPL; i++) {
+    const int c = lane + 64 * i;
+    if (c < nchunks) {
+      xq[i] = xr[c];
+      if (rr) rq[i] = rr[c];
+    }
+  }
   float v[CPL][8];
   float ss = 0.f;
 #pragma unroll
   for (int i = 0; i < CPL; i++) {
     const int c = lane + 64 * i;
     if (c < nchunks) {
-      const uint4 q = xr[c];
-      const uint32_t u[4] = {q.x, q.y, q.z, q.w};
+      const uint32_t u[4] = {xq[i].x, xq[i].y, xq[i].z, xq[i].w};
 #pragma unroll
       for (int e = 0; e < 4; e++) {
         v[i][2 * e] = Num::lo(u[e]);
         v[i][2 * e + 1] = Num::hi(u[e]);
       }
       if (rr) {
-        const uint4 r = rr[c];
-        const uint32_t ru[4] = {r.x, r.y, r.z, r.w};
+        const uint32_t ru[4] = {rq[i].x, rq[i].y, rq[i].z, rq[i].w};
         uint32_t so[4];
 #pragma unroll
         for (int e = 0; e < 4; e++) {
@@ -69,7 +90,6 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const RmsArgs a) {
   ss = wave_sum(ss);
   const float var = ss / (float)a.hidden;
   const float rs = 1.0f / sqrtf(var + a.eps);
-  const uint4* wr = reinterpret_cast<const uint4*>(a.w);
   uint4* orow = reinterpret_cast<uint4*>(a.out + row * a.ldo);
 #pragma unroll
   for (int i = 0; i < CPL; i++) {
@@ -79,8 +99,7 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const RmsArgs a) {
 #pragma unroll
       for (int e = 0; e < 4; e++) o[e] = Num::pack(v[i][2 * e] * rs, v[i][2 * e + 1] * rs);
       if (wr) {
-        const uint4 wq = wr[c];
-        const uint32_t wu[4] = {wq.x, wq.y, wq.z, wq.w};
+        const uint32_t wu[4] = {wq[i].x, wq[i].y, wq[i].z, wq[i].w};
 #pragma unroll
         for (int e = 0; e < 4; e++)
           o[e] = Num::pack(Num::lo(o[e]) * Num::lo(wu[e]), Num::hi(o[e]) * Num::hi(wu[e]));
