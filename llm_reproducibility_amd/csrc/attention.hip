@@ -143,7 +143,7 @@ __global__ __launch_bounds__(64) void attention_kernel(const AttnArgs a) {
 // is exactly that of attention_kernel above, so both kernels produce the same bits; this one just moves 1/G of
 // the bytes and hides the load latency behind the previous tile.
 // ------------------------------------------------------------------------------------------------
-template <int G>
+template <int G, bool DEEP>
 __global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs a) {
   __shared__ __attribute__((aligned(16))) uint8_t lds[2][16384];  // per buffer: K tile [32][128] (8 KiB), V^T tile [128][32] (8 KiB)
   const int b = blockIdx.z;
@@ -173,8 +173,14 @@ __global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs 
   // cooperative staging: 512 16-byte chunks per tile and operand, NCH per thread
   constexpr int NT = 64 * G;
   constexpr int NCH = (512 + NT - 1) / NT;
-  u32x4 kreg[NCH], vreg[NCH];
-  auto load_tile = [&](int tile) __attribute__((always_inline)) {
+  // Key tiles are fetched DEPTH tiles ahead into DEPTH register sets (set = tile % DEPTH).  DEEP is for decode: a
+  // single block of queries per sequence makes the kernel a chain of memory round trips, and one tile of arithmetic
+  // hides none of them.  Prefill has arithmetic to overlap and prefers the registers (more waves per SIMD).
+  constexpr int DEPTH = !DEEP ? 1 : (NCH <= 2 ? 4 : (NCH <= 4 ? 2 : 1));
+  u32x4 kregs[DEPTH][NCH], vregs[DEPTH][NCH];
+  auto load_tile = [&](int tile, int set) __attribute__((always_inline)) {
+    u32x4* kreg = kregs[set];
+    u32x4* vreg = vregs[set];
     const int k0 = min(tile * 32, a.max_len - 32);  // max_len is a multiple of 32: never past the cache
 #pragma unroll
     for (int i = 0; i < NCH; i++) {
@@ -185,7 +191,9 @@ __global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs 
       }
     }
   };
-  auto store_tile = [&](int buf) __attribute__((always_inline)) {
+  auto store_tile = [&](int buf, int set) __attribute__((always_inline)) {
+    const u32x4* kreg = kregs[set];
+    const u32x4* vreg = vregs[set];
 #pragma unroll
     for (int i = 0; i < NCH; i++) {
       const int ch = tid + i * NT;
@@ -205,12 +213,18 @@ __global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs 
   float l = 0.f;
 
   const int ntiles = last_pos / 32 + 1;
-  load_tile(0);
-  store_tile(0);
+#pragma unroll
+  for (int d = 0; d < DEPTH; d++)
+    if (d < ntiles) load_tile(d, d);
+  store_tile(0, 0);
   __syncthreads();
-  for (int tile = 0; tile < ntiles; tile++) {
+  for (int t0 = 0; t0 < ntiles; t0 += DEPTH) {
+#pragma unroll
+   for (int d = 0; d < DEPTH; d++) {
+    const int tile = t0 + d;
+    if (tile >= ntiles) break;
     const int cur = tile & 1;
-    if (tile + 1 < ntiles) load_tile(tile + 1);
+    if (tile + DEPTH < ntiles) load_tile(tile + DEPTH, d);  // set d held this tile and went to LDS a tile ago
     const int k0 = tile * 32;
     f32x4 s[2];
 #pragma unroll
@@ -263,8 +277,9 @@ __global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs 
       f32x4 scaled = {o[t][0] * alpha, o[t][1] * alpha, o[t][2] * alpha, o[t][3] * alpha};
       o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, scaled, 0, 0, 0);
     }
-    if (tile + 1 < ntiles) store_tile(cur ^ 1);
+    if (tile + 1 < ntiles) store_tile(cur ^ 1, (d + 1) % DEPTH);
     __syncthreads();
+   }
   }
   if (!qvalid) return;
   const float inv = 1.0f / l;
@@ -294,10 +309,14 @@ int attention_dispatch(const void* q, const void* k_cache, const void* vt_cache,
   const bool grouped = (max_len & 31) == 0 && (G == 1 || G == 2 || G == 4 || G == 8) && kv_heads <= 65535;
   if (grouped) {
     const dim3 grid((unsigned)((max_q_len + 15) / 16), (unsigned)kv_heads, (unsigned)batch);
-    if (G == 1) hipLaunchKernelGGL(attention_group_kernel<1>, grid, dim3(64), 0, stream, a);
-    else if (G == 2) hipLaunchKernelGGL(attention_group_kernel<2>, grid, dim3(128), 0, stream, a);
-    else if (G == 4) hipLaunchKernelGGL(attention_group_kernel<4>, grid, dim3(256), 0, stream, a);
-    else hipLaunchKernelGGL(attention_group_kernel<8>, grid, dim3(512), 0, stream, a);
+    const bool deep = max_q_len <= 16;  // decode: one block of queries per sequence
+    if (G == 1) hipLaunchKernelGGL((attention_group_kernel<1, false>), grid, dim3(64), 0, stream, a);
+    else if (G == 2 && deep) hipLaunchKernelGGL((attention_group_kernel<2, true>), grid, dim3(128), 0, stream, a);
+    else if (G == 2) hipLaunchKernelGGL((attention_group_kernel<2, false>), grid, dim3(128), 0, stream, a);
+    else if (G == 4 && deep) hipLaunchKernelGGL((attention_group_kernel<4, true>), grid, dim3(256), 0, stream, a);
+    else if (G == 4) hipLaunchKernelGGL((attention_group_kernel<4, false>), grid, dim3(256), 0, stream, a);
+    else if (deep) hipLaunchKernelGGL((attention_group_kernel<8, true>), grid, dim3(512), 0, stream, a);
+    else hipLaunchKernelGGL((attention_group_kernel<8, false>), grid, dim3(512), 0, stream, a);
   } else {
     const dim3 grid((unsigned)((max_q_len + 15) / 16), (unsigned)q_heads, (unsigned)batch);
     hipLaunchKernelGGL(attention_kernel, grid, dim3(64), 0, stream, a);
