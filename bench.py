@@ -91,7 +91,10 @@ def table(steps, warmup):
         gemm_row(f"o_proj 32B    M={M} K=8192 N=5120", M, 8192, 5120, 256)
     for M in (1, 64, 512, 4096):
         gemm_row(f"down_proj 32B M={M} K=25600 N=5120 leaf128", M, 25600, 5120, choose_leaf_k(25600))
-    for name, M, K, N in (("qkv 8B", 2048, 4096, 6144), ("gate_up 8B", 2048, 4096, 24576), ("lm_head 8B", 128, 4096, 151936)):
+    for name, M, K, N in (("qkv 8B", 2048, 4096, 6144), ("gate_up 8B", 2048, 4096, 24576), ("lm_head 8B", 128, 4096, 151936),
+                          ("qkv 8B", 1, 4096, 6144), ("qkv 8B", 32, 4096, 6144), ("qkv 8B", 128, 4096, 6144),
+                          ("gate_up 8B", 1, 4096, 24576), ("gate_up 8B", 32, 4096, 24576), ("gate_up 8B", 128, 4096, 24576),
+                          ("lm_head 8B", 1, 4096, 151936), ("lm_head 8B", 32, 4096, 151936)):
         X = torch.randn((M, K), device=dev).to(torch.bfloat16)
         W = (torch.randn((N, K), device=dev) * 0.02).to(torch.bfloat16)
         ms, _ = hip_time_ms(lambda: bio.matmul_persistent(X, W.t()), steps, warmup)
