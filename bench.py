@@ -26,7 +26,7 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # FETCH_SIZE 256,867 KiB x 1.999 (a plain copy of 49,152 KiB reads 24,592) + WRITE_SIZE 131,072 KiB x 1.000;
 # profiles/gemm_tree_wide_headline_counters.txt holds the runs.  Algorithmic bytes are 167.8 MB: the rest is the
 # seven parked tree levels (written and read back once each) and one operand fetch per XCD-local L2.
-TRAFFIC_BYTES_PER_LAUNCH = 659.9e6
+TRAFFIC_BYTES_PER_LAUNCH = 662.3e6
 
 
 def hip_time_ms(fn, steps, warmup):

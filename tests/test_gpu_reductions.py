@@ -135,7 +135,7 @@ def test_single_accumulator_mm_parity_and_batch_invariance(dev):
 
 
 def test_single_accumulator_mm_large_and_small_kernels_agree_bitwise(dev):
-    # M=2048 takes the wide pipeline, M<=64 the small-tile kernel: same MFMA chain per element, same bits
+    # M=2048 takes the wide pipeline, M<=64 the streaming kernels, M=300 the tiled one: same MFMA chain per element, same bits
     a = O.gaussian_bf16((2048, 1024), 1.0, 5)
     w = O.gaussian_bf16((4096, 1024), 0.05, 6)
     bias = O.gaussian_bf16((4096,), 1.0, 7)
