@@ -148,7 +148,9 @@ __global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs 
   __shared__ __attribute__((aligned(16))) uint8_t lds[2][16384];  // per buffer: K tile [32][128] (8 KiB), V^T tile [128][32] (8 KiB)
   const int b = blockIdx.z;
   const int kvh = blockIdx.y;
-  const int qb = blockIdx.x;
+  // causal attention: the last query blocks have the most keys, so they are dispatched first (longest work first
+  // keeps the tail of the launch short); which work-group computes a block has no numeric effect
+  const int qb = gridDim.x - 1 - blockIdx.x;
   const int qlen = a.q_len[b];
   if (qb * 16 >= qlen) return;  // uniform over the work-group
   const int tid = threadIdx.x;
