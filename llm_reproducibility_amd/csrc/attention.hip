@@ -92,8 +92,8 @@ __global__ __launch_bounds__(64) void attention_kernel(const AttnArgs a) {
         sv[4 * u + i] = v;
         tmax = fmaxf(tmax, v);
       }
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    tmax = xor_step<16, LaneMax>(tmax);
+    tmax = xor_step<32, LaneMax>(tmax);
     const float m_new = fmaxf(m, tmax);          // key 0 is visible to every query: m_new is finite from tile 0 on
     const float alpha = exp2f(m - m_new);         // exactly 1.0 when the tile adds nothing new
     float psum = 0.f;
@@ -103,8 +103,8 @@ __global__ __launch_bounds__(64) void attention_kernel(const AttnArgs a) {
       pv[e] = exp2f(sv[e] - m_new);
       psum += pv[e];
     }
-    psum += __shfl_xor(psum, 16, 64);
-    psum += __shfl_xor(psum, 32, 64);
+    psum = xor_step<16, LaneSum>(psum);
+    psum = xor_step<32, LaneSum>(psum);
     l = l * alpha + psum;
     m = m_new;
     // P as the MFMA "B" operand: k slots 0..3 = keys k0+4g.., slots 4..7 = keys k0+16+4g..
@@ -215,9 +215,10 @@ __global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs 
   float l = 0.f;
 
   const int ntiles = last_pos / 32 + 1;
+  // loads past the last tile are clamped to a valid address and never used: issuing them unconditionally keeps the
+  // number of loads in flight static, so the waits below can leave the newer tiles in flight
 #pragma unroll
-  for (int d = 0; d < DEPTH; d++)
-    if (d < ntiles) load_tile(d, d);
+  for (int d = 0; d < DEPTH; d++) load_tile(d, d);
   store_tile(0, 0);
   __syncthreads();
   for (int t0 = 0; t0 < ntiles; t0 += DEPTH) {
@@ -226,7 +227,7 @@ __global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs 
     const int tile = t0 + d;
     if (tile >= ntiles) break;
     const int cur = tile & 1;
-    if (tile + DEPTH < ntiles) load_tile(tile + DEPTH, d);  // set d held this tile and went to LDS a tile ago
+    load_tile(tile + DEPTH, d);  // set d held this tile and went to LDS a tile ago
     const int k0 = tile * 32;
     f32x4 s[2];
 #pragma unroll
@@ -251,8 +252,8 @@ __global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs 
         sv[4 * u + i] = v;
         tmax = fmaxf(tmax, v);
       }
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    tmax = xor_step<16, LaneMax>(tmax);
+    tmax = xor_step<32, LaneMax>(tmax);
     const float m_new = fmaxf(m, tmax);
     const float alpha = exp2f(m - m_new);
     float psum = 0.f;
@@ -262,8 +263,8 @@ __global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs 
       pv[e] = exp2f(sv[e] - m_new);
       psum += pv[e];
     }
-    psum += __shfl_xor(psum, 16, 64);
-    psum += __shfl_xor(psum, 32, 64);
+    psum = xor_step<16, LaneSum>(psum);
+    psum = xor_step<32, LaneSum>(psum);
     l = l * alpha + psum;
     m = m_new;
     const uint32_t p0 = pack_bf16x2(pv[0], pv[1]), p1 = pack_bf16x2(pv[2], pv[3]);

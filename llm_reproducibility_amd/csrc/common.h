@@ -76,16 +76,43 @@ struct Num16<true> {
 
 // Butterfly reductions over the 64 lanes of a wavefront.  The exchange pattern is fixed, so the
 // association order of the sum is a constant of the kernel: it cannot depend on the launch.
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
-  return v;
+// One step combines every lane with lane ^ OFF.  The partner's value travels through VALU cross-lane moves
+// (v_permlane32_swap / v_permlane16_swap for 32 and 16, DPP row rotate / quad permute for 8, 2 and 1) instead of
+// an LDS permute (__shfl_xor), which costs a round trip through the LDS crossbar per step; only the step of 4 has
+// no such move and keeps the permute.  Both operands of a step are the same pair as with __shfl_xor and the
+// operations are commutative, so the bits do not change.
+struct LaneSum { static __device__ __forceinline__ float f(float a, float b) { return a + b; } };
+struct LaneMax { static __device__ __forceinline__ float f(float a, float b) { return fmaxf(a, b); } };
+template <int OFF, typename Op>
+__device__ __forceinline__ float xor_step(float v) {
+  const uint32_t u = __builtin_bit_cast(uint32_t, v);
+  if (OFF == 32) {
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return Op::f(as_f32(r[0]), as_f32(r[1]));
+  } else if (OFF == 16) {
+    const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    return Op::f(as_f32(r[0]), as_f32(r[1]));
+  } else if (OFF == 8) {
+    return Op::f(v, as_f32(__builtin_amdgcn_update_dpp(0u, u, 0x128, 0xf, 0xf, false)));  // row_ror:8
+  } else if (OFF == 2) {
+    return Op::f(v, as_f32(__builtin_amdgcn_update_dpp(0u, u, 0x4e, 0xf, 0xf, false)));   // quad_perm [2,3,0,1]
+  } else if (OFF == 1) {
+    return Op::f(v, as_f32(__builtin_amdgcn_update_dpp(0u, u, 0xb1, 0xf, 0xf, false)));   // quad_perm [1,0,3,2]
+  } else {
+    return Op::f(v, __shfl_xor(v, OFF, kWave));
+  }
 }
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
-  return v;
+template <typename Op>
+__device__ __forceinline__ float wave_reduce(float v) {
+  v = xor_step<32, Op>(v);
+  v = xor_step<16, Op>(v);
+  v = xor_step<8, Op>(v);
+  v = xor_step<4, Op>(v);
+  v = xor_step<2, Op>(v);
+  return xor_step<1, Op>(v);
 }
+__device__ __forceinline__ float wave_sum(float v) { return wave_reduce<LaneSum>(v); }
+__device__ __forceinline__ float wave_max(float v) { return wave_reduce<LaneMax>(v); }
 
 inline int hip_code(hipError_t e) { return e == hipSuccess ? TBIK_OK : TBIK_ERR_HIP_BASE + (int)e; }
 
