@@ -104,10 +104,11 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
     wptr[i] = Ws + (int64_t)gr * p.ldw + c * 8;
     wdst[i] = lds_off(r, c);
   }
-  // Staging registers.  The tree kernel loads one stage ahead; the single-accumulator mm (no K split, so often a
-  // small grid in which every work-group is a chain of memory round trips) loads two stages ahead into two
-  // register sets that alternate with the parity of the stage.
-  constexpr int NSET = TREE ? 1 : 2;
+  // Staging registers.  Large tree tiles load one stage ahead (their merge stack needs the registers); the
+  // single-accumulator mm (no K split, so often a small grid in which every work-group is a chain of memory round
+  // trips) and the small tree tiles of decode-sized M load two stages ahead into two register sets that alternate
+  // with the parity of the stage.
+  constexpr int NSET = (TREE && TM * TN > 8) ? 1 : 2;
   u32x4 xregs[NSET][XCH], wregs[NSET][WCH];
 
   auto load_stage = [&](int s, int set) __attribute__((always_inline)) {
@@ -159,7 +160,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
   const int nouter = TREE ? p.T : (nstages + LS - 1) / LS;
 
   load_stage(0, 0);
-  if (!TREE) load_stage(min(1, nstages - 1), 1);
+  if (NSET == 2) load_stage(min(1, nstages - 1), 1);
   store_stage(0, 0);
   __syncthreads();
 
@@ -170,7 +171,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
       if (TREE || s < nstages) {
         // the stage after the last one re-reads the last one into the idle buffer: harmless, and it
         // keeps the staging registers free of control flow
-        if (TREE) load_stage(min(s + 1, nstages - 1), 0);
+        if (NSET == 1) load_stage(min(s + 1, nstages - 1), 0);
         else load_stage(min(s + 2, nstages - 1), i & 1);  // the set that held stage s, stored a stage ago
         const uint16_t* bx = smem + (s & 1) * STAGE;
         const uint16_t* bw = bx + BM * BK;
@@ -196,7 +197,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
               acc[a][b] = Num::mfma(fw[b], fx[a], fresh ? zero : acc[a][b]);
             }
         }
-        store_stage((s + 1) & 1, TREE ? 0 : (i + 1) & 1);
+        store_stage((s + 1) & 1, NSET == 1 ? 0 : (i + 1) & 1);
         __syncthreads();
       }
     }
