@@ -68,7 +68,10 @@ def cpu_baseline(budget_s=12.0, max_runs=30):
                       f"{len(ts)} runs in {spent:.1f} s, median {t:.2f} s each"}
 
 
-def table(steps, warmup):
+def table(steps, warmup, hot=False):
+    """Per-shape figures.  Unless `hot`, every case cycles through enough distinct input sets (more than 768 MB in
+    all) that nothing it reads is still in the 256 MB memory-side cache from the previous call: the GB/s are HBM
+    figures, as in a model whose every layer has its own weights."""
     import torch
     from oracle import tbik_oracle as O
     from llm_reproducibility_amd.bio import batch_invariant_ops as bio
@@ -76,11 +79,22 @@ def table(steps, warmup):
     dev = torch.device("cuda:0")
     rows = []
 
+    def cycling(make, nbytes, fn):
+        n = 1 if (hot or nbytes >= 768e6) else min(16, int(768e6 // nbytes) + 1)
+        sets = [make() for _ in range(n)]
+        state = [0]
+
+        def call():
+            args = sets[state[0] % n]
+            state[0] += 1
+            return fn(*args)
+        return call
+
     def gemm_row(name, M, K, N, leaf):
-        X = torch.randn((M, K), device=dev).to(torch.bfloat16)
-        W = (torch.randn((N, K), device=dev) * 0.02).to(torch.bfloat16)
-        ms, _ = hip_time_ms(lambda: matmul_tp_persistent(X, W.t(), leaf_k=leaf), steps, warmup)
+        def make():
+            return (torch.randn((M, K), device=dev).to(torch.bfloat16), (torch.randn((N, K), device=dev) * 0.02).to(torch.bfloat16))
         fl, by = 2.0 * M * N * K, 2.0 * (M * K + K * N + M * N)
+        ms, _ = hip_time_ms(cycling(make, by, lambda X, W: matmul_tp_persistent(X, W.t(), leaf_k=leaf)), steps, warmup)
         rows.append((name, ms * 1e3, fl / ms / 1e9, by / ms / 1e6))
 
     for M in (1, 16, 128, 2048):
@@ -95,33 +109,38 @@ def table(steps, warmup):
                           ("qkv 8B", 1, 4096, 6144), ("qkv 8B", 32, 4096, 6144), ("qkv 8B", 128, 4096, 6144),
                           ("gate_up 8B", 1, 4096, 24576), ("gate_up 8B", 32, 4096, 24576), ("gate_up 8B", 128, 4096, 24576),
                           ("lm_head 8B", 1, 4096, 151936), ("lm_head 8B", 32, 4096, 151936)):
-        X = torch.randn((M, K), device=dev).to(torch.bfloat16)
-        W = (torch.randn((N, K), device=dev) * 0.02).to(torch.bfloat16)
-        ms, _ = hip_time_ms(lambda: bio.matmul_persistent(X, W.t()), steps, warmup)
-        rows.append((f"batch-invariant mm {name} M={M} K={K} N={N}", ms * 1e3, 2.0 * M * N * K / ms / 1e9,
-                     2.0 * (M * K + K * N + M * N) / ms / 1e6))
+        def make(M=M, K=K, N=N):
+            return (torch.randn((M, K), device=dev).to(torch.bfloat16), (torch.randn((N, K), device=dev) * 0.02).to(torch.bfloat16))
+        by = 2.0 * (M * K + K * N + M * N)
+        ms, _ = hip_time_ms(cycling(make, by, lambda X, W: bio.matmul_persistent(X, W.t())), steps, warmup)
+        rows.append((f"batch-invariant mm {name} M={M} K={K} N={N}", ms * 1e3, 2.0 * M * N * K / ms / 1e9, by / ms / 1e6))
     for p in (2, 4, 8):
-        parts = [torch.randn((2048, 4096), device=dev).to(torch.bfloat16) for _ in range(p)]
-        ms, _ = hip_time_ms(lambda: tree_combine(parts), steps, warmup)
-        rows.append((f"tree_combine p={p} [2048,4096]", ms * 1e3, 0.0, (p + 1) * 2048 * 4096 * 2 / ms / 1e6))
+        by = (p + 1) * 2048 * 4096 * 2
+        make = lambda p=p: ([torch.randn((2048, 4096), device=dev).to(torch.bfloat16) for _ in range(p)],)  # noqa: E731
+        ms, _ = hip_time_ms(cycling(make, by, tree_combine), steps, warmup)
+        rows.append((f"tree_combine p={p} [2048,4096]", ms * 1e3, 0.0, by / ms / 1e6))
     w = torch.ones(4096, device=dev, dtype=torch.bfloat16)
     for r in (1, 7, 256, 4096):
-        x = torch.randn((r, 4096), device=dev).to(torch.bfloat16)
-        ms, _ = hip_time_ms(lambda: bio.rms_norm(x, w, 1e-6), steps, warmup)
-        rows.append((f"rmsnorm rows={r} hidden=4096", ms * 1e3, 0.0, (r * 4096 * 4 + 8192) / ms / 1e6))
+        by = r * 4096 * 4 + 8192
+        make = lambda r=r: (torch.randn((r, 4096), device=dev).to(torch.bfloat16),)  # noqa: E731
+        ms, _ = hip_time_ms(cycling(make, by, lambda x: bio.rms_norm(x, w, 1e-6)), steps, warmup)
+        rows.append((f"rmsnorm rows={r} hidden=4096", ms * 1e3, 0.0, by / ms / 1e6))
     for r in (1, 7, 256, 4096):
-        x = torch.randn((r, 151936), device=dev)
-        ms, _ = hip_time_ms(lambda: bio.log_softmax(x), max(steps // 4, 3), warmup)
-        rows.append((f"log_softmax rows={r} vocab=151936 (8 B/elem)", ms * 1e3, 0.0, r * 151936 * 8 / ms / 1e6))
+        by = r * 151936 * 8
+        make = lambda r=r: (torch.randn((r, 151936), device=dev),)  # noqa: E731
+        ms, _ = hip_time_ms(cycling(make, by, bio.log_softmax), max(steps // 4, 3), warmup)
+        rows.append((f"log_softmax rows={r} vocab=151936 (8 B/elem)", ms * 1e3, 0.0, by / ms / 1e6))
     for r in (1, 7, 256, 4096):
-        x = torch.randn((r, 4096), device=dev)
-        ms, _ = hip_time_ms(lambda: bio.mean_dim(x, -1), steps, warmup)
-        rows.append((f"mean rows={r} n=4096", ms * 1e3, 0.0, r * 4096 * 4 / ms / 1e6))
+        by = r * 4096 * 4
+        make = lambda r=r: (torch.randn((r, 4096), device=dev),)  # noqa: E731
+        ms, _ = hip_time_ms(cycling(make, 2 * by, lambda x: bio.mean_dim(x, -1)), steps, warmup)
+        rows.append((f"mean rows={r} n=4096", ms * 1e3, 0.0, by / ms / 1e6))
     from llm_reproducibility_amd import ops
     for r in (1, 256, 4096):
-        x = torch.randn((r, 2 * 12288), device=dev).to(torch.bfloat16)
-        ms, _ = hip_time_ms(lambda: ops.bi_silu_mul(x), steps, warmup)
-        rows.append((f"silu_mul rows={r} inter=12288 (6 B/elem)", ms * 1e3, 0.0, r * 12288 * 6 / ms / 1e6))
+        by = r * 12288 * 6
+        make = lambda r=r: (torch.randn((r, 2 * 12288), device=dev).to(torch.bfloat16),)  # noqa: E731
+        ms, _ = hip_time_ms(cycling(make, by, ops.bi_silu_mul), steps, warmup)
+        rows.append((f"silu_mul rows={r} inter=12288 (6 B/elem)", ms * 1e3, 0.0, by / ms / 1e6))
     # fixed-order attention (Qwen3-8B heads: 32 query, 8 key/value, head_dim 128)
     Hq, Hkv, D = 32, 8, 128
     def i32(v):
@@ -129,14 +148,19 @@ def table(steps, warmup):
     for name, B, qlen, ctx in (("prefill 8 x 512", 8, 512, 512), ("prefill 1 x 4096", 1, 4096, 4096),
                                ("decode 128 seqs ctx 768", 128, 1, 768), ("decode 8 seqs ctx 4096", 8, 1, 4096)):
         L = ((ctx + 31) // 32) * 32
-        q = torch.randn((B * qlen, Hq, D), device=dev).to(torch.bfloat16)
-        kc = torch.randn((B, Hkv, L, D), device=dev).to(torch.bfloat16)
-        vt = torch.randn((B, Hkv, D, L), device=dev).to(torch.bfloat16)
         qs, ql, cl = i32([b * qlen for b in range(B)]), i32([qlen] * B), i32([ctx] * B)
-        ms, _ = hip_time_ms(lambda: ops.bi_attention_bf16(q, kc, vt, qs, ql, cl, qlen, D ** -0.5), max(steps // 2, 3), warmup)
         pairs = B * Hq * (qlen * (2 * ctx - qlen + 1) // 2)          # causal (query, key) pairs
         byts = 2.0 * (2 * B * Hkv * ctx * D + 2 * B * qlen * Hq * D)   # K, V once; q and out
+
+        def make(B=B, qlen=qlen, L=L):
+            return (torch.randn((B * qlen, Hq, D), device=dev).to(torch.bfloat16),
+                    torch.randn((B, Hkv, L, D), device=dev).to(torch.bfloat16),
+                    torch.randn((B, Hkv, D, L), device=dev).to(torch.bfloat16))
+        ms, _ = hip_time_ms(cycling(make, byts, lambda q, kc, vt: ops.bi_attention_bf16(q, kc, vt, qs, ql, cl, qlen, D ** -0.5)),
+                            max(steps // 2, 3), warmup)
         rows.append((f"attention {name}", ms * 1e3, 4.0 * pairs * D / ms / 1e9, byts / ms / 1e6))
+    print("inputs " + ("reused by every call (hot in the memory-side cache)" if hot else
+                       "cycled through more than 768 MB of distinct buffers (cold in the 256 MB memory-side cache)"), file=sys.stderr)
     print(f"{'case':52s} {'us':>10s} {'TFLOP/s':>9s} {'%MFMA':>6s} {'GB/s':>9s} {'%HBM':>6s}", file=sys.stderr)
     for name, us, tf, gbs in rows:
         print(f"{name:52s} {us:10.1f} {tf:9.1f} {100 * tf / PEAK_BF16_TFLOPS:6.1f} {gbs:9.1f} {100 * gbs / PEAK_HBM_GBS:6.1f}",
@@ -149,6 +173,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--table", action="store_true", help="also print the per-shape table to stderr")
+    ap.add_argument("--table-hot", action="store_true", help="with --table: reuse one input set per case (cache-hot figures)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run 5 plain device copies of X (50,331,648 B read + as many written each) so that a "
@@ -202,7 +227,7 @@ def main():
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     if args.table:
-        table(max(args.steps // 2, 5), max(args.warmup // 2, 2))
+        table(max(args.steps // 2, 5), max(args.warmup // 2, 2), hot=args.table_hot)
     print(json.dumps(out))
 
 

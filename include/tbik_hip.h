@@ -78,7 +78,7 @@ size_t tbik_gemm_workspace_bytes(int M, int N, int K, int leaf_k);
 
 /*
  * out[i] = adjacent-pair binary tree over parts[0..nparts-1][i], bf16 adds (round to nearest even
- * at every node); nparts in {1,2,4,8}; all buffers contiguous, numel elements, 2-byte aligned
+ * at every node); nparts a power of two up to 32; all buffers contiguous, numel elements, 2-byte aligned
  * (16-byte aligned buffers take the vector path).  `out` may alias parts[0].
  * Replaces: the local adds of tree_all_reduce_sum_native, src/tbik/tree_based_all_reduce.py:32-37,
  *           simple_matmul.py:35-38, and packed_tree_reduce / custom_tree_all_reduce,

@@ -356,7 +356,7 @@ static bool make_plan(int M, int N, int K, int leaf_k, bool f16, Plan* pl) {
   int T, flb, level_k;
   if (M <= 0 || N <= 0 || tbik_tree_params(K, leaf_k, &T, &flb, &level_k) != TBIK_OK) return false;
   const int lb = level_k - 1;
-  const int max_split = lb >= 3 ? 8 : (1 << lb);
+  const int max_split = lb >= 5 ? 32 : (1 << lb);
   const int64_t wide_tiles = (int64_t)((M + 127) / 128) * ((N + 255) / 256);
   int split = 1;
   bool wide = false;
@@ -366,6 +366,7 @@ static bool make_plan(int M, int N, int K, int leaf_k, bool f16, Plan* pl) {
     // (17 ns per k per round; 5 TB/s and 4 us for the combine).
     double best = 0;
     for (int sp = 1; sp <= max_split; sp *= 2) {
+      if (sp > 8 && wide_tiles * sp > 256) break;  // finer cuts only while the whole grid still runs as one round
       const double rounds = (double)((wide_tiles * sp + 255) / 256);
       double t = rounds * ((double)K / sp) * 0.0173;
       if (sp > 1) t += 4.0 + (double)(sp + 1) * M * N * 2.0 / 5.0e6;
@@ -380,7 +381,7 @@ static bool make_plan(int M, int N, int K, int leaf_k, bool f16, Plan* pl) {
     const int bm = M <= 16 ? 16 : (M <= 64 ? 64 : 128), bn = M <= 16 ? 64 : 128;
     const int64_t tiles = (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
     split = 1;
-    while (tiles * split < 512 && split < max_split) split *= 2;
+    while (tiles * split < 512 && split < max_split && split < 8) split *= 2;
   }
   int ls = 0;
   while ((1 << ls) < split) ls++;
@@ -474,11 +475,11 @@ int gemm_dispatch(bool tree, bool f16, const void* A, int64_t lda, const void* B
     else rc = leaf_k == 256 ? launch_tree<4, false>(a, pl.split, stream) : launch_tree<2, false>(a, pl.split, stream);
   }
   if (rc != TBIK_OK || pl.split == 1) return rc;
-  const void* parts[8];
+  const void* parts[32];
   for (int i = 0; i < pl.split; i++) parts[i] = wsb + (size_t)i * M * N * sizeof(uint16_t);
   if (ldc == N) return tree_combine_bias_dispatch(parts, pl.split, C, (int64_t)M * N, bias, N, f16, stream);
   for (int m = 0; m < M && rc == TBIK_OK; m++) {  // strided C (rare): row by row
-    const void* rp[8];
+    const void* rp[32];
     for (int i = 0; i < pl.split; i++) rp[i] = static_cast<const uint8_t*>(parts[i]) + (size_t)m * N * sizeof(uint16_t);
     rc = tree_combine_bias_dispatch(rp, pl.split, static_cast<uint16_t*>(C) + (int64_t)m * ldc, N, bias, N, f16, stream);
   }

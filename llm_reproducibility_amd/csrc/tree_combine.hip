@@ -1,4 +1,4 @@
-// Shard combine: out[i] = adjacent-pair binary tree over up to 8 bf16 (or fp16) partials, every node rounded to
+// Shard combine: out[i] = adjacent-pair binary tree over up to 32 bf16 (or fp16) partials, every node rounded to
 // the element type.  This is the arithmetic of the reference's cross-GPU tree all-reduce
 // (src/tbik/tree_based_all_reduce.py:32-37; packed_tree_reduce,
 // mini_allreduce/tbik_kernel/csrc/allreduce/custom_all_reduce.cuh:203-234) applied to partials that
@@ -8,7 +8,7 @@
 namespace tbik {
 
 struct CombineArgs {
-  const uint16_t* parts[8];
+  const uint16_t* parts[32];
   uint16_t* out;
   int64_t numel;
   const uint16_t* bias;  // optional [ncols] row vector added (in bf16) after the tree; element i is in column i % ncols
@@ -16,8 +16,8 @@ struct CombineArgs {
 };
 
 template <int NP, bool F16>
-__device__ __forceinline__ uint32_t tree_node(const uint32_t (&v)[8]) {
-  uint32_t w[8];
+__device__ __forceinline__ uint32_t tree_node(const uint32_t (&v)[NP]) {
+  uint32_t w[NP];
 #pragma unroll
   for (int i = 0; i < NP; i++) w[i] = v[i];
 #pragma unroll
@@ -36,7 +36,7 @@ __global__ __launch_bounds__(256) void combine_vec_kernel(const CombineArgs a, i
 #pragma unroll
     for (int p = 0; p < NP; p++) in[p] = reinterpret_cast<const uint4*>(a.parts[p])[i];
     uint4 o;
-    uint32_t v[8];
+    uint32_t v[NP];
 #pragma unroll
     for (int p = 0; p < NP; p++) v[p] = in[p].x;
     o.x = tree_node<NP, F16>(v);
@@ -65,7 +65,7 @@ template <int NP, bool F16>
 __global__ __launch_bounds__(256) void combine_scalar_kernel(const CombineArgs a, int64_t begin) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = begin + (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < a.numel; i += stride) {
-    uint32_t v[8];
+    uint32_t v[NP];
 #pragma unroll
     for (int p = 0; p < NP; p++) v[p] = a.parts[p][i];
     uint32_t r = tree_node<NP, F16>(v);
@@ -95,13 +95,13 @@ static int launch_combine(const CombineArgs& a, bool vec_ok, hipStream_t stream)
 int tree_combine_bias_dispatch(const void* const* parts, int nparts, void* out, int64_t numel, const void* bias, int N,
                                bool f16, hipStream_t stream) {
   if (numel < 0 || (bias && N <= 0)) return TBIK_ERR_INVALID;
-  if (nparts != 1 && nparts != 2 && nparts != 4 && nparts != 8) return TBIK_ERR_INVALID;
+  if (nparts < 1 || nparts > 32 || (nparts & (nparts - 1))) return TBIK_ERR_INVALID;
   if (numel == 0) return TBIK_OK;
   if (!parts || !out) return TBIK_ERR_INVALID;
   CombineArgs a;
   bool vec_ok = (reinterpret_cast<uintptr_t>(out) & 15) == 0;
   if (reinterpret_cast<uintptr_t>(out) & 1) return TBIK_ERR_ALIGNMENT;
-  for (int p = 0; p < 8; p++) a.parts[p] = nullptr;
+  for (int p = 0; p < 32; p++) a.parts[p] = nullptr;
   for (int p = 0; p < nparts; p++) {
     if (!parts[p]) return TBIK_ERR_INVALID;
     if (reinterpret_cast<uintptr_t>(parts[p]) & 1) return TBIK_ERR_ALIGNMENT;
@@ -118,14 +118,18 @@ int tree_combine_bias_dispatch(const void* const* parts, int nparts, void* out, 
       case 1: return launch_combine<1, true>(a, vec_ok, stream);
       case 2: return launch_combine<2, true>(a, vec_ok, stream);
       case 4: return launch_combine<4, true>(a, vec_ok, stream);
-      default: return launch_combine<8, true>(a, vec_ok, stream);
+      case 8: return launch_combine<8, true>(a, vec_ok, stream);
+      case 16: return launch_combine<16, true>(a, vec_ok, stream);
+      default: return launch_combine<32, true>(a, vec_ok, stream);
     }
   }
   switch (nparts) {
     case 1: return launch_combine<1, false>(a, vec_ok, stream);
     case 2: return launch_combine<2, false>(a, vec_ok, stream);
     case 4: return launch_combine<4, false>(a, vec_ok, stream);
-    default: return launch_combine<8, false>(a, vec_ok, stream);
+    case 8: return launch_combine<8, false>(a, vec_ok, stream);
+    case 16: return launch_combine<16, false>(a, vec_ok, stream);
+    default: return launch_combine<32, false>(a, vec_ok, stream);
   }
 }
 

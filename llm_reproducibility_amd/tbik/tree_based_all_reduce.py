@@ -17,13 +17,13 @@ from .. import ops
 
 
 def tree_combine(parts: Sequence[torch.Tensor]) -> torch.Tensor:
-    """Adjacent-pair binary tree over 1, 2, 4 or 8 same-shaped bf16 partials; returns a new tensor."""
+    """Adjacent-pair binary tree over a power-of-two number of same-shaped partials; returns a new tensor."""
     n = len(parts)
     if n == 0 or n & (n - 1) != 0:
         raise ValueError("the number of partials must be a power of 2")
-    if n > 8:
-        # wider worlds: reduce groups of 8 first; adjacent-pair trees compose
-        return tree_combine([tree_combine(parts[i:i + 8]) for i in range(0, n, 8)])
+    if n > 32:
+        # wider worlds: reduce groups of 32 first; adjacent-pair trees compose
+        return tree_combine([tree_combine(parts[i:i + 32]) for i in range(0, n, 32)])
     if any(p.dtype != parts[0].dtype for p in parts):
         raise NotImplementedError("tree_combine takes partials of one dtype")
     if any(p.shape != parts[0].shape for p in parts):

@@ -140,6 +140,12 @@ def test_invariance_qwen3_32b_down_proj_leaf128(dev):
     _invariance(dev, 25600, 5120, (1, 64, 512), "gauss", 4096)
 
 
+def test_invariance_with_k_cut_into_32_subtrees(dev):
+    # 32 leaves and few column tiles: the small batches are cut into 16 and 32 one-leaf shards, the large one is not
+    _invariance(dev, 8192, 2048, (64, 128, 200), "gauss", 1024)
+    _invariance(dev, 4096, 1024, (100,), "gauss", 512)
+
+
 def test_reference_smoke_script_shape(dev):
     # simple_matmul.py: M,K,N = 1024,6144,2048, both operands ~ N(0,1), row-major B, TP=4, batch halves
     M, K, N = 1024, 6144, 2048
@@ -154,8 +160,8 @@ def test_reference_smoke_script_shape(dev):
 
 def test_tree_combine_matches_oracle_bitwise(dev):
     for numel_shape in [(2048, 4096), (7, 33), (1, 5)]:
-        parts = [O.gaussian_bf16(numel_shape, 1.0, s) for s in range(8)]
-        for n in (1, 2, 4, 8):
+        parts = [O.gaussian_bf16(numel_shape, 1.0, s) for s in range(64)]
+        for n in (1, 2, 4, 8, 16, 32, 64):
             got = tree_combine([p.to(dev) for p in parts[:n]])
             assert_bitwise(got, O.tree_combine(parts[:n]), f"{numel_shape} n={n}")
     # unaligned views take the scalar path: same bits
