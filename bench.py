@@ -99,12 +99,25 @@ def table(steps, warmup, hot=False):
 
     for M in (1, 16, 128, 2048):
         gemm_row(f"down_proj 8B  M={M} K=12288 N=4096", M, 12288, 4096, 256)
+    def library_row(M, K, N):
+        # context only: the vendor library GEMM behind torch.matmul (no tree, reduction order not fixed) on like operands
+        def make():
+            return (torch.randn((M, K), device=dev).to(torch.bfloat16), (torch.randn((N, K), device=dev) * 0.02).to(torch.bfloat16))
+        fl, by = 2.0 * M * N * K, 2.0 * (M * K + K * N + M * N)
+        ms, _ = hip_time_ms(cycling(make, by, lambda X, W: torch.matmul(X, W.t())), steps, warmup)
+        rows.append((f"  [torch.matmul, not invariant] M={M} K={K} N={N}", ms * 1e3, fl / ms / 1e9, by / ms / 1e6))
+
+    for M in (1, 128, 2048):
+        library_row(M, 12288, 4096)
     for p in (2, 4, 8):
         gemm_row(f"  shard TP={p}  M=2048 K={12288 // p} N=4096", 2048, 12288 // p, 4096, 256)
     for M in (1, 64, 512, 4096):
         gemm_row(f"o_proj 32B    M={M} K=8192 N=5120", M, 8192, 5120, 256)
     for M in (1, 64, 512, 4096):
         gemm_row(f"down_proj 32B M={M} K=25600 N=5120 leaf128", M, 25600, 5120, choose_leaf_k(25600))
+    library_row(4096, 8192, 5120)
+    library_row(4096, 25600, 5120)
+    library_row(2048, 4096, 24576)
     for name, M, K, N in (("qkv 8B", 2048, 4096, 6144), ("gate_up 8B", 2048, 4096, 24576), ("lm_head 8B", 128, 4096, 151936),
                           ("qkv 8B", 1, 4096, 6144), ("qkv 8B", 32, 4096, 6144), ("qkv 8B", 128, 4096, 6144),
                           ("gate_up 8B", 1, 4096, 24576), ("gate_up 8B", 32, 4096, 24576), ("gate_up 8B", 128, 4096, 24576),
