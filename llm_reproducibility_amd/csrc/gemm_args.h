@@ -45,6 +45,20 @@ struct StreamArgs {
 };
 int gemm_single_acc_stream_launch(const StreamArgs& a, bool f16, hipStream_t stream);
 
+// gemm_tree_strip.hip: tree-ordered 16-bit GEMM for at most 16 rows, K cut over the waves of a work-group
+struct StripArgs {
+  const uint16_t* X;   // [M,K], row stride ldx
+  const uint16_t* W;   // [N,K], row stride ldw
+  uint16_t* C;         // [M,N], row stride ldc
+  const uint16_t* bias;
+  int64_t ldx, ldw, ldc;
+  int M, N, K;
+  int flb, lb;         // K = flb * leaf_k * 2^lb
+  int vec_store;
+};
+int gemm_tree_strip_waves(int M, int N, int K, int lb);  // waves per strip, or 0: use another kernel
+int gemm_tree_strip_launch(const StripArgs& a, int leaf_k, int waves, bool f16, hipStream_t stream);
+
 // tree_combine.hip
 int tree_combine_bias_dispatch(const void* const* parts, int nparts, void* out, int64_t numel, const void* bias, int N,
                                bool f16, hipStream_t stream);

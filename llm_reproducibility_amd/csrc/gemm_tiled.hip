@@ -399,6 +399,7 @@ static bool make_plan(int M, int N, int K, int leaf_k, bool f16, Plan* pl) {
 size_t gemm_workspace_bytes(int M, int N, int K, int leaf_k, bool f16) {
   Plan pl;
   if (!make_plan(M, N, K, leaf_k, f16, &pl)) return 0;
+  if (gemm_tree_strip_waves(M, N, K, pl.lb + (pl.split > 1 ? __builtin_ctz((unsigned)pl.split) : 0))) return 0;  // no workspace on that path
   return pl.partial_bytes + pl.parked_bytes;
 }
 
@@ -447,6 +448,16 @@ int gemm_dispatch(bool tree, bool f16, const void* A, int64_t lda, const void* B
   }
 
   if (leaf_k != 256 && leaf_k != 128) return TBIK_ERR_UNSUPPORTED;
+  {
+    // a handful of rows: one launch, K cut over the waves of a work-group, nothing goes through the workspace
+    int T, flb, level_k;
+    if (tbik_tree_params(K, leaf_k, &T, &flb, &level_k) != TBIK_OK) return TBIK_ERR_INVALID;
+    const int waves = gemm_tree_strip_waves(M, N, K, level_k - 1);
+    if (waves) {
+      StripArgs sa{a.X, a.W, a.C, a.bias, a.ldx, a.ldw, a.ldc, M, N, K, flb, level_k - 1, a.vec_store};
+      return gemm_tree_strip_launch(sa, leaf_k, waves, f16, stream);
+    }
+  }
   Plan pl;
   if (!make_plan(M, N, K, leaf_k, f16, &pl)) return TBIK_ERR_INVALID;
   const size_t need = pl.partial_bytes + pl.parked_bytes;

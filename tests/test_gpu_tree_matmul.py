@@ -79,6 +79,37 @@ def test_integer_inputs_match_oracle_bitwise(dev, M, N, K, leaf):
     assert_bitwise(got, want, f"{M}x{N}x{K}")
 
 
+# (M, N, K, leaf): a few rows (up to 16 when the tree has at most four aligned subtrees) and a grid of 16-column strips that loads every CU alike: the one-launch kernel that
+# cuts K over the waves of a work-group (2/4/8 waves, FLB in {1,2,3,5,25}, up to three binary levels inside a wave,
+# a ragged last strip)
+STRIP_SHAPES = [
+    (1, 4096, 512, 256), (3, 2056, 1024, 256), (4, 1024, 2048, 256), (2, 3000, 4096, 256), (4, 1040, 6144, 256),
+    (2, 4090, 12288, 256), (1, 8192, 4096, 256), (3, 1024, 16384, 256), (4, 1040, 8192, 128), (1, 4096, 25600, 128),
+    (2, 4096, 1280, 128), (8, 2560, 9728, 256), (16, 1024, 1536, 256), (13, 4096, 2560, 128),
+]
+
+
+@pytest.mark.parametrize("M,N,K,leaf", STRIP_SHAPES)
+def test_few_rows_one_launch_kernel_matches_oracle_bitwise(dev, M, N, K, leaf):
+    print("case", M, N, K, leaf, flush=True)
+    A_wide = O.integer_bf16((M, K + 8), -9, 9, 30 + M)
+    A = A_wide[:, 8:]                       # a strided view (row stride K + 8)
+    Wnk = O.integer_bf16((N, K), -7, 7, 40 + N % 97)
+    bias = O.integer_bf16((N,), -300, 300, 5)
+    want = O.matmul_tree(A, Wnk.t(), leaf=leaf)
+    Ad, Wd = A_wide.to(dev)[:, 8:], Wnk.to(dev)
+    got = matmul_tp_persistent(Ad, Wd.t(), leaf_k=leaf)
+    assert got.shape == (M, N) and got.is_contiguous()
+    assert_bitwise(got, want, f"{M}x{N}x{K}")
+    assert_bitwise(matmul_tp_persistent(Ad, Wd.t(), bias.to(dev), leaf_k=leaf), O.matmul_tree(A, Wnk.t(), bias, leaf=leaf), "bias")
+    # the same rows inside a batch of 40 go through another kernel: same bits
+    big = torch.cat([Ad, O.integer_bf16((40 - M, K), -9, 9, 77).to(dev)])
+    assert_bitwise(matmul_tp_persistent(big, Wd.t(), leaf_k=leaf)[:M], want, "rows inside a larger batch")
+    if leaf == 256:
+        h = matmul_tp_persistent(Ad.to(torch.float16), Wd.to(torch.float16).t(), leaf_k=leaf)
+        assert_bitwise(h, O.matmul_tree(A.to(torch.float16), Wnk.to(torch.float16).t(), leaf=leaf), "fp16")
+
+
 def test_bias_strided_a_and_row_major_b(dev):
     M, N, K = 70, 96, 1536
     A_wide = O.integer_bf16((M, 2 * K), -9, 9, 1)
