@@ -259,9 +259,20 @@ int gemm_single_acc_stream_launch(const StreamArgs& a, bool f16, hipStream_t str
   // one block of rows, and all of X fits the staging registers of one pass and 40 KiB of LDS (several work-groups
   // per CU)
   if (a.M <= 16 && (int64_t)a.M * a.K <= ROWS_MAX_ELEMS && (int64_t)a.M * (a.K * 2 + 16) <= 40 * 1024) {
-    if (a.N <= 16 * 1024)  // at most 1024 strips: one per work-group spreads them over all CUs
-      return a.M * a.K <= ROWS_MAX_ELEMS / 4 ? (f16 ? stream_rows_launch<1, true>(a, stream) : stream_rows_launch<1, false>(a, stream))
-                                             : (f16 ? stream_rows_launch<4, true>(a, stream) : stream_rows_launch<4, false>(a, stream));
+    // Strips per work-group.  What bounds one pass over the weights is the number of misses a CU keeps in flight, so
+    // the grid should put the same number of work-groups on every CU: the score is the share of CU slots that the
+    // last round of work-groups leaves used (measured: gate_up of an 8B model, 1536 strips, 41 us as 384 groups of
+    // four, 37 us as 512 groups of three).  One strip per work-group restages X for every strip and is only
+    // considered while X is small; two strips per work-group measured worse than either neighbour throughout.
+    const int64_t strips = ((int64_t)a.N + 15) / 16;
+    auto score = [&](int nw, double weight) {
+      const int64_t groups = (strips + nw - 1) / nw;
+      return weight * (double)groups / (double)(((groups + 255) / 256) * 256);
+    };
+    const double s3 = score(3, 1.0), s4 = score(4, 0.98);
+    const double s1 = a.M * a.K <= ROWS_MAX_ELEMS / 4 ? score(1, 0.95) : 0.0;
+    if (s1 > s3 && s1 > s4) return f16 ? stream_rows_launch<1, true>(a, stream) : stream_rows_launch<1, false>(a, stream);
+    if (s3 >= s4) return f16 ? stream_rows_launch<3, true>(a, stream) : stream_rows_launch<3, false>(a, stream);
     return f16 ? stream_rows_launch<4, true>(a, stream) : stream_rows_launch<4, false>(a, stream);
   }
   const int mb = (a.M + 15) / 16;
