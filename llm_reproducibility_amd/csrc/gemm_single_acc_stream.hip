@@ -144,80 +144,88 @@ __global__ __launch_bounds__(NWAVES * 64) void gemm_single_acc_stream_kernel(con
 
   const uint16_t* wp = p.W + (int64_t)min(n0 + r, p.N - 1) * p.ldw + 8 * g;
 
-  // staging of X: thread t moves 16-byte chunk q % (KW/8) of row q / (KW/8), q = t + 256 i, i < XLD
+  // staging of X: thread t moves 16-byte chunk q % (KW/8) of row q / (KW/8), q = t + NT i, i < XLD
   const uint16_t* xsrc[XLD];
   uint32_t xdst[XLD];
-  int xk[XLD];
 #pragma unroll
   for (int i = 0; i < XLD; i++) {
     const int q = tid + NT * i;
     const int row = q / (KW / 8), c = q % (KW / 8);
     xsrc[i] = p.X + (int64_t)min(row, p.M - 1) * p.ldx + c * 8;
     xdst[i] = row * ROWB + c * 16;
-    xk[i] = c * 8;
   }
   const int nsteps = p.K / 32;
-  const int nwin = (nsteps + WS - 1) / WS;
+  const int nfull = nsteps / WS;  // whole windows; the steps after them are handled at the end
 
   u32x4 xr[XLD];
   bf16x8 wa[WS], wb[WS];
+  // Every load of the main loop is issued unconditionally and addresses a whole window (one base pointer, constant
+  // offsets): a window past the end re-reads the last one and is never used, so the number of loads in flight is
+  // static and the waits can leave the next window in flight.
   auto load_x = [&](int w) __attribute__((always_inline)) {
+    const int64_t off = (int64_t)min(w, nfull - 1) * KW;
 #pragma unroll
-    for (int i = 0; i < XLD; i++)
-      xr[i] = w * KW + xk[i] < p.K ? *reinterpret_cast<const u32x4*>(xsrc[i] + (int64_t)w * KW) : u32x4{0, 0, 0, 0};
+    for (int i = 0; i < XLD; i++) xr[i] = *reinterpret_cast<const u32x4*>(xsrc[i] + off);
   };
   auto store_x = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < XLD; i++) *reinterpret_cast<u32x4*>(xs + buf * XBUF + xdst[i]) = xr[i];
   };
   auto load_w = [&](bf16x8* w, int win) __attribute__((always_inline)) {
+    const uint16_t* base = wp + (int64_t)min(win, nfull - 1) * KW;
 #pragma unroll
-    for (int u = 0; u < WS; u++) {
-      const int s = min(win * WS + u, nsteps - 1);  // past the end: a valid address, the step is not used
-      w[u] = *reinterpret_cast<const bf16x8*>(wp + (int64_t)s * 32);
-    }
+    for (int u = 0; u < WS; u++) w[u] = *reinterpret_cast<const bf16x8*>(base + u * 32);
   };
 
   f32x4 acc[MB];
 #pragma unroll
   for (int b = 0; b < MB; b++) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
   const uint32_t xfrag = r * ROWB + g * 16;
-  auto compute = [&](const bf16x8* w, int win, int buf) __attribute__((always_inline)) {
-    const int left = nsteps - win * WS;  // steps of this window that exist (uniform)
+  auto compute = [&](const bf16x8* w, int buf) __attribute__((always_inline)) {
 #pragma unroll
     for (int u = 0; u < WS; u++) {
-      if (u < left) {
 #pragma unroll
-        for (int b = 0; b < MB; b++) {
-          const bf16x8 x = *reinterpret_cast<const bf16x8*>(xs + buf * XBUF + xfrag + b * 16 * ROWB + u * 64);
-          acc[b] = Num::mfma(w[u], x, acc[b]);
-        }
+      for (int b = 0; b < MB; b++) {
+        const bf16x8 x = *reinterpret_cast<const bf16x8*>(xs + buf * XBUF + xfrag + b * 16 * ROWB + u * 64);
+        acc[b] = Num::mfma(w[u], x, acc[b]);
       }
     }
   };
 
-  load_x(0);
-  load_w(wa, 0);
-  store_x(0);
-  __syncthreads();
-  for (int win = 0; win < nwin; win += 2) {
-    // even window: weights in wa, X in buffer 0
-    if (win + 1 < nwin) {
+  if (nfull > 0) {
+    load_x(0);
+    load_w(wa, 0);
+    store_x(0);
+    __syncthreads();
+    int win = 0;
+    for (; win + 1 < nfull; win += 2) {
+      // even window: weights in wa, X in buffer 0
+      __builtin_amdgcn_sched_barrier(0);
       load_x(win + 1);
       load_w(wb, win + 1);
-    }
-    compute(wa, win, 0);
-    if (win + 1 < nwin) store_x(1);
-    __syncthreads();
-    if (win + 1 >= nwin) break;
-    // odd window: weights in wb, X in buffer 1
-    if (win + 2 < nwin) {
+      __builtin_amdgcn_sched_barrier(0);
+      compute(wa, 0);
+      store_x(1);
+      __syncthreads();
+      // odd window: weights in wb, X in buffer 1
+      __builtin_amdgcn_sched_barrier(0);
       load_x(win + 2);
       load_w(wa, win + 2);
+      __builtin_amdgcn_sched_barrier(0);
+      compute(wb, 1);
+      store_x(0);
+      __syncthreads();
     }
-    compute(wb, win + 1, 1);
-    if (win + 2 < nwin) store_x(0);
-    __syncthreads();
+    if (win < nfull) compute(wa, 0);  // an odd number of windows: the last one is already in wa and buffer 0
+  }
+  // the steps after the last whole window (K not a multiple of the window): fragments straight from global memory
+  for (int s = nfull * WS; s < nsteps; s++) {
+    const bf16x8 w = *reinterpret_cast<const bf16x8*>(wp + (int64_t)s * 32);
+#pragma unroll
+    for (int b = 0; b < MB; b++) {
+      const bf16x8 x = *reinterpret_cast<const bf16x8*>(p.X + (int64_t)min(b * 16 + r, p.M - 1) * p.ldx + (int64_t)s * 32 + 8 * g);
+      acc[b] = Num::mfma(w, x, acc[b]);
+    }
   }
 
   stream_store<MB, F16>(p, acc, n0, r, g);
