@@ -31,6 +31,9 @@ HIPCC_FLAGS = [
 # scheduler only lengthens live ranges there (more spills at the 256-register limit), so it is switched off for them.
 EXTRA_FLAGS = {
     "gemm_tree_wide.hip": ["-mllvm", "-enable-misched=false"],
+    # attention rescales its output accumulators every key tile: with the accumulators in ordinary registers that is
+    # one multiply each, in accumulation registers it is a read, a multiply and a write back
+    "attention.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
 }
 
 

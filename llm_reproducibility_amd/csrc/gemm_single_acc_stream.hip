@@ -273,8 +273,8 @@ int gemm_single_acc_stream_launch(const StreamArgs& a, bool f16, hipStream_t str
   // one block of rows, and all of X fits the staging registers of one pass and 40 KiB of LDS (several work-groups
   // per CU)
   if (a.M <= 16 && (int64_t)a.M * a.K <= ROWS_MAX_ELEMS && (int64_t)a.M * (a.K * 2 + 16) <= 40 * 1024) {
-    // Strips per work-group.  What bounds one pass over the weights is the number of misses a CU keeps in flight, so
-    // the grid should put the same number of work-groups on every CU: the score is the share of CU slots that the
+    // Strips per work-group.  HBM bandwidth is shared about equally among the CUs that ask for it, so the CU with
+    // the most work-groups finishes last and the grid should put the same number on every CU: the score is the share of CU slots that the
     // last round of work-groups leaves used (measured: gate_up of an 8B model, 1536 strips, 41 us as 384 groups of
     // four, 37 us as 512 groups of three).  One strip per work-group restages X for every strip and is only
     // considered while X is small; two strips per work-group measured worse than either neighbour throughout.
