@@ -110,6 +110,31 @@ def test_few_rows_one_launch_kernel_matches_oracle_bitwise(dev, M, N, K, leaf):
         assert_bitwise(h, O.matmul_tree(A.to(torch.float16), Wnk.to(torch.float16).t(), leaf=leaf), "fp16")
 
 
+@pytest.mark.parametrize("M,N,K", [(2, 4096, 4096), (16, 1024, 3072), (96, 512, 4096), (300, 1024, 12288), (256, 4096, 2048)])
+def test_c_abi_writes_into_a_strided_and_a_misaligned_output(dev, M, N, K):
+    """The entry point itself (no wrapper): C is a column block of a wider matrix (ldc > N), then the same block
+    shifted by one element (2-byte aligned only, scalar stores); every kernel family and the K-cut path."""
+    from llm_reproducibility_amd import _lib
+    L = _lib.lib()
+    print("case", M, N, K, flush=True)
+    A = O.integer_bf16((M, K), -9, 9, 3).to(dev)
+    W = O.integer_bf16((N, K), -7, 7, 4).to(dev)
+    bias = O.integer_bf16((N,), -300, 300, 5).to(dev)
+    want = matmul_tp_persistent(A, W.t(), bias)
+    nws = L.tbik_gemm_workspace_bytes(M, N, K, 256)
+    ws = torch.empty(max(nws, 1), device=dev, dtype=torch.uint8)
+    stream = torch.cuda.current_stream().cuda_stream
+    for shift in (8, 9):
+        wide = torch.full((M, N + 24), 7.0, device=dev, dtype=torch.bfloat16)
+        cptr = wide.data_ptr() + 2 * shift
+        rc = L.tbik_gemm_bf16(A.data_ptr(), K, W.data_ptr(), 1, K, cptr, N + 24, M, N, K, 256, bias.data_ptr(),
+                              ws.data_ptr() if nws else None, nws, stream)
+        assert rc == 0, rc
+        torch.cuda.synchronize()
+        assert_bitwise(wide[:, shift:shift + N], want, f"shift {shift}")
+        assert bool((wide[:, :shift] == 7).all()) and bool((wide[:, shift + N:] == 7).all()), "wrote outside its block"
+
+
 def test_bias_strided_a_and_row_major_b(dev):
     M, N, K = 70, 96, 1536
     A_wide = O.integer_bf16((M, 2 * K), -9, 9, 1)
