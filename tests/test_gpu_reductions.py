@@ -168,6 +168,28 @@ def test_single_accumulator_mm_streaming_kernels_on_ragged_shapes(dev):
     assert torch.equal(bio.matmul_persistent(a1.to(dev), w1.to(dev).t()).cpu(), O.matmul_single_acc(a1, w1.t()))
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 6144, 4096), (5, 1000, 1120), (40, 24576, 512), (64, 1544, 2048), (100, 520, 1024), (300, 4096, 4096)])
+def test_single_accumulator_mm_c_abi_strided_and_misaligned_output(dev, M, N, K):
+    """bi_gemm_bf16 itself (no wrapper): C is a column block of a wider matrix, then the same block shifted by one
+    element (scalar stores): the streaming kernels with 1/3/4/8 strips per work-group, the tiled and the quad kernel."""
+    from llm_reproducibility_amd import _lib
+    L = _lib.lib()
+    print("case", M, N, K, flush=True)
+    A = O.integer_bf16((M, K), -9, 9, 3).to(dev)
+    W = O.integer_bf16((N, K), -7, 7, 4).to(dev)
+    bias = O.integer_bf16((N,), -5, 5, 5).to(dev)
+    want = bio.matmul_persistent(A, W.t(), bias)
+    assert torch.equal(want[:8].cpu(), O.matmul_single_acc(A[:8].cpu(), W.cpu().t(), bias.cpu()))
+    stream = torch.cuda.current_stream().cuda_stream
+    for shift in (8, 9):
+        wide = torch.full((M, N + 24), 7.0, device=dev, dtype=torch.bfloat16)
+        rc = L.bi_gemm_bf16(A.data_ptr(), K, W.data_ptr(), 1, K, wide.data_ptr() + 2 * shift, N + 24, M, N, K, bias.data_ptr(), stream)
+        assert rc == 0, rc
+        torch.cuda.synchronize()
+        assert torch.equal(wide[:, shift:shift + N], want), f"shift {shift}"
+        assert bool((wide[:, :shift] == 7).all()) and bool((wide[:, shift + N:] == 7).all()), "wrote outside its block"
+
+
 def test_single_accumulator_mm_fp16(dev):
     a = O.gaussian_bf16((300, 1000), 1.0, 0).to(torch.float16)
     w = O.gaussian_bf16((200, 1000), 0.05, 1).to(torch.float16)
