@@ -202,6 +202,32 @@ def test_invariance_with_k_cut_into_32_subtrees(dev):
     _invariance(dev, 4096, 1024, (100,), "gauss", 512)
 
 
+def test_random_shapes_tp_batch_and_row_invariance(dev):
+    """Seeded sweep over (leaf, leaves, M, N): every legal simulated TP split, a random batch prefix and a random single
+    row reproduce the bits of the full call, whichever kernels the dispatcher picks for the pieces."""
+    import random
+    rng = random.Random(5)
+    for it in range(40):
+        leaf = rng.choice([256, 256, 128])
+        T = rng.choice([2, 4, 6, 8, 12, 16, 24, 32, 40, 48, 64])
+        M = rng.choice([1, 3, 4, 5, 16, 17, 64, 65, 128, 200, 300, 600])
+        N = rng.choice([64, 520, 1024, 1040, 2560, 4096, 4104])
+        K = leaf * T
+        print("case", it, M, N, K, leaf, flush=True)
+        X = O.gaussian_bf16((M, K), 1.0, it).to(dev)
+        Wt = O.gaussian_bf16((N, K), 0.02, 1000 + it).to(dev).t()
+        full = matmul_tp_persistent(X, Wt, leaf_k=leaf)
+        flb = O.tree_params(K, leaf)[1]
+        for p in (2, 4, 8):
+            # a split is legal when every shard keeps the odd part of the leaf count (or is a single leaf of a pair)
+            if T % p == 0 and (O.tree_params(K // p, leaf)[1] == flb or (flb == 2 and T // p == 1)):
+                assert_bitwise(sim_tp(X, Wt, p, leaf), full, f"case {it} TP={p}")
+        m2 = rng.randint(1, M)
+        assert_bitwise(matmul_tp_persistent(X[:m2], Wt, leaf_k=leaf), full[:m2], f"case {it} prefix {m2}")
+        i = rng.randrange(M)
+        assert_bitwise(matmul_tp_persistent(X[i:i + 1], Wt, leaf_k=leaf), full[i:i + 1], f"case {it} row {i}")
+
+
 def test_reference_smoke_script_shape(dev):
     # simple_matmul.py: M,K,N = 1024,6144,2048, both operands ~ N(0,1), row-major B, TP=4, batch halves
     M, K, N = 1024, 6144, 2048
