@@ -243,15 +243,29 @@ __global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs 
     }
     float sv[8];
     float tmax = -INFINITY;
+    // only the tiles on the causal diagonal need the mask: when every key of the tile is visible to every query of
+    // this wave (a uniform condition) the selects are skipped; the values are the same either way.  Prefill only:
+    // in decode the tile loop is one dependent chain and a branch on a freshly computed value lengthens it.
+    if (!DEEP && __builtin_amdgcn_ballot_w64(k0 + 31 > qpos) == 0) {
 #pragma unroll
-    for (int u = 0; u < 2; u++)
+      for (int u = 0; u < 2; u++)
 #pragma unroll
-      for (int i = 0; i < 4; i++) {
-        const int key = k0 + 16 * u + 4 * g + i;
-        const float v = (key <= qpos) ? s[u][i] * a.scale_log2 : -INFINITY;
-        sv[4 * u + i] = v;
-        tmax = fmaxf(tmax, v);
-      }
+        for (int i = 0; i < 4; i++) {
+          const float v = s[u][i] * a.scale_log2;
+          sv[4 * u + i] = v;
+          tmax = fmaxf(tmax, v);
+        }
+    } else {
+#pragma unroll
+      for (int u = 0; u < 2; u++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const int key = k0 + 16 * u + 4 * g + i;
+          const float v = (key <= qpos) ? s[u][i] * a.scale_log2 : -INFINITY;
+          sv[4 * u + i] = v;
+          tmax = fmaxf(tmax, v);
+        }
+    }
     tmax = xor_step<16, LaneMax>(tmax);
     tmax = xor_step<32, LaneMax>(tmax);
     const float m_new = fmaxf(m, tmax);
@@ -270,6 +284,12 @@ __global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs 
     const uint32_t p0 = pack_bf16x2(pv[0], pv[1]), p1 = pack_bf16x2(pv[2], pv[3]);
     const uint32_t p2 = pack_bf16x2(pv[4], pv[5]), p3 = pack_bf16x2(pv[6], pv[7]);
     const bf16x8 pf = __builtin_bit_cast(bf16x8, u32x4{p0, p1, p2, p3});
+    // rescale the output accumulators only when some row's maximum moved (uniform over the wave): x * 1.0f is x bit
+    // for bit, and after the first tiles of a long row the maximum rarely moves (prefill only, as above)
+    if (DEEP || __builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+      for (int t = 0; t < 8; t++) o[t] = f32x4{o[t][0] * alpha, o[t][1] * alpha, o[t][2] * alpha, o[t][3] * alpha};
+    }
 #pragma unroll
     for (int t = 0; t < 8; t++) {
       const int vr = 16 * t + j;
@@ -277,8 +297,7 @@ __global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs 
       const uint2 va = *reinterpret_cast<const uint2*>(&lds[cur][8192 + vr * 64 + ((g ^ sw) << 3)]);
       const uint2 vb = *reinterpret_cast<const uint2*>(&lds[cur][8192 + vr * 64 + (((4 + g) ^ sw) << 3)]);
       const bf16x8 vf = __builtin_bit_cast(bf16x8, u32x4{va.x, va.y, vb.x, vb.y});
-      f32x4 scaled = {o[t][0] * alpha, o[t][1] * alpha, o[t][2] * alpha, o[t][3] * alpha};
-      o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, scaled, 0, 0, 0);
+      o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[t], 0, 0, 0);
     }
     if (tile + 1 < ntiles) store_tile(cur ^ 1, (d + 1) % DEPTH);
     __syncthreads();
