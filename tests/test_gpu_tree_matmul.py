@@ -228,6 +228,22 @@ def test_random_shapes_tp_batch_and_row_invariance(dev):
         assert_bitwise(matmul_tp_persistent(X[i:i + 1], Wt, leaf_k=leaf), full[i:i + 1], f"case {it} row {i}")
 
 
+@pytest.mark.parametrize("M,K,N,leaf", [(2048, 12288, 4096, 256), (512, 25600, 5120, 128), (128, 12288, 4096, 256), (1, 12288, 4096, 256)])
+def test_repeated_calls_return_the_same_bits(dev, M, K, N, leaf):
+    """Run-to-run determinism under load: 25 back-to-back calls (with other work interleaved on the stream) return
+    the bits of the first one.  Guards the asynchronous parts of the kernels: direct-to-LDS loads, parked tree levels
+    and their read-back, K-cut partials."""
+    print("case", M, K, N, leaf, flush=True)
+    X = O.gaussian_bf16((M, K), 1.0, 3).to(dev)
+    Wt = O.gaussian_bf16((N, K), 0.02, 4).to(dev).t()
+    first = matmul_tp_persistent(X, Wt, leaf_k=leaf)
+    noise = torch.empty(64 << 20, device=dev, dtype=torch.uint8)
+    for i in range(25):
+        noise.fill_(i)                     # evicts caches and reuses freed workspaces between the calls
+        again = matmul_tp_persistent(X, Wt, leaf_k=leaf)
+        assert torch.equal(bits(again), bits(first)), f"call {i} differs"
+
+
 def test_reference_smoke_script_shape(dev):
     # simple_matmul.py: M,K,N = 1024,6144,2048, both operands ~ N(0,1), row-major B, TP=4, batch halves
     M, K, N = 1024, 6144, 2048
