@@ -248,6 +248,42 @@ def test_silu_mul_parity_and_batch_invariance(dev):
     assert ops.bi_silu_mul(z.to(dev)).cpu().tolist() == [[0.0, 80.0, 0, 0, 0, 0, 0, 0]]
 
 
+def test_random_shapes_of_the_reductions(dev):
+    """Seeded sweep over row counts and widths the fixed-shape tests do not visit (hidden sizes that are not powers of
+    two, vocabularies around the 1024-wide pieces, means over inner dimensions): tolerance against fp64 library
+    routines or the oracle, and a random row alone reproduces its bits inside the batch."""
+    import random
+    from llm_reproducibility_amd import ops
+    rng = random.Random(3)
+    for it in range(30):
+        rows = rng.choice([1, 2, 7, 33, 256, 1000])
+        hid = rng.choice([64, 128, 136, 1000, 1024, 2560, 5120, 8192])
+        print("case", it, rows, hid, flush=True)
+        x = O.gaussian_bf16((rows, hid), 1.0, it)
+        w = (1 + 0.1 * torch.randn(hid, generator=torch.Generator().manual_seed(it))).to(torch.bfloat16)
+        got = bio.rms_norm(x.to(dev), w.to(dev), 1e-6)
+        ulp = O.bf16_ulp_distance(got.cpu(), O.rmsnorm(x, w, 1e-6))
+        assert ulp.max() <= 2 and (ulp > 0).float().mean() < 0.02, ("rmsnorm", rows, hid)
+        r = rng.randrange(rows)
+        assert torch.equal(bio.rms_norm(x[r:r + 1].to(dev), w.to(dev), 1e-6), got[r:r + 1]), ("rmsnorm row", rows, hid, r)
+        cols = rng.choice([1, 5, 1023, 1024, 1025, 4096, 32000, 50257, 152064])
+        rows2 = min(rows, 64)
+        lx = 3 * torch.randn((rows2, cols), generator=torch.Generator().manual_seed(100 + it))
+        ls = bio.log_softmax(lx.to(dev))
+        assert (ls.cpu().double() - torch.log_softmax(lx.double(), -1)).abs().max() < 2e-5, ("log_softmax", rows2, cols)
+        r = rng.randrange(rows2)
+        assert torch.equal(bio.log_softmax(lx[r:r + 1].to(dev)), ls[r:r + 1]), ("log_softmax row", rows2, cols, r)
+        assert (bio.softmax(lx.to(dev)).cpu().double() - torch.softmax(lx.double(), -1)).abs().max() < 1e-6, ("softmax", rows2, cols)
+        shp = rng.choice([(rows, 1000), (3, rows, 17), (rows, 5, 64), (2, 3, 4, 5), (rows, 40000)])
+        mx = torch.randn(shp, generator=torch.Generator().manual_seed(200 + it))
+        d = rng.randrange(len(shp))
+        mean = bio.mean_dim(mx.to(dev), d, keepdim=bool(it & 1))
+        assert (mean.cpu().double() - mx.double().mean(d, keepdim=bool(it & 1))).abs().max() < 1e-5, ("mean", shp, d)
+        inter = rng.choice([8, 64, 1000, 12288])
+        gu = O.gaussian_bf16((rows, 2 * inter), 2.0, 300 + it)
+        assert O.bf16_ulp_distance(ops.bi_silu_mul(gu.to(dev)).cpu(), O.silu_mul(gu)).max() <= 1, ("silu_mul", rows, inter)
+
+
 def test_aten_overrides_route_to_the_hip_kernels(dev):
     a = O.gaussian_bf16((20, 512), 1.0, 0).to(dev)
     w = O.gaussian_bf16((64, 512), 0.1, 1).to(dev)
