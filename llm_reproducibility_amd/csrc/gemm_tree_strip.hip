@@ -162,8 +162,8 @@ __global__ __launch_bounds__(64 * S) __attribute__((amdgpu_waves_per_eu(4, 8))) 
 // Waves per strip for a problem, or 0 when this kernel is not the one to use.  Measured on MI355X: HBM bandwidth
 // is shared about equally among the CUs that ask for it, so in a single pass over the weights the CU with the most
 // strips finishes last and every CU has to carry the same number -- a grid of 320 strips (two on every fourth CU)
-// streams at 3 TB/s where 256 or 512 strips reach 5 -- and the activation rows, which every lane fetches for itself, cost as much as the weights once there
-// are more than a few of them (unless the tree has so few aligned subtrees that the K-cut grid of the tiled kernel
+// streams at 3 TB/s where 256 or 512 strips reach 5 -- and the activation rows, which every lane fetches for
+// itself, cost as much as the weights once there are more than a few of them (unless the tree has so few aligned subtrees that the K-cut grid of the tiled kernel
 // cannot fill the chip either).  Four waves per strip are the best cut of K (two chunks of 4 KiB in flight each);
 // beyond a few hundred MB of weights the tiled kernel streams as fast and nothing is gained.
 int gemm_tree_strip_waves(int M, int N, int K, int lb) {
