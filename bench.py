@@ -239,6 +239,11 @@ def main():
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
+        # context, measured in the same run after the timed region: the vendor library's plain GEMM on the same operands
+        # (reduction order not fixed, no tree; not a code path of this library)
+        lib_ms, _ = hip_time_ms(lambda: torch.matmul(X, W.t()), args.steps, args.warmup)
+        out["context"] = {"vendor_gemm_same_operands_TFLOPs": round(flops / (lib_ms * 1e-3) / 1e12, 2),
+                          "note": "torch.matmul (vendor library), reduction order not fixed, no tree"}
     if args.table:
         table(max(args.steps // 2, 5), max(args.warmup // 2, 2), hot=args.table_hot)
     print(json.dumps(out))
