@@ -262,6 +262,16 @@ int bi_qk_norm_rope_cache_bf16(const void* qkv, int64_t ld,
                                int64_t tokens, int q_heads, int kv_heads, int head_dim, int max_len, int batch,
                                float eps, tbik_stream_t stream);
 
+/*
+ * Greedy sampling: out[r] (int64) = index of the largest element of row r of x [rows, cols] (bf16, row stride ld
+ * elements), ties resolved to the lowest index; the pair order (value, then lowest index) is total, so the result
+ * does not depend on how a row is split over lanes.  A NaN is never selected (a row of NaNs gives 0).
+ * Replaces: the token choice of the engine that the reference drives (vllm_generate, simple_inference.py:62-105,
+ *           which samples inside vLLM and compares per-step log-probabilities); for the greedy decoding of the
+ *           end-to-end invariance check the tie rule has to be fixed, which an unordered arg-max does not do.
+ */
+int bi_argmax_bf16(const void* x, int64_t ld, void* out, int64_t rows, int cols, tbik_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

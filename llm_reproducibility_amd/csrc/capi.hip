@@ -16,6 +16,7 @@ int log_softmax_dispatch(const void* x, int64_t ldx, void* out, int64_t ldo, int
 int attention_dispatch(const void* q, const void* k_cache, const void* vt_cache, void* out, const int* q_start,
                        const int* q_len, const int* ctx_len, int batch, int max_q_len, int q_heads, int kv_heads,
                        int head_dim, int max_len, float scale, hipStream_t stream);
+int argmax_dispatch(const void* x, int64_t ld, void* out, int64_t rows, int cols, hipStream_t stream);
 int mean_dispatch(const void* x, void* out, int64_t outer, int64_t n, int64_t inner, int dtype_code, hipStream_t stream);
 int gemm_f32_dispatch(bool tree, const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C,
                       int64_t ldc, int M, int N, int K, int leaf_k, const void* bias, hipStream_t stream);
@@ -29,7 +30,7 @@ int silu_mul_dispatch(const void* gate_up, int64_t ld_in, void* out, int64_t ld_
 
 extern "C" {
 
-int tbik_abi_version(void) { return 8; }
+int tbik_abi_version(void) { return 9; }
 
 const char* tbik_error_string(int code) {
   switch (code) {
@@ -154,6 +155,10 @@ int bi_qk_norm_rope_cache_bf16(const void* qkv, int64_t ld, const void* q_weight
   return tbik::qk_norm_rope_cache_dispatch(qkv, ld, q_weight, k_weight, inv_freq, positions, seq_of_token, q_out, k_cache,
                                            vt_cache, tokens, q_heads, kv_heads, head_dim, max_len, batch, eps,
                                            static_cast<hipStream_t>(stream));
+}
+
+int bi_argmax_bf16(const void* x, int64_t ld, void* out, int64_t rows, int cols, tbik_stream_t stream) {
+  return tbik::argmax_dispatch(x, ld, out, rows, cols, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

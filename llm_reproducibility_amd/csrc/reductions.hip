@@ -384,6 +384,66 @@ static int mean_launch(const void* x, void* out, int64_t outer, int64_t n, int64
   return hip_code(hipGetLastError());
 }
 
+// ------------------------------------------------------------------------------------------------
+// Greedy sampling: index of the largest element of each row, ties resolved to the lowest index (a NaN is never
+// selected; a row of NaNs gives index 0).  "Largest value, then lowest index" is a total order on (value, index)
+// pairs, so the result does not depend on how the row is cut over lanes and waves: batch invariant by construction.
+// One work-group of 1024 threads per row, 16-byte packs of 8 bf16.
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ void argmax_take(float& bv, int& bi, float v, int i) {
+  if (v > bv || (v == bv && i < bi)) {
+    bv = v;
+    bi = i;
+  }
+}
+
+__global__ __launch_bounds__(1024) void argmax_rows_kernel(const uint16_t* x, int64_t ld, int64_t* out, int cols) {
+  __shared__ float sv[16];
+  __shared__ int si[16];
+  const uint16_t* xr = x + (int64_t)blockIdx.x * ld;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+  const bool vec = ((reinterpret_cast<uintptr_t>(xr) & 15) == 0);
+  const int npacks = vec ? cols / 8 : 0;
+  for (int q = tid; q < npacks; q += 1024) {
+    const uint4 pk = *reinterpret_cast<const uint4*>(xr + (int64_t)q * 8);
+    const uint32_t w[4] = {pk.x, pk.y, pk.z, pk.w};
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      argmax_take(bv, bi, bf16_lo(w[e]), q * 8 + 2 * e);
+      argmax_take(bv, bi, bf16_hi(w[e]), q * 8 + 2 * e + 1);
+    }
+  }
+  for (int i = npacks * 8 + tid; i < cols; i += 1024) argmax_take(bv, bi, bf16_bits_to_f32(xr[i]), i);
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    const float ov = __shfl_xor(bv, off);
+    const int oi = __shfl_xor(bi, off);
+    argmax_take(bv, bi, ov, oi);
+  }
+  if (lane == 0) {
+    sv[wave] = bv;
+    si[wave] = bi;
+  }
+  __syncthreads();
+  if (tid == 0) {
+#pragma unroll
+    for (int w = 1; w < 16; w++) argmax_take(bv, bi, sv[w], si[w]);
+    out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
+  }
+}
+
+int argmax_dispatch(const void* x, int64_t ld, void* out, int64_t rows, int cols, hipStream_t stream) {
+  if (rows < 0 || cols <= 0 || ld < cols) return TBIK_ERR_INVALID;
+  if (rows == 0) return TBIK_OK;
+  if (!x || !out || rows > 0x7fffffff) return TBIK_ERR_INVALID;
+  if ((reinterpret_cast<uintptr_t>(x) & 1) || (reinterpret_cast<uintptr_t>(out) & 7)) return TBIK_ERR_ALIGNMENT;
+  hipLaunchKernelGGL(argmax_rows_kernel, dim3((unsigned)rows), dim3(1024), 0, stream, static_cast<const uint16_t*>(x), ld,
+                     static_cast<int64_t*>(out), cols);
+  return hip_code(hipGetLastError());
+}
+
 int mean_dispatch(const void* x, void* out, int64_t outer, int64_t n, int64_t inner, int dtype_code, hipStream_t stream) {
   if (outer < 0 || n <= 0 || inner <= 0) return TBIK_ERR_INVALID;
   if (outer == 0) return TBIK_OK;

@@ -116,10 +116,9 @@ class Qwen3Decoder:
 
     @staticmethod
     def _greedy(logits: torch.Tensor) -> torch.Tensor:
-        """argmax with ties resolved to the lowest index (exact: a max and a min, no order dependence)."""
-        mx = logits.max(dim=-1, keepdim=True).values
-        idx = torch.arange(logits.shape[-1], device=logits.device)
-        return torch.where(logits == mx, idx, logits.shape[-1]).min(dim=-1).values
+        """argmax with ties resolved to the lowest index (a total order on (value, index): no dependence on how the
+        row is reduced)."""
+        return ops.bi_argmax(logits)
 
     # ------------------------------------------------------------------------------------------
     @torch.no_grad()

@@ -417,3 +417,15 @@ def bi_qk_norm_rope_cache_bf16(qkv: torch.Tensor, q_weight: torch.Tensor, k_weig
         k_cache.shape[2], k_cache.shape[0], eps, _stream(qkv))
     _lib.check(rc, "bi_qk_norm_rope_cache_bf16")
     return q_out
+
+
+def bi_argmax(logits: torch.Tensor) -> torch.Tensor:
+    """Index (int64) of the largest element of each row of a 2-D bf16 tensor, ties resolved to the lowest index."""
+    _require_gpu(logits)
+    if logits.dim() != 2 or logits.dtype != torch.bfloat16:
+        raise NotImplementedError("bi_argmax takes a 2-D bfloat16 tensor")
+    x = logits if logits.stride(1) == 1 else logits.contiguous()
+    out = torch.empty((x.shape[0],), device=x.device, dtype=torch.int64)
+    rc = _lib.lib().bi_argmax_bf16(x.data_ptr(), x.stride(0) if x.shape[0] > 1 else max(x.stride(0), x.shape[1]), out.data_ptr(), x.shape[0], x.shape[1], _stream(x))
+    _lib.check(rc, "bi_argmax_bf16")
+    return out

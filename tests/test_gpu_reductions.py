@@ -284,6 +284,27 @@ def test_random_shapes_of_the_reductions(dev):
         assert O.bf16_ulp_distance(ops.bi_silu_mul(gu.to(dev)).cpu(), O.silu_mul(gu)).max() <= 1, ("silu_mul", rows, inter)
 
 
+def test_argmax_lowest_index_on_ties(dev):
+    from llm_reproducibility_amd import ops
+    g = torch.Generator().manual_seed(7)
+    for rows, cols in ((1, 151936), (7, 151936), (128, 151936), (3, 5), (4, 1000), (2, 8), (5, 1031)):
+        x = torch.randn((rows, cols), generator=g).to(torch.bfloat16)   # bf16 values collide often: many ties
+        want = torch.where(x == x.max(dim=-1, keepdim=True).values, torch.arange(cols), cols).min(dim=-1).values
+        got = ops.bi_argmax(x.to(dev))
+        assert got.dtype == torch.int64 and torch.equal(got.cpu(), want), (rows, cols)
+        r = rows - 1
+        assert torch.equal(ops.bi_argmax(x[r:r + 1].to(dev)), got[r:r + 1]), "row alone"
+    flat = torch.zeros((3, 4096), dtype=torch.bfloat16)
+    flat[1, 77] = -0.0
+    flat[2] = -1
+    flat[2, 4000] = 5
+    flat[2, 123] = 5
+    assert ops.bi_argmax(flat.to(dev)).tolist() == [0, 0, 123]
+    wide = torch.randn((6, 300), generator=g).to(torch.bfloat16).to(dev)
+    view = wide[:, 3:203]                                                # strided, 2-byte aligned rows
+    assert torch.equal(ops.bi_argmax(view), ops.bi_argmax(view.contiguous()))
+
+
 def test_aten_overrides_route_to_the_hip_kernels(dev):
     a = O.gaussian_bf16((20, 512), 1.0, 0).to(dev)
     w = O.gaussian_bf16((64, 512), 0.1, 1).to(dev)
