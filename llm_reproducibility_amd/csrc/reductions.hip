@@ -406,13 +406,23 @@ __global__ __launch_bounds__(1024) void argmax_rows_kernel(const uint16_t* x, in
   int bi = 0x7fffffff;
   const bool vec = ((reinterpret_cast<uintptr_t>(xr) & 15) == 0);
   const int npacks = vec ? cols / 8 : 0;
-  for (int q = tid; q < npacks; q += 1024) {
-    const uint4 pk = *reinterpret_cast<const uint4*>(xr + (int64_t)q * 8);
-    const uint32_t w[4] = {pk.x, pk.y, pk.z, pk.w};
+  // eight packs in flight per thread (a pack past the end re-reads the last one and is skipped): one round trip
+  // covers 64 Ki elements of the row
+  for (int q0 = tid; q0 < npacks; q0 += 8 * 1024) {
+    uint4 pk[8];
 #pragma unroll
-    for (int e = 0; e < 4; e++) {
-      argmax_take(bv, bi, bf16_lo(w[e]), q * 8 + 2 * e);
-      argmax_take(bv, bi, bf16_hi(w[e]), q * 8 + 2 * e + 1);
+    for (int u = 0; u < 8; u++) pk[u] = *reinterpret_cast<const uint4*>(xr + (int64_t)min(q0 + u * 1024, npacks - 1) * 8);
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+      const int q = q0 + u * 1024;
+      if (q < npacks) {
+        const uint32_t w[4] = {pk[u].x, pk[u].y, pk[u].z, pk[u].w};
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          argmax_take(bv, bi, bf16_lo(w[e]), q * 8 + 2 * e);
+          argmax_take(bv, bi, bf16_hi(w[e]), q * 8 + 2 * e + 1);
+        }
+      }
     }
   }
   for (int i = npacks * 8 + tid; i < cols; i += 1024) argmax_take(bv, bi, bf16_bits_to_f32(xr[i]), i);
