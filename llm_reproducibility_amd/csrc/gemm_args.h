@@ -32,6 +32,7 @@ struct QuadArgs {
   int vec_store;
 };
 int gemm_single_acc_quad_launch(const QuadArgs& a, hipStream_t stream);
+int gemm_single_acc_slab_launch(const QuadArgs& a, hipStream_t stream);  // at most 128 rows; TBIK_ERR_UNSUPPORTED: use another kernel
 
 // gemm_single_acc_stream.hip: single-accumulator 16-bit GEMM for at most 64 rows, weights streamed from global memory
 struct StreamArgs {

@@ -18,18 +18,28 @@
 namespace tbik {
 
 namespace quad {
-constexpr int BM = 128, BN = 256, BK = 64, NT = 256, NWAVE = 4, TM = 4, TN = 8;
-constexpr int ROWS = BM + BN, STAGE_BYTES = ROWS * BK * 2, NSLOT = 3;
-constexpr int NDMA = ROWS / 8 / NWAVE;  // 12 direct loads per wave per slice (8 rows of 128 B each)
-constexpr int XDMA = BM / 8 / NWAVE;    // of which X rows: 4
+constexpr int BM = 128, BK = 64, NT = 256, NWAVE = 4, TM = 4, NSLOT = 3;
+constexpr int XDMA = BM / 8 / NWAVE;    // direct loads of X rows per wave per slice: 4 (8 rows of 128 B each)
+template <int TN>
+struct Shape {
+  static constexpr int BN = 2 * TN * 16;          // two waves across N, TN MFMA tiles each
+  static constexpr int ROWS = BM + BN;
+  static constexpr int STAGE_BYTES = ROWS * BK * 2;
+  static constexpr int NDMA = ROWS / 8 / NWAVE;   // direct loads per wave per slice: 12 for the 256-wide tile
+};
 }  // namespace quad
 
 __device__ __forceinline__ void quad_dma16(uint32_t lds_addr, uint32_t voff, const void* base) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(base) : "memory");
 }
 
+// TN = 8: the 128x256 tile of the large shapes.  TN = 1..4: the same pipeline on 128x32 .. 128x128 tiles for 33..128
+// rows, where the call is one pass over the weights and the tile width is chosen so that every CU gets the same
+// number of work-groups.
+template <int TN>
 __global__ __launch_bounds__(quad::NT) void gemm_single_acc_quad_kernel(const QuadArgs p) {
   using namespace quad;
+  constexpr int BN = Shape<TN>::BN, STAGE_BYTES = Shape<TN>::STAGE_BYTES, NDMA = Shape<TN>::NDMA;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -101,30 +111,36 @@ __global__ __launch_bounds__(quad::NT) void gemm_single_acc_quad_kernel(const Qu
     const int pslot = slot == 0 ? NSLOT - 1 : slot - 1;
 #pragma unroll
     for (int kk = 0; kk < 2; kk++) {
+      // The MFMAs of a k step go out in groups; behind every group follow two fragment reads of the next k step
+      // ((s,1) from this slot, or (s+1,0) from the next slot, which the mid-slice barrier has made visible) and one
+      // direct load: slice s+3 goes into the slot slice s vacates at the mid-slice barrier (first half of its loads
+      // in the second k step of s, second half in the first k step of s+1).  The 256-wide tile has eight groups of
+      // four MFMAs (half a row of tiles each), the narrow tiles four groups of one row.
+      constexpr int NG = TN == 8 ? 8 : 4;
+      constexpr int H1 = (NDMA + 1) / 2, H2 = NDMA - H1;
+      static_assert(H1 <= NG && TM + TN <= 2 * NG, "schedule does not fit the groups");
 #pragma unroll
-      for (int q = 0; q < 8; q++) {
+      for (int q = 0; q < NG; q++) {
+        const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+        if constexpr (TN == 8) {
 #pragma unroll
-        for (int bb = 0; bb < 4; bb++) {
-          const int a = q >> 1, b = (q & 1) * 4 + bb;
-          const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-          acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[kk][b], fx[kk][a], (s == 0 && kk == 0) ? zero : acc[a][b], 0, 0, 0);
-        }
-        // fragments of the next k step: (s,1) from this slot, or (s+1,0) from the next slot, which the mid-slice
-        // barrier has made visible
-        if (q < 6) {
-          const int rslot = kk == 0 ? slot : nslot;
-          if (q < 2) {
-            read_x(kk ^ 1, rslot, kk ^ 1, 2 * q);
-            read_x(kk ^ 1, rslot, kk ^ 1, 2 * q + 1);
-          } else {
-            read_w(kk ^ 1, rslot, kk ^ 1, 2 * (q - 2));
-            read_w(kk ^ 1, rslot, kk ^ 1, 2 * (q - 2) + 1);
+          for (int bb = 0; bb < 4; bb++) {
+            const int a = q >> 1, b = (q & 1) * 4 + bb;
+            acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[kk][b], fx[kk][a], (s == 0 && kk == 0) ? zero : acc[a][b], 0, 0, 0);
           }
+        } else {
+#pragma unroll
+          for (int b = 0; b < TN; b++)
+            acc[q][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[kk][b], fx[kk][q], (s == 0 && kk == 0) ? zero : acc[q][b], 0, 0, 0);
         }
-        // operand prefetch, one load per group: slice s+3 goes into the slot slice s vacates at the mid-slice
-        // barrier (first half of its loads in the second k step of s, second half in the first k step of s+1)
-        if (kk == 1 && q < NDMA / 2) dma_one(s + 3, slot, q);
-        if (kk == 0 && q < NDMA / 2 && s > 0) dma_one(s + 2, pslot, NDMA / 2 + q);
+        const int rslot = kk == 0 ? slot : nslot;
+#pragma unroll
+        for (int f = 2 * q; f < 2 * q + 2; f++) {
+          if (f < TM) read_x(kk ^ 1, rslot, kk ^ 1, f);
+          else if (f - TM < TN) read_w(kk ^ 1, rslot, kk ^ 1, f - TM);
+        }
+        if (kk == 1 && q < H1) dma_one(s + 3, slot, q);
+        if (kk == 0 && q < H2 && s > 0) dma_one(s + 2, pslot, H1 + q);
         __builtin_amdgcn_sched_barrier(0);
       }
       if (kk == 0) {
@@ -166,17 +182,51 @@ __global__ __launch_bounds__(quad::NT) void gemm_single_acc_quad_kernel(const Qu
   }
 }
 
-int gemm_single_acc_quad_launch(const QuadArgs& a, hipStream_t stream) {
+template <int TN>
+static int quad_launch(const QuadArgs& a, hipStream_t stream) {
   using namespace quad;
-  constexpr size_t smem = (size_t)NSLOT * STAGE_BYTES;  // 144 KiB
+  constexpr int BN = Shape<TN>::BN;
+  constexpr size_t smem = (size_t)NSLOT * Shape<TN>::STAGE_BYTES;  // 144 KiB for the 256-wide tile
   const int64_t tiles = (int64_t)((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
   if (tiles <= 0 || tiles > 0x7fffffff || a.K < BK || (a.K % BK) != 0) return TBIK_ERR_UNSUPPORTED;
   if (a.ldx >= (1 << 22) || a.ldw >= (1 << 22)) return TBIK_ERR_UNSUPPORTED;  // 32-bit in-tile byte offsets
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_single_acc_quad_kernel),
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_single_acc_quad_kernel<TN>),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
   if (e != hipSuccess) return hip_code(e);
-  hipLaunchKernelGGL(gemm_single_acc_quad_kernel, dim3((unsigned)tiles), dim3(NT), smem, stream, a);
+  hipLaunchKernelGGL(gemm_single_acc_quad_kernel<TN>, dim3((unsigned)tiles), dim3(NT), smem, stream, a);
   return hip_code(hipGetLastError());
+}
+
+int gemm_single_acc_quad_launch(const QuadArgs& a, hipStream_t stream) { return quad_launch<8>(a, stream); }
+
+// 33..128 rows: one row of tiles, so the call is one pass over the weights.  A work-group's time is set by the
+// length of K (the ring is a chain of slices, each about a memory round trip), not by the width of its tile, so the
+// whole grid has to be resident at once: at most one work-group per CU for the 96- and 128-column tiles (84 and
+// 96 KiB of LDS), two for the 32- and 64-column ones.  Among the widths that fit, the one that leaves the fewest
+// of those slots idle wins (HBM bandwidth is shared about equally among the CUs), wider tiles preferred on ties
+// because they re-read the activations less often.  Returns TBIK_ERR_UNSUPPORTED when no width qualifies (wide
+// weight matrices run faster on the 256-column tile even with idle CUs: 110 against 214 us at N=51200).
+int gemm_single_acc_slab_launch(const QuadArgs& a, hipStream_t stream) {
+  if (a.M <= 0 || a.M > quad::BM) return TBIK_ERR_UNSUPPORTED;
+  int best = 0;
+  double best_score = 0.0;
+  for (int tn = 4; tn >= 1; tn--) {
+    const int64_t tiles = ((int64_t)a.N + 32 * tn - 1) / (32 * tn);
+    const int64_t slots = tn <= 2 ? 512 : 256;
+    if (tiles < 128 || tiles > slots) continue;
+    const double score = (double)tiles / (double)(((tiles + 255) / 256) * 256) * (1.0 + 0.01 * tn);
+    if (score > best_score) {
+      best_score = score;
+      best = tn;
+    }
+  }
+  switch (best) {
+    case 4: return quad_launch<4>(a, stream);
+    case 3: return quad_launch<3>(a, stream);
+    case 2: return quad_launch<2>(a, stream);
+    case 1: return quad_launch<1>(a, stream);
+    default: return TBIK_ERR_UNSUPPORTED;
+  }
 }
 
 }  // namespace tbik

@@ -435,6 +435,13 @@ int gemm_dispatch(bool tree, bool f16, const void* A, int64_t lda, const void* B
     // large problems whose K is a whole number of 64-wide slices take the one-wave-per-SIMD pipeline (same MFMA
     // chain per element, so the same bits as the tiled kernel)
     const int64_t wide_tiles = (int64_t)((M + 127) / 128) * ((N + 255) / 256);
+    // 33..128 rows: one row of 128-row tiles whose width balances the grid, when such a grid exists (same MFMA chain
+    // per element again; measured faster than the streaming kernel from 33 rows on)
+    if (!f16 && M > 32 && M <= 128 && (K & 63) == 0 && lda < (1 << 22) && ldb_n < (1 << 22)) {
+      QuadArgs qa{a.X, a.W, a.C, a.bias, a.ldx, a.ldw, a.ldc, M, N, K, a.vec_store};
+      const int rc = gemm_single_acc_slab_launch(qa, stream);
+      if (rc != TBIK_ERR_UNSUPPORTED) return rc;
+    }
     if (!f16 && M > 64 && wide_tiles >= 128 && (K & 63) == 0 && lda < (1 << 22) && ldb_n < (1 << 22)) {
       QuadArgs qa{a.X, a.W, a.C, a.bias, a.ldx, a.ldw, a.ldc, M, N, K, a.vec_store};
       return gemm_single_acc_quad_launch(qa, stream);

@@ -141,13 +141,27 @@ def test_single_accumulator_mm_large_and_small_kernels_agree_bitwise(dev):
     bias = O.gaussian_bf16((4096,), 1.0, 7)
     ad, wd, bd = a.to(dev), w.to(dev), bias.to(dev)
     full = bio.matmul_persistent(ad, wd.t(), bd)
-    for m in (1, 3, 16, 17, 33, 48, 64, 300):          # every row-block count of the streaming kernels, then the tiled one
+    for m in (1, 3, 16, 17, 32, 33, 48, 64, 128, 300):  # streaming kernels, the one-round 128-row tiles (33..128), the tiled one
         assert torch.equal(bio.matmul_persistent(ad[:m], wd.t(), bd), full[:m]), m
     want = O.matmul_single_acc(a[:256], w.t(), bias)
     assert not O.outside_tolerance(full[:256], want).any()
     ai = O.integer_bf16((2048, 512), -9, 9, 8)
     wi = O.integer_bf16((4096, 512), -7, 7, 9)
     assert torch.equal(bio.matmul_persistent(ai.to(dev), wi.to(dev).t()).cpu(), O.matmul_single_acc(ai, wi.t()))
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 6144, 4096), (65, 8200, 1024), (33, 24576, 512), (100, 16384, 512), (128, 16400, 256), (40, 12296, 1088)])
+def test_single_accumulator_mm_one_round_tiles_match_oracle_bitwise(dev, M, N, K):
+    """33..128 rows on a grid of 128-row tiles that is resident at once (tile widths 32, 64, 96 and 128, ragged last
+    tiles, bias): integer inputs, so the oracle's bits are the only right answer."""
+    print("case", M, N, K, flush=True)
+    a = O.integer_bf16((M, K), -9, 9, 21)
+    w = O.integer_bf16((N, K), -7, 7, 22)
+    bias = O.integer_bf16((N,), -5, 5, 23)
+    got = bio.matmul_persistent(a.to(dev), w.to(dev).t(), bias.to(dev))
+    assert torch.equal(got.cpu(), O.matmul_single_acc(a, w.t(), bias))
+    row = bio.matmul_persistent(a[M - 1:M].to(dev), w.to(dev).t(), bias.to(dev))   # the same row through the streaming kernel
+    assert torch.equal(row, got[M - 1:M])
 
 
 def test_single_accumulator_mm_streaming_kernels_on_ragged_shapes(dev):
