@@ -4,7 +4,8 @@
  * Every entry point
  *   - takes plain device pointers, sizes and element strides (no torch types),
  *   - enqueues its kernels on the caller's `stream` (a hipStream_t; NULL = the default stream),
- *   - allocates nothing, synchronises nothing, keeps no mutable global state (re-entrant),
+ *   - allocates nothing, synchronises nothing and is re-entrant; the only state it keeps is a once-per-device
+ *     flag per kernel that remembers that the kernel's dynamic-LDS limit has been raised on that device,
  *   - validates shapes / alignment on the host BEFORE launching and returns a TBIK_* code
  *     (0 = success); codes >= TBIK_ERR_HIP_BASE are TBIK_ERR_HIP_BASE + hipError_t.
  *
@@ -185,6 +186,14 @@ int tbik_gemm_f16(const void* A, int64_t lda,
                   void* workspace, size_t workspace_bytes,
                   tbik_stream_t stream);
 int tbik_tree_combine_f16(const void* const* parts, int nparts, void* out, int64_t numel, tbik_stream_t stream);
+/*
+ * The same adjacent-pair tree over fp32 partials (a node is one fp32 addition; 4-byte aligned buffers, 16-byte
+ * aligned ones take the vector path).
+ * Replaces: the float instantiation of the reference's tree reduce,
+ *           mini_allreduce/tbik_kernel/csrc/allreduce/custom_all_reduce.cuh:203-234 (instantiated for float in custom_all_reduce.cu:118-122), and the
+ *           local adds of tree_all_reduce_sum_native on float32 tensors, src/tbik/tree_based_all_reduce.py:32-37.
+ */
+int tbik_tree_combine_f32(const void* const* parts, int nparts, void* out, int64_t numel, tbik_stream_t stream);
 int bi_gemm_f16(const void* A, int64_t lda,
                 const void* B, int64_t ldb_k, int64_t ldb_n,
                 void* C, int64_t ldc,

@@ -11,7 +11,7 @@ import os
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG_DIR, "libtbik_hip.so")
 
-ABI_VERSION = 9
+ABI_VERSION = 10
 TBIK_OK = 0
 TBIK_ERR_INVALID = 1
 TBIK_ERR_ALIGNMENT = 2
@@ -20,7 +20,7 @@ TBIK_ERR_WORKSPACE = 4
 
 EXPORTS = (
     "tbik_abi_version", "tbik_error_string", "tbik_tree_params", "tbik_gemm_bf16", "tbik_gemm_workspace_bytes",
-    "tbik_tree_combine_bf16",
+    "tbik_tree_combine_bf16", "tbik_tree_combine_f32",
     "bi_gemm_bf16", "bi_rmsnorm_bf16", "bi_log_softmax_workspace_bytes", "bi_log_softmax_f32", "bi_mean_dim", "bi_attention_bf16", "bi_silu_mul_bf16",
     "tbik_gemm_f16", "tbik_gemm_f16_workspace_bytes", "tbik_tree_combine_f16", "bi_gemm_f16", "tbik_gemm_f32", "bi_gemm_f32", "bi_rmsnorm_f16", "bi_silu_mul_f16", "bi_qk_norm_rope_cache_bf16", "bi_argmax_bf16",
 )
@@ -74,6 +74,8 @@ def lib() -> ctypes.CDLL:
     L.tbik_gemm_f16_workspace_bytes.restype = sz
     L.tbik_tree_combine_f16.argtypes = L.tbik_tree_combine_bf16.argtypes
     L.tbik_tree_combine_f16.restype = i32
+    L.tbik_tree_combine_f32.argtypes = L.tbik_tree_combine_bf16.argtypes
+    L.tbik_tree_combine_f32.restype = i32
     L.bi_gemm_f16.argtypes = L.bi_gemm_bf16.argtypes
     L.bi_gemm_f16.restype = i32
     L.tbik_gemm_f32.argtypes = [vp, i64, vp, i64, i64, vp, i64, i32, i32, i32, i32, vp, vp]

@@ -8,6 +8,7 @@ int gemm_dispatch(bool tree, bool f16, const void* A, int64_t lda, const void* B
                   hipStream_t stream);
 size_t gemm_workspace_bytes(int M, int N, int K, int leaf_k, bool f16);
 int tree_combine_dispatch(const void* const* parts, int nparts, void* out, int64_t numel, bool f16, hipStream_t stream);
+int tree_combine_f32_dispatch(const void* const* parts, int nparts, void* out, int64_t numel, hipStream_t stream);
 int rmsnorm_dispatch(const void* x, int64_t ldx, const void* res, int64_t ldr, const void* w, void* out, int64_t ldo,
                      void* res_out, int64_t ldro, int64_t rows, int hidden, float eps, bool f16, hipStream_t stream);
 size_t lsm_workspace_bytes(int64_t rows, int64_t cols);
@@ -30,7 +31,7 @@ int silu_mul_dispatch(const void* gate_up, int64_t ld_in, void* out, int64_t ld_
 
 extern "C" {
 
-int tbik_abi_version(void) { return 9; }
+int tbik_abi_version(void) { return 10; }
 
 const char* tbik_error_string(int code) {
   switch (code) {
@@ -79,6 +80,10 @@ int tbik_gemm_f16(const void* A, int64_t lda, const void* B, int64_t ldb_k, int6
 
 int tbik_tree_combine_f16(const void* const* parts, int nparts, void* out, int64_t numel, tbik_stream_t stream) {
   return tbik::tree_combine_dispatch(parts, nparts, out, numel, true, static_cast<hipStream_t>(stream));
+}
+
+int tbik_tree_combine_f32(const void* const* parts, int nparts, void* out, int64_t numel, tbik_stream_t stream) {
+  return tbik::tree_combine_f32_dispatch(parts, nparts, out, numel, static_cast<hipStream_t>(stream));
 }
 
 int bi_gemm_f16(const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C, int64_t ldc, int M,

@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/tbik_hip.h"
 
 namespace tbik {
@@ -115,5 +117,19 @@ __device__ __forceinline__ float wave_sum(float v) { return wave_reduce<LaneSum>
 __device__ __forceinline__ float wave_max(float v) { return wave_reduce<LaneMax>(v); }
 
 inline int hip_code(hipError_t e) { return e == hipSuccess ? TBIK_OK : TBIK_ERR_HIP_BASE + (int)e; }
+
+// Raises a kernel's dynamic-LDS limit the first time the kernel is launched on a device.  The limit is a property of
+// the loaded function on that device, so setting it again on every launch only costs host time on the decode path.
+// `done` is one flag word per kernel instantiation (a function-local static at the call site), one bit per device.
+inline hipError_t ensure_dynamic_lds(const void* kern, int bytes, std::atomic<uint64_t>& done) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
+    return hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  const uint64_t bit = 1ull << dev;
+  if (done.load(std::memory_order_acquire) & bit) return hipSuccess;
+  const hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e == hipSuccess) done.fetch_or(bit, std::memory_order_release);
+  return e;
+}
 
 }  // namespace tbik

@@ -61,7 +61,8 @@ int gemm_tree_strip_waves(int M, int N, int K, int lb);  // waves per strip, or 
 int gemm_tree_strip_launch(const StripArgs& a, int leaf_k, int waves, bool f16, hipStream_t stream);
 
 // tree_combine.hip
+// ldo != 0: `out` is a [numel / N, N] matrix with row stride ldo (the partials stay contiguous)
 int tree_combine_bias_dispatch(const void* const* parts, int nparts, void* out, int64_t numel, const void* bias, int N,
-                               bool f16, hipStream_t stream);
+                               bool f16, hipStream_t stream, int64_t ldo = 0);
 
 }  // namespace tbik

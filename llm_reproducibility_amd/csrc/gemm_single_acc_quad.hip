@@ -30,7 +30,9 @@ struct Shape {
 }  // namespace quad
 
 __device__ __forceinline__ void quad_dma16(uint32_t lds_addr, uint32_t voff, const void* base) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(base) : "memory");
+  // wait states inside the statement (the compiler cannot see the instructions): five between a vector instruction
+  // that wrote a scalar operand and the load that reads it, one between the write of m0 and the load; m0 is clobbered
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(base) : "memory", "m0");
 }
 
 // TN = 8: the 128x256 tile of the large shapes.  TN = 1..4: the same pipeline on 128x32 .. 128x128 tiles for 33..128
@@ -190,8 +192,8 @@ static int quad_launch(const QuadArgs& a, hipStream_t stream) {
   const int64_t tiles = (int64_t)((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
   if (tiles <= 0 || tiles > 0x7fffffff || a.K < BK || (a.K % BK) != 0) return TBIK_ERR_UNSUPPORTED;
   if (a.ldx >= (1 << 22) || a.ldw >= (1 << 22)) return TBIK_ERR_UNSUPPORTED;  // 32-bit in-tile byte offsets
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_single_acc_quad_kernel<TN>),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+  static std::atomic<uint64_t> done{0};
+  hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(gemm_single_acc_quad_kernel<TN>), (int)smem, done);
   if (e != hipSuccess) return hip_code(e);
   hipLaunchKernelGGL(gemm_single_acc_quad_kernel<TN>, dim3((unsigned)tiles), dim3(NT), smem, stream, a);
   return hip_code(hipGetLastError());

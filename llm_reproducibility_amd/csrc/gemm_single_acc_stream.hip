@@ -238,7 +238,8 @@ static int stream_launch_nw(const StreamArgs& a, hipStream_t stream) {
   constexpr int smem = 2 * MB * 16 * stream::rowb(WS);
   auto kern = gemm_single_acc_stream_kernel<MB, WS, NWAVES, F16>;
   if (smem > 64 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    static std::atomic<uint64_t> done{0};
+    hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, done);
     if (e != hipSuccess) return hip_code(e);
   }
   hipLaunchKernelGGL(kern, dim3((unsigned)groups), dim3(NWAVES * 64), smem, stream, a);

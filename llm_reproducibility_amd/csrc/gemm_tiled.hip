@@ -309,8 +309,8 @@ static int launch(const GemmArgs& a, int split, hipStream_t stream) {
   constexpr size_t smem = (size_t)2 * (BM + BN) * BK * sizeof(uint16_t);
   auto kern = gemm_kernel<WAVES_M, WAVES_N, TM, TN, LS, LBMAX, TREE, F16>;
   if (smem > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    static std::atomic<uint64_t> done{0};
+    hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), (int)smem, done);
     if (e != hipSuccess) return hip_code(e);
   }
   const int64_t tiles = (int64_t)((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
@@ -495,13 +495,8 @@ int gemm_dispatch(bool tree, bool f16, const void* A, int64_t lda, const void* B
   if (rc != TBIK_OK || pl.split == 1) return rc;
   const void* parts[32];
   for (int i = 0; i < pl.split; i++) parts[i] = wsb + (size_t)i * M * N * sizeof(uint16_t);
-  if (ldc == N) return tree_combine_bias_dispatch(parts, pl.split, C, (int64_t)M * N, bias, N, f16, stream);
-  for (int m = 0; m < M && rc == TBIK_OK; m++) {  // strided C (rare): row by row
-    const void* rp[32];
-    for (int i = 0; i < pl.split; i++) rp[i] = static_cast<const uint8_t*>(parts[i]) + (size_t)m * N * sizeof(uint16_t);
-    rc = tree_combine_bias_dispatch(rp, pl.split, static_cast<uint16_t*>(C) + (int64_t)m * ldc, N, bias, N, f16, stream);
-  }
-  return rc;
+  // one launch adds the shards (and the bias) in tree order, into C's own row stride
+  return tree_combine_bias_dispatch(parts, pl.split, C, (int64_t)M * N, bias, N, f16, stream, ldc);
 }
 
 }  // namespace tbik

@@ -48,18 +48,23 @@ size_t wide_workspace_bytes(int M, int N, int lb, int split) {
 }
 
 // One 16-byte-per-lane direct global->LDS load: lane l's 16 bytes land at lds_addr + 16*l.
+// The compiler cannot see inside the statement, so the statement carries its own wait states: a vector-memory
+// instruction must not read a scalar register less than five states after a vector instruction wrote it (which is
+// how a spilled scalar comes back: v_readlane_b32), and the load must not follow the write of m0 directly.  m0 is
+// declared clobbered so that the compiler never keeps a value of its own there.
 __device__ __forceinline__ void dma16(uint32_t lds_addr, uint32_t voff, const void* base) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %1, %2"
                :
                : "s"(lds_addr), "v"(voff), "s"(base)
-               : "memory");
+               : "memory", "m0");
 }
 
 // 16-byte-per-lane store to (wave-uniform base) + voff, scalar-base addressing: no per-lane 64-bit pointer.
 __device__ __forceinline__ void store16_sbase(void* base, uint32_t voff, u32x4 v) {
-  // the wait states keep the next instruction from overwriting the data registers while the store still reads
-  // them (a hazard the compiler handles for its own stores, but cannot see inside an asm statement)
-  asm volatile("global_store_dwordx4 %0, %1, %2\n\ts_nop 1" : : "v"(voff), "v"(v), "s"(base) : "memory");
+  // the wait states behind the store keep the next instruction from overwriting the data registers while the store
+  // still reads them, the ones in front of it cover a scalar base that a vector instruction has just written
+  // (hazards the compiler handles for its own instructions, but cannot see inside an asm statement)
+  asm volatile("s_nop 4\n\tglobal_store_dwordx4 %0, %1, %2\n\ts_nop 1" : : "v"(voff), "v"(v), "s"(base) : "memory");
 }
 
 // TREE = false: the same pipeline with ONE fp32 accumulator run over all of K (the batch-invariant mm); T counts
@@ -381,17 +386,20 @@ int gemm_tree_wide_launch(const WideArgs& a, int leaf_k, int split, hipStream_t 
   if (a.ldx >= (1 << 22) || a.ldw >= (1 << 22)) return TBIK_ERR_UNSUPPORTED;  // 32-bit in-tile byte offsets
   if (leaf_k == 256) {
     auto kern = gemm_tree_wide_kernel<4>;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    static std::atomic<uint64_t> done{0};
+    hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), (int)smem, done);
     if (e != hipSuccess) return hip_code(e);
     hipLaunchKernelGGL(kern, dim3((unsigned)tiles, (unsigned)split), dim3(NT), smem, stream, a);
   } else if (leaf_k == 0) {  // single accumulator over K (a multiple of 256)
     auto kern = gemm_tree_wide_kernel<4, false>;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    static std::atomic<uint64_t> done{0};
+    hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), (int)smem, done);
     if (e != hipSuccess) return hip_code(e);
     hipLaunchKernelGGL(kern, dim3((unsigned)tiles, 1u), dim3(NT), smem, stream, a);
   } else if (leaf_k == 128) {
     auto kern = gemm_tree_wide_kernel<2>;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    static std::atomic<uint64_t> done{0};
+    hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), (int)smem, done);
     if (e != hipSuccess) return hip_code(e);
     hipLaunchKernelGGL(kern, dim3((unsigned)tiles, (unsigned)split), dim3(NT), smem, stream, a);
   } else {

@@ -37,10 +37,17 @@ class DecoderConfig:
     rms_eps: float = 1e-6
 
 
+def _normal_bf16(shape, gen: torch.Generator, device) -> torch.Tensor:
+    """N(0, 0.02) in bf16 on `device`, drawn where the generator lives (CPU: the same values on every machine;
+    GPU: seconds instead of minutes for the 8B-parameter configuration)."""
+    w = torch.randn(shape, generator=gen, dtype=torch.float32, device=gen.device)
+    return w.mul_(0.02).to(torch.bfloat16).to(device)
+
+
 class _Layer:
     def __init__(self, cfg: DecoderConfig, tp_size: int, gen: torch.Generator, device):
         def w(*shape):
-            return (torch.randn(shape, generator=gen, dtype=torch.float32) * 0.02).to(torch.bfloat16).to(device)
+            return _normal_bf16(shape, gen, device)
         H, D = cfg.hidden_size, cfg.head_dim
         self.input_norm = torch.ones(H, dtype=torch.bfloat16, device=device)
         self.post_norm = torch.ones(H, dtype=torch.bfloat16, device=device)
@@ -54,21 +61,30 @@ class _Layer:
 
 class Qwen3Decoder:
     def __init__(self, cfg: DecoderConfig, tp_size: int = 1, seed: int = 0, device="cuda:0", use_graphs: bool = False,
-                 fused_rope: bool = True):
+                 fused_rope: bool = True, init_on_device: bool = False):
         assert cfg.head_dim == 128, "the attention kernel is built for head_dim 128"
         self.cfg, self.tp_size, self.device = cfg, tp_size, torch.device(device)
         # decode steps replayed from one captured HIP graph (same kernels, same order, same bits as eager; the
         # per-step host work shrinks to one graph launch, which is what bounds small batches)
         self.use_graphs = use_graphs
         self.fused_rope = fused_rope
-        gen = torch.Generator().manual_seed(seed)
-        emb = lambda *shape: (torch.randn(shape, generator=gen, dtype=torch.float32) * 0.02).to(torch.bfloat16).to(self.device)  # noqa: E731
+        gen = torch.Generator(device=self.device if init_on_device else "cpu").manual_seed(seed)
+        emb = lambda *shape: _normal_bf16(shape, gen, self.device)  # noqa: E731
         self.embed = emb(cfg.vocab_size, cfg.hidden_size)
         self.layers = [_Layer(cfg, tp_size, gen, self.device) for _ in range(cfg.num_layers)]
         self.final_norm = torch.ones(cfg.hidden_size, dtype=torch.bfloat16, device=self.device)
         self.lm_head = emb(cfg.vocab_size, cfg.hidden_size)
         self.inv_freq = compute_inv_freq(cfg.head_dim, cfg.rope_theta, self.device)  # fp32 table built on the CPU
         self.scale = 1.0 / math.sqrt(cfg.head_dim)
+
+    def set_tp(self, tp_size: int) -> None:
+        """Re-shard the row-split layers (o_proj, down_proj) of THIS model over `tp_size` simulated ranks: the
+        weights stay where they are, only the K slices and the shard tree change."""
+        for layer in self.layers:
+            for lin in (layer.o_proj, layer.down_proj):
+                assert lin.weight.shape[1] % tp_size == 0
+                lin.tp_size = tp_size
+        self.tp_size = tp_size
 
     # ------------------------------------------------------------------------------------------
     def _rope(self, x: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:

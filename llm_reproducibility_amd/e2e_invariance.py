@@ -32,8 +32,9 @@ def main(argv=None) -> int:
     prompts = torch.randint(0, cfg.vocab_size, (args.prompts, args.prompt_len), generator=g).tolist()
     results, ref = [], None
     ok = True
+    model = Qwen3Decoder(cfg, tp_size=args.tp[0], seed=0, init_on_device=True)
     for tp in args.tp:
-        model = Qwen3Decoder(cfg, tp_size=tp, seed=0)
+        model.set_tp(tp)
         for bs in args.batches:
             bs = min(bs, args.prompts)
             torch.cuda.synchronize()
@@ -48,8 +49,6 @@ def main(argv=None) -> int:
             results.append({"tp": tp, "batch": bs, "identical_to_reference_run": same, "seconds": round(dt, 2),
                             "new_tokens_per_s": round(bs * args.new_tokens / dt, 1)})
             print(json.dumps(results[-1]), flush=True)
-        del model
-        torch.cuda.empty_cache()
     print(json.dumps({"config": vars(args), "all_identical": ok}))
     return 0 if ok else 1
 

@@ -79,7 +79,10 @@ def tbik_row_parallel_forward(self, input_):
     else:
         output = output_parallel
     if (not self.skip_bias_add) and self.bias is not None:
-        output += self.bias
+        # once per reduced output: on every rank after the tree all-reduce; on rank 0 only when the caller reduces
+        # the partial outputs itself (reduce_results=False), or that reduction would add the bias tp_size times
+        if self.reduce_results or self.tp_size == 1 or self.tp_rank == 0:
+            output += self.bias
     output = output.reshape(*lead, output.shape[-1])
     output_bias = self.bias if self.skip_bias_add else None
     if not self.return_bias:
@@ -131,6 +134,8 @@ class RMSNorm(nn.Module):
         return x if residual is None else (x, residual)
 
     def forward_fused(self, x, residual=None):
+        if x.dtype not in (torch.bfloat16, torch.float16) or x.shape[-1] > 8192 or x.shape[-1] % 8 != 0:
+            return self.forward_native(x, residual)   # shapes and dtypes the fused kernel does not take
         return rms_norm(x, self.weight, self.variance_epsilon, residual)
 
     forward = forward_native

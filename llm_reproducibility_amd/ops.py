@@ -139,8 +139,14 @@ def _tree_combine_impl(parts: List[torch.Tensor]) -> torch.Tensor:
     out = torch.empty_like(ps[0])
     arr = (ctypes.c_void_p * len(ps))(*[p.data_ptr() for p in ps])
     L = _lib.lib()
-    rc = (L.tbik_tree_combine_f16 if _is_f16(*ps) else L.tbik_tree_combine_bf16)(arr, len(ps), out.data_ptr(), out.numel(), _stream(out))
-    _lib.check(rc, "tbik_tree_combine_bf16")
+    if ps[0].dtype == torch.float32:
+        if any(p.dtype != torch.float32 for p in ps):
+            raise NotImplementedError("tree_combine takes partials of one dtype")
+        fn = L.tbik_tree_combine_f32
+    else:
+        fn = L.tbik_tree_combine_f16 if _is_f16(*ps) else L.tbik_tree_combine_bf16
+    rc = fn(arr, len(ps), out.data_ptr(), out.numel(), _stream(out))
+    _lib.check(rc, "tbik_tree_combine")
     return out
 
 

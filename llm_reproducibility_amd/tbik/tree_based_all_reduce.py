@@ -28,17 +28,7 @@ def tree_combine(parts: Sequence[torch.Tensor]) -> torch.Tensor:
         raise NotImplementedError("tree_combine takes partials of one dtype")
     if any(p.shape != parts[0].shape for p in parts):
         raise ValueError("partials must have the same shape")
-    if parts[0].dtype == torch.float32:
-        ops._require_gpu(*parts)
-        # an fp32 node is one elementwise fp32 addition: the tree order is all there is to fix
-        result = list(parts)
-        step = 1
-        while step < n:
-            for left in range(0, n, 2 * step):
-                result[left] = result[left] + result[left + step]
-            step *= 2
-        return result[0] if n > 1 else result[0].clone()
-    if parts[0].dtype not in (torch.bfloat16, torch.float16):
+    if parts[0].dtype not in (torch.bfloat16, torch.float16, torch.float32):
         raise NotImplementedError("tree_combine is implemented for bfloat16, float16 and float32 partials")
     return ops.tree_combine(list(parts))
 

@@ -19,6 +19,12 @@ reference and cites the lines it follows (paths relative to the reference checko
 * mean ....................... src/bio/batch_invariant_ops.py:331-349
 * RMSNorm .................... src/patch/patch_batch_invariant.py:9-16 -> vLLM RMSNorm.forward_native
                                (vllm==0.11.0 is not vendored in the reference; the public formula is restated)
+* causal attention ........... src/patch/patch_training_inference_align.py:171-487 (what the fixed-order kernel
+                               computes: softmax(q k^T * scale, causal) v per head, grouped-query heads)
+* rotary embedding ........... src/patch/patch_training_inference_align.py:35-44 (inverse frequencies in fp32 on
+                               the CPU) + the rotate-half form of the engine that the reference drives
+* greedy token choice ........ simple_inference.py:62-105 (sampling inside the engine; the tie rule -- lowest
+                               index -- is this build's, the reference leaves it to the library)
 
 Pin status (what checks each function independently of its own formula; see tests/test_oracle_*.py):
 
@@ -37,6 +43,17 @@ Pin status (what checks each function independently of its own formula; see test
   to closed forms (silu(0) = 0, silu(x) -> x for large x) and to a float64 evaluation.
 * `log_softmax`, `mean_lastdim`: pinned to float64 library routines and closed-form cases; the
   reference's in-block reduction order (Triton `tl.sum`) is backend defined, so tolerance only.
+* `matmul_single_acc`: pinned by exact rational arithmetic with an independent round-to-nearest-even on
+  integer operands (any accumulation narrower than fp32 fails it), by a case in which a bias added
+  before the rounding and one added after it give different bits, and by a case in which the
+  reference's detour through fp16 (src/bio/batch_invariant_ops.py:119-123) gives different bits -- the
+  single rounding is the documented choice.
+* `causal_attention`, `rotate_half_rope`, `qk_norm_rope`, `argmax_lowest_index`: pinned to the library
+  routine `torch.nn.functional.scaled_dot_product_attention` in float64, to closed forms (uniform
+  scores -> running mean of V, a dominant key -> its value, rotation by pi/2 and by 0, norm
+  preservation) and to brute force; the reference's own kernels for them (Triton unified attention,
+  vLLM rotary embedding and sampler) are backend defined or absent, so tolerance only: PARITY UNPINNED
+  at the bit level.
 """
 from __future__ import annotations
 
@@ -251,6 +268,111 @@ def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
     g, u = gate_up[..., :inter].float(), gate_up[..., inter:]
     s = (g / (1.0 + torch.exp(-g))).to(gate_up.dtype)
     return s * u
+
+
+# --------------------------------------------------------------------------------------------
+# attention, rotary embedding, greedy choice (the callers either side of the row-split GEMM)
+# --------------------------------------------------------------------------------------------
+def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float) -> torch.Tensor:
+    """Textbook causal grouped-query attention of ONE sequence in float64.
+
+    q [n, Hq, D] are the LAST n positions of the sequence whose keys / values are k, v [L, Hkv, D]
+    (n == L: prefill; n == 1: decode; 1 < n < L: chunked prefill).  Query head h reads KV head
+    h // (Hq // Hkv).  Returns float64 [n, Hq, D]: softmax over the keys at positions <= the query's,
+    then the weighted sum of the values.  This is what _kernel_unified_attention_2d computes per
+    (query, head) (src/patch/patch_training_inference_align.py:171-487), without its tiling.
+    """
+    n, Hq, D = q.shape
+    L, Hkv, _ = k.shape
+    assert Hq % Hkv == 0 and n <= L
+    rep = Hq // Hkv
+    qd, kd, vd = q.double(), k.double(), v.double()
+    out = torch.empty((n, Hq, D), dtype=torch.float64)
+    for h in range(Hq):
+        kh, vh = kd[:, h // rep], vd[:, h // rep]              # [L, D]
+        s = (qd[:, h] @ kh.t()) * scale                        # [n, L]
+        qpos = torch.arange(L - n, L)[:, None]
+        s = s.masked_fill(torch.arange(L)[None, :] > qpos, float("-inf"))
+        s = s - s.max(dim=-1, keepdim=True).values
+        p = torch.exp(s)
+        out[:, h] = (p / p.sum(dim=-1, keepdim=True)) @ vh
+    return out
+
+
+def rope_inv_freq(rotary_dim: int, base: float) -> torch.Tensor:
+    """fp32 inverse frequencies computed on the CPU, src/patch/patch_training_inference_align.py:36-41."""
+    arange = torch.arange(0, rotary_dim, 2, dtype=torch.float)
+    return 1.0 / (base ** (arange / rotary_dim))
+
+
+def rotate_half_rope(x: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor) -> torch.Tensor:
+    """Rotate-half rotary embedding: channel pair (i, i + D/2) of x [tokens, heads, D] is turned by the
+    angle positions[t] * inv_freq[i].  Angle and rotation in float64 from the fp32 table, one rounding
+    to the input dtype."""
+    half = x.shape[-1] // 2
+    ang = positions.double()[:, None] * inv_freq.double()[None, :]
+    cos, sin = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+    xd = x.double()
+    a, b = xd[..., :half], xd[..., half:]
+    return torch.cat((a * cos - b * sin, b * cos + a * sin), dim=-1).to(x.dtype)
+
+
+def qk_norm_rope(x: torch.Tensor, weight: torch.Tensor, eps: float, positions: torch.Tensor,
+                 inv_freq: torch.Tensor) -> torch.Tensor:
+    """Per-head RMSNorm (as `rmsnorm`: the normalised value rounded to the input dtype, then the weight)
+    followed by `rotate_half_rope` -- the Qwen3 q/k path in front of the attention (model wiring
+    simple_rl.py:320-338: qk_norm, head_dim 128)."""
+    return rotate_half_rope(rmsnorm(x, weight, eps), positions, inv_freq)
+
+
+def argmax_lowest_index(x: torch.Tensor) -> torch.Tensor:
+    """Index of the largest element of each row, ties to the LOWEST index, NaNs never selected
+    (a row of NaNs gives 0).  Brute force over the row in Python order for small inputs is
+    `max(range(n), key=lambda i: (x[i], -i))`; this is the vectorised form."""
+    xf = x.float()
+    xf = torch.where(torch.isnan(xf), torch.full_like(xf, float("-inf")), xf)
+    m = xf.max(dim=-1, keepdim=True).values
+    idx = torch.arange(x.shape[-1]).expand_as(xf)
+    big = torch.full_like(idx, x.shape[-1])
+    return torch.where(xf == m, idx, big).min(dim=-1).values
+
+
+def decoder_prefill_logits(weights: dict, prompt: Sequence[int], num_q_heads: int, num_kv_heads: int, head_dim: int,
+                           rms_eps: float, rope_theta: float, leaf: int = LEAF_BF16) -> torch.Tensor:
+    """Last-token logits of a Qwen3-architecture decoder on one prompt, composed from the per-op oracles above with
+    a rounding to bf16 wherever the kernels round (every op boundary): embedding -> [RMSNorm -> qkv (single
+    accumulator mm) -> per-head q/k RMSNorm + rotary -> causal attention -> o_proj (tree matmul) -> add + RMSNorm ->
+    gate_up (mm) -> SiLU * up -> down_proj (tree matmul)] x layers -> add + RMSNorm -> lm_head (mm).
+    Model wiring as the reference's harness uses it (simple_rl.py:320-338: qk_norm, head_dim, GQA); the row-split
+    layers are the patched RowParallelLinear forward (src/patch/patch_tp_invariant.py:11-46).
+
+    `weights`: CPU bf16 tensors: embed [V,H], lm_head [V,H], final_norm [H], layers = list of dicts with
+    input_norm, post_norm [H], q_norm, k_norm [D], qkv_w [(Hq+2Hkv)D, H], gate_up_w [2I, H], o_w [H, Hq*D],
+    down_w [H, I].
+    """
+    Hq, Hkv, D = num_q_heads, num_kv_heads, head_dim
+    tok = torch.tensor(list(prompt), dtype=torch.long)
+    pos = torch.arange(len(prompt))
+    inv = rope_inv_freq(D, rope_theta)
+    x = weights["embed"][tok]
+    residual = None
+    for lw in weights["layers"]:
+        if residual is None:
+            residual = x
+            h = rmsnorm(x, lw["input_norm"], rms_eps)
+        else:
+            h, residual = rmsnorm(x, lw["input_norm"], rms_eps, residual=residual)
+        qkv = matmul_single_acc(h, lw["qkv_w"].t())
+        q = qk_norm_rope(qkv[:, : Hq * D].reshape(-1, Hq, D), lw["q_norm"], rms_eps, pos, inv)
+        k = qk_norm_rope(qkv[:, Hq * D: (Hq + Hkv) * D].reshape(-1, Hkv, D), lw["k_norm"], rms_eps, pos, inv)
+        v = qkv[:, (Hq + Hkv) * D:].reshape(-1, Hkv, D)
+        att = causal_attention(q, k, v, 1.0 / math.sqrt(D)).to(torch.bfloat16).reshape(-1, Hq * D)
+        x = matmul_tree(att, lw["o_w"].t(), leaf=leaf)
+        h, residual = rmsnorm(x, lw["post_norm"], rms_eps, residual=residual)
+        act = silu_mul(matmul_single_acc(h, lw["gate_up_w"].t()))
+        x = matmul_tree(act, lw["down_w"].t(), leaf=leaf)
+    h, _ = rmsnorm(x, weights["final_norm"], rms_eps, residual=residual)
+    return matmul_single_acc(h[-1:], weights["lm_head"].t())[0]
 
 
 # --------------------------------------------------------------------------------------------

@@ -17,8 +17,14 @@ def test_rmsnorm_parity_and_batch_invariance(dev):
     xd, wd = x.to(dev), w.to(dev)
     full = bio.rms_norm(xd, wd, 1e-6)
     want = O.rmsnorm(x[:300], w, 1e-6)
+    # stated tolerance: within 1 bf16 ulp of the oracle OR within 2^-8 of the output scale.  The kernel's fp32 sum of
+    # squares runs in another order than the CPU's, so the normalised value may land on the other side of a rounding
+    # boundary (1 ulp); the bf16 multiply by the weight can carry that step into the binade below, where the same
+    # absolute step counts as 2 ulp -- never more, and only on a small fraction of the elements.
+    assert not O.outside_tolerance(full[:300], want).any()
     ulp = O.bf16_ulp_distance(full[:300].cpu(), want)
-    assert ulp.max() <= 2 and (ulp > 0).float().mean() < 0.02, (ulp.max(), (ulp > 0).float().mean())
+    assert ulp.max() <= 2 and (ulp > 0).float().mean() < 0.02 and (ulp > 1).float().mean() < 1e-3, \
+        (ulp.max(), (ulp > 0).float().mean(), (ulp > 1).float().mean())
     for r in ROWS:
         assert torch.equal(bio.rms_norm(xd[:r], wd, 1e-6), full[:r]), r
     assert torch.equal(bio.rms_norm(xd[1234:1235], wd, 1e-6), full[1234:1235])
@@ -58,12 +64,13 @@ def test_add_rmsnorm_parity(dev):
     out, new_res = bio.rms_norm(x.to(dev), w.to(dev), 1e-6, residual=res.to(dev))
     want, want_res = O.rmsnorm(x, w, 1e-6, residual=res)
     assert torch.equal(new_res.cpu(), want_res)
-    assert O.bf16_ulp_distance(out.cpu(), want).max() <= 2
+    assert not O.outside_tolerance(out, want).any() and O.bf16_ulp_distance(out.cpu(), want).max() <= 2
     for hidden in (8, 64, 520, 1024, 5120, 8192):
         xs = O.gaussian_bf16((5, hidden), 2.0, hidden)
         ws = O.gaussian_bf16((hidden,), 1.0, hidden + 1)
         got = bio.rms_norm(xs.to(dev), ws.to(dev), 1e-5)
-        assert O.bf16_ulp_distance(got.cpu(), O.rmsnorm(xs, ws, 1e-5)).max() <= 2, hidden
+        ws_want = O.rmsnorm(xs, ws, 1e-5)
+        assert not O.outside_tolerance(got, ws_want).any() and O.bf16_ulp_distance(got.cpu(), ws_want).max() <= 2, hidden
 
 
 def test_log_softmax_parity_and_batch_invariance(dev):
@@ -303,7 +310,7 @@ def test_argmax_lowest_index_on_ties(dev):
     g = torch.Generator().manual_seed(7)
     for rows, cols in ((1, 151936), (7, 151936), (128, 151936), (3, 5), (4, 1000), (2, 8), (5, 1031)):
         x = torch.randn((rows, cols), generator=g).to(torch.bfloat16)   # bf16 values collide often: many ties
-        want = torch.where(x == x.max(dim=-1, keepdim=True).values, torch.arange(cols), cols).min(dim=-1).values
+        want = O.argmax_lowest_index(x)
         got = ops.bi_argmax(x.to(dev))
         assert got.dtype == torch.int64 and torch.equal(got.cpu(), want), (rows, cols)
         r = rows - 1

@@ -157,3 +157,47 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libtbik_hip.so"))
     with pytest.raises(RuntimeError, match="only implementation"):
         _lib.lib()
+
+
+def test_tree_all_reduce_wrapper_contract(monkeypatch):
+    """tree_all_reduce_sum[_native] without a process group: the world size comes from a stand-in, the gather from a
+    stand-in that hands every rank's partial over, the adds from the CPU oracle.  Checks the ValueError of the reference
+    (src/tbik/tree_based_all_reduce.py:26-27), that the input is not aliased, and that the wrapper's result is the
+    adjacent-pair tree over the gathered partials in rank order."""
+    import torch
+    import torch.distributed as dist
+    from oracle import tbik_oracle as O
+    from llm_reproducibility_amd.tbik import tree_based_all_reduce as tar
+
+    world = {"n": 3}
+    monkeypatch.setattr(dist, "get_world_size", lambda group=None: world["n"])
+    x = O.integer_bf16((4, 16), -300, 300, 0)
+    for n in (3, 5, 6, 12):
+        world["n"] = n
+        with pytest.raises(ValueError):
+            tar.tree_all_reduce_sum(x)
+        with pytest.raises(ValueError):
+            tar.tree_all_reduce_sum_native(x)
+    partials = [O.integer_bf16((4, 16), -300, 300, 10 + r) for r in range(8)]
+    calls = []
+
+    def fake_all_gather(out_list, inp, group=None):
+        calls.append((len(out_list), inp.is_contiguous(), group))
+        for r, o in enumerate(out_list):
+            o.copy_(partials[r])
+
+    monkeypatch.setattr(dist, "all_gather", fake_all_gather)
+    monkeypatch.setattr(tar, "tree_combine", lambda parts: O.tree_combine(list(parts)))
+    for n in (1, 2, 4, 8):
+        world["n"] = n
+        calls.clear()
+        before = partials[0].clone()
+        got = tar.tree_all_reduce_sum(partials[0].t().contiguous().t(), device_group="grp")   # a non-contiguous view
+        assert calls == [(n, True, "grp")]
+        assert torch.equal(got, O.tree_combine(partials[:n]))
+        assert got.data_ptr() != partials[0].data_ptr() and torch.equal(partials[0], before)
+    # the tree, not a left-to-right sum: the two differ on these partials
+    seq = partials[0].clone()
+    for q in partials[1:8]:
+        seq = seq + q
+    assert not torch.equal(seq, O.tree_combine(partials))

@@ -1,5 +1,6 @@
 """Pins the CPU oracles of the batch-invariant reductions against library routines and closed forms (no GPU)."""
 import math
+from fractions import Fraction
 
 import pytest
 import torch
@@ -68,11 +69,80 @@ def test_rmsnorm_residual_semantics():
     assert torch.equal(y, want)
 
 
-def test_single_accumulator_matmul_is_one_rounding_of_the_fp32_product():
-    a = O.gaussian_bf16((8, 320), 1.0, 6)
-    b = O.gaussian_bf16((320, 24), 0.1, 7)
-    bias = O.gaussian_bf16((24,), 1.0, 8)
-    assert torch.equal(O.matmul_single_acc(a, b, bias), (a.float() @ b.float() + bias.float()).to(torch.bfloat16))
+def _rne_bf16(x: Fraction) -> float:
+    """Round an exact rational to the nearest bf16 (8 significant bits), ties to even -- integer arithmetic only."""
+    if x == 0:
+        return 0.0
+    sign = -1 if x < 0 else 1
+    x = abs(x)
+    e = 0
+    while x >= 256:          # scale into [128, 256): 8 significant bits are then the integer part
+        x /= 2
+        e += 1
+    while x < 128:
+        x *= 2
+        e -= 1
+    n = x.numerator // x.denominator
+    rem = x - n
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and n % 2 == 1):
+        n += 1
+    return float(sign * Fraction(n) * Fraction(2) ** e)
+
+
+def test_single_accumulator_matmul_against_exact_rational_arithmetic():
+    # integer operands: every product and every partial sum is an integer below 2^24, so an fp32 accumulator is exact
+    # in ANY order and the result is one rounding of the exact sum (+ bias); sums reach the thousands, so an
+    # accumulator with fewer bits (bf16: 8, fp16: 11) cannot reproduce them
+    a = O.integer_bf16((6, 320), -9, 9, 11)
+    b = O.integer_bf16((320, 5), -7, 7, 12)
+    bias = O.integer_bf16((5,), -300, 300, 13)          # multiples of 2 above 256 are bf16 values; make them so
+    bias = (bias.float() / 4).round().mul(4).to(torch.bfloat16)
+    got = O.matmul_single_acc(a, b, bias)
+    ai, bi, ci = a.double().long().tolist(), b.double().long().tolist(), bias.double().long().tolist()
+    big = 0
+    for m in range(6):
+        for n in range(5):
+            exact = sum(ai[m][k] * bi[k][n] for k in range(320)) + ci[n]
+            big = max(big, abs(exact))
+            assert got[m, n].item() == _rne_bf16(Fraction(exact)), (m, n, exact)
+    assert big > 512                                     # the rounding is exercised, not only exact values
+    nb = O.matmul_single_acc(a, b)
+    for m in range(6):
+        for n in range(5):
+            assert nb[m, n].item() == _rne_bf16(Fraction(sum(ai[m][k] * bi[k][n] for k in range(320))))
+
+
+def test_single_accumulator_matmul_adds_the_bias_before_the_one_rounding():
+    # sum = 257 (needs rounding: bf16 has 256 and 258), bias = 1.  Bias BEFORE the rounding (the reference adds it to
+    # the fp32 accumulator, src/bio/batch_invariant_ops.py:115-118): 258, exact.  Bias AFTER: bf16(257) = 256 (tie to
+    # even), 256 + 1 = 257 -> 256.  The two differ, the oracle must give the first.
+    a = torch.zeros((1, 264), dtype=torch.bfloat16)
+    a[0, :257] = 1
+    b = torch.ones((264, 1), dtype=torch.bfloat16)
+    bias = torch.ones((1,), dtype=torch.bfloat16)
+    assert O.matmul_single_acc(a, b, bias).item() == 258.0
+    after = (O.matmul_single_acc(a, b) + bias).item()
+    assert after == 256.0                                # what a bias applied to the rounded output would give
+
+
+def test_single_accumulator_matmul_rounds_once_not_through_fp16():
+    # 1 + 2^-8 + 2^-12: straight to bf16 it lies above the midpoint of 1 and 1 + 2^-7 -> rounds up.  Through fp16 first
+    # (the reference's detour, src/bio/batch_invariant_ops.py:119-123) the 2^-12 is lost, the value becomes the
+    # midpoint itself and the tie goes to 1.0; and anything above 65504 becomes inf.  The documented choice here is the
+    # single rounding.
+    a = torch.tensor([[1.0, 2.0 ** -8, 2.0 ** -12, 0, 0, 0, 0, 0]], dtype=torch.bfloat16)
+    b = torch.ones((8, 1), dtype=torch.bfloat16)
+    got = O.matmul_single_acc(a, b).item()
+    assert got == 1.0 + 2.0 ** -7
+    detour = (a.float() @ b.float()).half().to(torch.bfloat16).item()
+    assert detour == 1.0 and detour != got
+    big = torch.full((1, 8), 128.0, dtype=torch.bfloat16)
+    bb = torch.full((8, 1), 128.0, dtype=torch.bfloat16)
+    assert O.matmul_single_acc(big, bb).item() == 131072.0 and math.isinf((big.float() @ bb.float()).half().item())
+    # fp16 operands: the same single rounding to fp16
+    ah, bh = O.gaussian_bf16((5, 64), 1.0, 20).half(), O.gaussian_bf16((64, 3), 1.0, 21).half()
+    want = (ah.double() @ bh.double())
+    assert ((O.matmul_single_acc(ah, bh).double() - want).abs() <= want.abs() * 2.0 ** -11 + 1e-6).all()
 
 
 def test_silu_mul_matches_library_float64_and_closed_forms():
