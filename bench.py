@@ -22,16 +22,36 @@ if ROOT not in sys.path:
 M_, K_, N_ = 2048, 12288, 4096
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
-# HBM bytes one headline launch moves, from the hardware counters (not measured live: counters need the profiler).
-# FETCH_SIZE 256,867 KiB x 1.999 (a plain copy of 49,152 KiB reads 24,592) + WRITE_SIZE 131,072 KiB x 1.000;
-# profiles/gemm_tree_wide_headline_counters.txt holds the runs.  Algorithmic bytes are 167.8 MB: the rest is the
-# seven parked tree levels (written and read back once each) and one operand fetch per XCD-local L2.
-TRAFFIC_BYTES_PER_LAUNCH = 662.3e6
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "gemm_tree_wide_headline_counters.txt")
 
 
-def hip_time_ms(fn, steps, warmup):
-    """Average milliseconds per call, from HIP events on the stream the kernels are launched on."""
+def traffic_from_profile():
+    """HBM bytes one headline launch moves, read from the tracked rocprofv3 counter summary (FETCH_SIZE and WRITE_SIZE
+    passes, each scaled by what the same counter reads for a plain copy of known size).  Counters need the profiler,
+    so this is a figure of that profile, not of this run; None when the summary is missing."""
+    import re
+    try:
+        with open(TRAFFIC_PROFILE) as f:
+            m = re.search(r"traffic\s*=\s*([0-9.]+)\s*MB per launch", f.read())
+        return float(m.group(1)) * 1e6 if m else None
+    except OSError:
+        return None
+
+
+def hip_time_ms(fn, steps, warmup, settle_ms=0.0):
+    """Average milliseconds per call, from HIP events on the stream the kernels are launched on.
+
+    settle_ms > 0: the same call is first repeated for about that long.  After an idle period the chip's power
+    management takes some 25 ms of continuous load to settle: the first ten headline launches run at 225 us, the next
+    ten at 270-280 us, and only after about a hundred the rate is steady (210-215 us).  A benchmark of a handful of
+    steps taken right after the host-side set-up would measure that transient, not the kernel."""
     import torch
+    if settle_ms > 0:
+        t_end = time.perf_counter() + settle_ms * 1e-3
+        while time.perf_counter() < t_end:
+            for _ in range(8):
+                fn()
+            torch.cuda.synchronize()
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -65,7 +85,45 @@ def cpu_baseline(budget_s=12.0, max_runs=30):
     return {"value": round(2.0 * M_ * N_ * K_ / t / 1e12, 4), "unit": "TFLOP/s", "cores": torch.get_num_threads(),
             "kind": "port",
             "sample": f"oracle matmul_tree on the full X[{M_},{K_}] and W[{N_},{K_}] of the headline workload, "
-                      f"{len(ts)} runs in {spent:.1f} s, median {t:.2f} s each"}
+                      f"{len(ts)} runs in {spent:.1f} s, median {t:.2f} s each"}, O.matmul_tree(X, Wt)
+
+
+def ceiling(settle_ms):
+    """What the chip sustains on bf16 MFMAs alone (register operands, one work-group per CU, 2 waves per SIMD: the wave
+    shape of the tree kernel) for constant and for random operands, and on a one-pass read of 1 GiB (cold in the 256 MB
+    memory-side cache).  Steady-state figures (same load phase as the headline)."""
+    import ctypes
+    import torch
+    from llm_reproducibility_amd import _lib
+    L = _lib.lib()
+    dev = torch.device("cuda:0")
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    stream = torch.cuda.current_stream().cuda_stream
+    out = torch.empty(cus * 512, device=dev, dtype=torch.float32)
+    res = {"work_groups": cus}
+    iters = 800        # 800 x 16 MFMAs x 2 waves per SIMD = the MFMA count of one headline launch per SIMD on 256 CUs
+    g = torch.Generator().manual_seed(0)
+    ops_rand = torch.randn(32768, generator=g)
+    ops_rand[:16384] *= 0.02                      # a operands like the weights, b operands like the activations
+    for name, src in (("constant", torch.full((32768,), 1.0)), ("random", ops_rand)):
+        buf = src.to(torch.bfloat16).to(dev)
+
+        def run():
+            _lib.check(L.tbik_probe_mfma_bf16(buf.data_ptr(), out.data_ptr(), cus, 8, iters, stream), "tbik_probe_mfma_bf16")
+        ms, _ = hip_time_ms(run, 30, 5, settle_ms)
+        flop = float(cus) * 8 * iters * 16 * 16384
+        res[f"mfma_only_{name}_operands_TFLOPs"] = round(flop / (ms * 1e-3) / 1e12, 1)
+    nbytes = 1 << 30
+    big = torch.empty(nbytes // 4, device=dev, dtype=torch.int32).random_()
+    sink = torch.empty(cus * 16 * 256, device=dev, dtype=torch.int32)
+
+    def read():
+        _lib.check(L.tbik_probe_read(big.data_ptr(), nbytes, sink.data_ptr(), cus * 16, stream), "tbik_probe_read")
+    ms, _ = hip_time_ms(read, 20, 3, settle_ms)
+    res["one_pass_read_1GiB_GBps"] = round(nbytes / (ms * 1e-3) / 1e9, 1)
+    res["note"] = ("MFMA-only loop on register operands and a plain grid-stride read: ceilings of any bf16 matmul kernel "
+                   "on such data and of any one-pass kernel, measured in this run")
+    return res
 
 
 def table(steps, warmup, hot=False):
@@ -188,6 +246,11 @@ def main():
     ap.add_argument("--table", action="store_true", help="also print the per-shape table to stderr")
     ap.add_argument("--table-hot", action="store_true", help="with --table: reuse one input set per case (cache-hot figures)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--settle-ms", type=float, default=60.0,
+                    help="continuous load (the step itself) in front of the warm-up steps, so that the timed steps see "
+                         "the chip's settled state and not the transient that follows the host-side set-up; 0 disables")
+    ap.add_argument("--ceiling", action="store_true",
+                    help="also measure the MFMA-only and the one-pass-read ceilings of this chip (reported in `context`)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run 5 plain device copies of X (50,331,648 B read + as many written each) so that a "
                          "counter run can scale FETCH_SIZE / WRITE_SIZE by what a copy of known size reads")
@@ -202,16 +265,27 @@ def main():
 
     _lib.lib()
     dev = torch.device("cuda:0")
+    # host-side work first (the GPU idles meanwhile): the CPU baseline, whose product is also the parity reference
+    cpu, want = (None, None) if args.no_cpu_baseline else cpu_baseline()
     X = O.silu_gated_bf16((M_, K_), 0).to(dev)
     W = O.gaussian_bf16((N_, K_), 0.02, 1).to(dev)      # [N,K], K contiguous
     Wt = W.t()
     step = lambda: matmul_tp_persistent(X, Wt)          # noqa: E731
     C = step()
-    # sanity inside the bench: TP invariance of what is being timed (not timed itself)
+    # parity inside the bench (not timed): what is being timed equals the simulated TP=4 run bit for bit and agrees
+    # with the CPU oracle on the same inputs within the stated tolerance (1 bf16 ulp, or 2^-8 of the output scale)
     from llm_reproducibility_amd.tbik import tree_combine
     parts = [matmul_tp_persistent(X[:, r * 3072:(r + 1) * 3072], W[:, r * 3072:(r + 1) * 3072].t()) for r in range(4)]
     assert torch.equal(tree_combine(parts), C), "TP=4 result differs from TP=1"
     del parts
+    parity = None
+    if want is not None:
+        bad = O.outside_tolerance(C, want)
+        ulp = O.bf16_ulp_distance(C.cpu(), want)
+        assert not bad.any(), f"{int(bad.sum())} elements outside the tolerance against the CPU oracle"
+        parity = {"vs_cpu_oracle_full_size": "within 1 bf16 ulp or 2^-8 of the output scale",
+                  "bit_equal_fraction": round(float((ulp == 0).float().mean()), 4), "max_ulp": int(ulp.max()),
+                  "tp4_bitwise_equal": True}
 
     if args.calibrate_copy:
         Y = torch.empty_like(X)
@@ -220,7 +294,9 @@ def main():
         torch.cuda.synchronize()
         del Y
 
-    ms, wall_ms = hip_time_ms(step, args.steps, args.warmup)
+    # the figure right after the idle period (the transient), for the record; then the settled rate, which is `value`
+    cold_ms, _ = hip_time_ms(step, args.steps, args.warmup)
+    ms, wall_ms = hip_time_ms(step, args.steps, args.warmup, args.settle_ms)
     flops = 2.0 * M_ * N_ * K_
     algo_bytes = 2.0 * (M_ * K_ + K_ * N_ + M_ * N_)
     tflops = flops / (ms * 1e-3) / 1e12
@@ -234,16 +310,27 @@ def main():
         "pct_bf16_mfma_peak": round(100 * tflops / PEAK_BF16_TFLOPS, 2),
         "algorithmic_GBps": round(algo_bytes / (ms * 1e-3) / 1e9, 1),
         "roofline": {"bound": "mfma", "achieved": round(tflops, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(tflops / PEAK_BF16_TFLOPS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH,
+                     "frac": round(tflops / PEAK_BF16_TFLOPS, 4), "traffic": traffic_from_profile(),
+                     "traffic_source": "profiles/gemm_tree_wide_headline_counters.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
+                                       "scaled by a copy of known size; a figure of that profile, not of this run)",
                      "kernel_avg_us": round(ms * 1e3, 2)},
     }
-    if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline()
-        # context, measured in the same run after the timed region: the vendor library's plain GEMM on the same operands
-        # (reduction order not fixed, no tree; not a code path of this library)
-        lib_ms, _ = hip_time_ms(lambda: torch.matmul(X, W.t()), args.steps, args.warmup)
-        out["context"] = {"vendor_gemm_same_operands_TFLOPs": round(flops / (lib_ms * 1e-3) / 1e12, 2),
-                          "note": "torch.matmul (vendor library), reduction order not fixed, no tree"}
+    if cpu is not None:
+        out["cpu_baseline"] = cpu
+    context = {"settle_ms": args.settle_ms,
+               "settle_note": "the timed steps follow settle_ms of the same step run back to back (then the warm-up steps): "
+                              "after idling the chip needs about 25 ms of load to reach its steady rate",
+               "first_steps_after_idle_TFLOPs": round(flops / (cold_ms * 1e-3) / 1e12, 2)}
+    if parity is not None:
+        context["parity"] = parity
+    # the vendor library's plain GEMM on the same operands, measured the same way (reduction order not fixed, no tree;
+    # not a code path of this library)
+    lib_ms, _ = hip_time_ms(lambda: torch.matmul(X, Wt), args.steps, args.warmup, args.settle_ms)
+    context["vendor_gemm_same_operands_TFLOPs"] = round(flops / (lib_ms * 1e-3) / 1e12, 2)
+    context["note"] = "torch.matmul (vendor library), reduction order not fixed, no tree"
+    if args.ceiling:
+        context["ceiling"] = ceiling(args.settle_ms)
+    out["context"] = context
     if args.table:
         table(max(args.steps // 2, 5), max(args.warmup // 2, 2), hot=args.table_hot)
     print(json.dumps(out))
