@@ -283,8 +283,11 @@ def main():
         bad = O.outside_tolerance(C, want)
         ulp = O.bf16_ulp_distance(C.cpu(), want)
         assert not bad.any(), f"{int(bad.sum())} elements outside the tolerance against the CPU oracle"
-        parity = {"vs_cpu_oracle_full_size": "within 1 bf16 ulp or 2^-8 of the output scale",
-                  "bit_equal_fraction": round(float((ulp == 0).float().mean()), 4), "max_ulp": int(ulp.max()),
+        scale = float(want.float().abs().max())
+        parity = {"vs_cpu_oracle_full_size": "every element within 1 bf16 ulp or 2^-8 of the output scale",
+                  "bit_equal_fraction": round(float((ulp == 0).float().mean()), 5),
+                  "within_1_ulp_fraction": round(float((ulp <= 1).float().mean()), 6),
+                  "max_abs_diff_over_scale": float((C.cpu().float() - want.float()).abs().max()) / scale,
                   "tp4_bitwise_equal": True}
 
     if args.calibrate_copy:
