@@ -27,6 +27,7 @@ extern "C" {
 #define TBIK_ERR_ALIGNMENT    2   /* pointer or leading dimension not aligned for 16-byte accesses  */
 #define TBIK_ERR_UNSUPPORTED  3   /* layout or tree depth this build has no kernel for              */
 #define TBIK_ERR_WORKSPACE    4   /* workspace missing or too small                                 */
+#define TBIK_ERR_SCRATCH_LIMIT 5  /* the problem needs more than TBIK_STATIC_SCRATCH_BYTES of scratch */
 #define TBIK_ERR_HIP_BASE     1000
 
 typedef void* tbik_stream_t;  /* hipStream_t */
@@ -76,6 +77,27 @@ int tbik_gemm_bf16(const void* A, int64_t lda,
  * Replaces: the in-register tensor `S` of the reference kernel, src/tbik/tree_based_matmul.py:85.
  */
 size_t tbik_gemm_workspace_bytes(int M, int N, int K, int leaf_k);
+
+/*
+ * tbik_gemm_bf16 for callers that cannot allocate device memory: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  Same arguments (without the workspace), same kernels, same bits; the workspace is
+ * a fixed array of TBIK_STATIC_SCRATCH_BYTES inside the library, one copy per GPU, held until the process ends.  A
+ * problem whose tbik_gemm_workspace_bytes() exceeds that size returns TBIK_ERR_SCRATCH_LIMIT before anything is
+ * launched (decode- and mid-sized batches fit; the 2048-row benchmark shape does not).  The call allocates and frees
+ * nothing.  The first call on a device resolves the array's device address (hipGetSymbolAddress): make that call
+ * outside a graph capture.  Every call on a GPU uses that GPU's one array, whose contents are scratch (written
+ * before they are read, nothing has to start at zero): two calls that overlap in time on one GPU -- different
+ * streams, or two graphs replayed concurrently -- race on it and must be ordered by the caller.
+ * No counterpart in the reference (its Triton kernel keeps the merge stack in registers and allocates only its
+ * output through torch, src/tbik/tree_based_matmul.py:251).
+ */
+#define TBIK_STATIC_SCRATCH_BYTES (32 * 1024 * 1024)
+int tbik_gemm_bf16_static(const void* A, int64_t lda,
+                          const void* B, int64_t ldb_k, int64_t ldb_n,
+                          void* C, int64_t ldc,
+                          int M, int N, int K, int leaf_k,
+                          const void* bias_or_null,
+                          tbik_stream_t stream);
 
 /*
  * out[i] = adjacent-pair binary tree over parts[0..nparts-1][i], bf16 adds (round to nearest even

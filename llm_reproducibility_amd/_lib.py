@@ -17,13 +17,15 @@ TBIK_ERR_INVALID = 1
 TBIK_ERR_ALIGNMENT = 2
 TBIK_ERR_UNSUPPORTED = 3
 TBIK_ERR_WORKSPACE = 4
+TBIK_ERR_SCRATCH_LIMIT = 5
+STATIC_SCRATCH_BYTES = 32 * 1024 * 1024
 
 EXPORTS = (
     "tbik_abi_version", "tbik_error_string", "tbik_tree_params", "tbik_gemm_bf16", "tbik_gemm_workspace_bytes",
     "tbik_tree_combine_bf16", "tbik_tree_combine_f32",
     "bi_gemm_bf16", "bi_rmsnorm_bf16", "bi_log_softmax_workspace_bytes", "bi_log_softmax_f32", "bi_mean_dim", "bi_attention_bf16", "bi_silu_mul_bf16",
     "tbik_gemm_f16", "tbik_gemm_f16_workspace_bytes", "tbik_tree_combine_f16", "bi_gemm_f16", "tbik_gemm_f32", "bi_gemm_f32", "bi_rmsnorm_f16", "bi_silu_mul_f16", "bi_qk_norm_rope_cache_bf16", "bi_argmax_bf16",
-    "tbik_probe_mfma_bf16", "tbik_probe_read",
+    "tbik_probe_mfma_bf16", "tbik_probe_read", "tbik_gemm_bf16_static",
 )
 
 _lib = None
@@ -93,6 +95,8 @@ def lib() -> ctypes.CDLL:
     L.bi_qk_norm_rope_cache_bf16.restype = i32
     L.bi_argmax_bf16.argtypes = [vp, i64, vp, i64, i32, vp]
     L.bi_argmax_bf16.restype = i32
+    L.tbik_gemm_bf16_static.argtypes = [vp, i64, vp, i64, i64, vp, i64, i32, i32, i32, i32, vp, vp]
+    L.tbik_gemm_bf16_static.restype = i32
     L.tbik_probe_mfma_bf16.argtypes = [vp, vp, i32, i32, i32, vp]
     L.tbik_probe_mfma_bf16.restype = i32
     L.tbik_probe_read.argtypes = [vp, i64, vp, i32, vp]

@@ -42,6 +42,7 @@ const char* tbik_error_string(int code) {
     case TBIK_ERR_ALIGNMENT: return "pointer or leading dimension not aligned for 16-byte accesses";
     case TBIK_ERR_UNSUPPORTED: return "layout, dtype or tree depth not supported by this build";
     case TBIK_ERR_WORKSPACE: return "workspace missing or too small";
+    case TBIK_ERR_SCRATCH_LIMIT: return "the problem needs more scratch than the library's fixed array (TBIK_STATIC_SCRATCH_BYTES): use the entry point that takes a workspace";
     default: return code >= TBIK_ERR_HIP_BASE ? hipGetErrorString((hipError_t)(code - TBIK_ERR_HIP_BASE)) : "unknown";
   }
 }
