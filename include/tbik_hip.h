@@ -143,18 +143,32 @@ int bi_rmsnorm_bf16(const void* x, int64_t ldx,
                     tbik_stream_t stream);
 
 /*
- * Bytes of workspace bi_log_softmax_f32 needs for a [rows, cols] input.
+ * Bytes of workspace bi_log_softmax / bi_log_softmax_f32 need for a [rows, cols] input.  (A call of at least 192 rows
+ * of at most 154,624 elements whose rows allow 16-byte accesses runs as one launch with the row resident on chip and
+ * does not touch the workspace; it may then be NULL.)
  */
 size_t bi_log_softmax_workspace_bytes(int64_t rows, int64_t cols);
 
 /*
- * out[r, :] = x[r, :] - max - log(sum(exp(x[r, :] - max))), fp32, last dimension.
- * Every row is cut into fixed 4096-element segments (a function of `cols` only); segment
- * (max, sum) pairs go to `workspace` and are merged in segment order, so row r's result does not
- * depend on `rows`.  `write_softmax` != 0 writes exp(log_softmax) instead.
+ * out[r, :] = x[r, :] - max - log(sum(exp(x[r, :] - max))), last dimension, fp32 arithmetic.
+ * dtype codes: 0 = fp32, 1 = bf16, 2 = fp16; the output is fp32 or has the input's type (the reference's kernel loads
+ * the input dtype directly and the aten override's half_to_float asks for an fp32 result).
+ * Every row is cut into fixed 4096-element segments (a function of `cols` only); segment (max, sum) pairs are merged
+ * in segment order, so row r's result does not depend on `rows`.  Small batches run as two launches over
+ * (row, segment) work-groups with the pairs in `workspace`; from 192 rows on, one work-group per row keeps the row on
+ * chip between its one read and its one write -- the same expression, the same bits.  `write_softmax` != 0 writes
+ * exp(log_softmax) instead.  ldx / ldo are row strides in elements.
  * Replaces: log_softmax + _log_softmax_kernel, src/bio/batch_invariant_ops.py:263-301 and
  *           :200-260 (aten::_log_softmax / aten::_softmax overrides, :450-456).
  */
+int bi_log_softmax(const void* x, int64_t ldx, int in_dtype_code,
+                   void* out, int64_t ldo, int out_dtype_code,
+                   int64_t rows, int64_t cols,
+                   void* workspace, size_t workspace_bytes,
+                   int write_softmax,
+                   tbik_stream_t stream);
+
+/* bi_log_softmax with fp32 input and output. */
 int bi_log_softmax_f32(const void* x, int64_t ldx,
                        void* out, int64_t ldo,
                        int64_t rows, int64_t cols,

@@ -25,7 +25,7 @@ EXPORTS = (
     "tbik_tree_combine_bf16", "tbik_tree_combine_f32",
     "bi_gemm_bf16", "bi_rmsnorm_bf16", "bi_log_softmax_workspace_bytes", "bi_log_softmax_f32", "bi_mean_dim", "bi_attention_bf16", "bi_silu_mul_bf16",
     "tbik_gemm_f16", "tbik_gemm_f16_workspace_bytes", "tbik_tree_combine_f16", "bi_gemm_f16", "tbik_gemm_f32", "bi_gemm_f32", "bi_rmsnorm_f16", "bi_silu_mul_f16", "bi_qk_norm_rope_cache_bf16", "bi_argmax_bf16",
-    "tbik_probe_mfma_bf16", "tbik_probe_read", "tbik_gemm_bf16_static",
+    "tbik_probe_mfma_bf16", "tbik_probe_read", "tbik_gemm_bf16_static", "bi_log_softmax",
 )
 
 _lib = None
@@ -69,6 +69,8 @@ def lib() -> ctypes.CDLL:
     L.bi_log_softmax_workspace_bytes.restype = sz
     L.bi_log_softmax_f32.argtypes = [vp, i64, vp, i64, i64, i64, vp, sz, i32, vp]
     L.bi_log_softmax_f32.restype = i32
+    L.bi_log_softmax.argtypes = [vp, i64, i32, vp, i64, i32, i64, i64, vp, sz, i32, vp]
+    L.bi_log_softmax.restype = i32
     L.bi_mean_dim.argtypes = [vp, vp, i64, i64, i64, i32, vp]
     L.bi_mean_dim.restype = i32
     L.tbik_gemm_f16.argtypes = L.tbik_gemm_bf16.argtypes

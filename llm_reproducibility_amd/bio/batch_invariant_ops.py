@@ -42,13 +42,13 @@ def log_softmax(input: torch.Tensor, dim: int = -1) -> torch.Tensor:
     """log_softmax over the last dimension (reference :263-301); output dtype = input dtype."""
     if dim != -1 and dim != input.ndim - 1:
         raise ValueError("This implementation only supports log_softmax along the last dimension")
-    return ops.bi_log_softmax_f32(input.float(), False).to(input.dtype)
+    return _run_softmax(input, False, False)
 
 
 def softmax(input: torch.Tensor, dim: int = -1) -> torch.Tensor:
     if dim != -1 and dim != input.ndim - 1:
         raise ValueError("This implementation only supports softmax along the last dimension")
-    return ops.bi_log_softmax_f32(input.float(), True).to(input.dtype)
+    return _run_softmax(input, True, False)
 
 
 def mean_dim(input: torch.Tensor, dim: int, keepdim: bool = False, dtype: Optional[torch.dtype] = None) -> torch.Tensor:
@@ -85,20 +85,25 @@ def addmm_batch_invariant(bias, a, b):
     return matmul_persistent(a, b, bias=bias)
 
 
+def _run_softmax(input, write_softmax: bool, to_float: bool):
+    """fp32, bf16 and fp16 go to the kernel as they are (it reads the input dtype itself); anything else is computed
+    in fp32 and cast back."""
+    if input.dtype in (torch.float32, torch.bfloat16, torch.float16):
+        return ops.bi_log_softmax(input, write_softmax, to_float)
+    out = ops.bi_log_softmax(input.float(), write_softmax, False)
+    return out if to_float else out.to(input.dtype)
+
+
 def _log_softmax_batch_invariant(input, dim, _half_to_float):
-    out = ops.bi_log_softmax_f32(_last_dim_f32(input, dim), False)
-    return out if _half_to_float else out.to(input.dtype)
+    if dim != -1 and dim != input.ndim - 1:
+        raise ValueError("This implementation only supports softmax along the last dimension")
+    return _run_softmax(input, False, bool(_half_to_float))
 
 
 def _softmax_batch_invariant(input, dim, _half_to_float):
-    out = ops.bi_log_softmax_f32(_last_dim_f32(input, dim), True)
-    return out if _half_to_float else out.to(input.dtype)
-
-
-def _last_dim_f32(input, dim):
     if dim != -1 and dim != input.ndim - 1:
         raise ValueError("This implementation only supports softmax along the last dimension")
-    return input.float()
+    return _run_softmax(input, True, bool(_half_to_float))
 
 
 def mean_batch_invariant(input, dim, keepdim=False, dtype: Optional[torch.dtype] = None):

@@ -12,8 +12,8 @@ int tree_combine_f32_dispatch(const void* const* parts, int nparts, void* out, i
 int rmsnorm_dispatch(const void* x, int64_t ldx, const void* res, int64_t ldr, const void* w, void* out, int64_t ldo,
                      void* res_out, int64_t ldro, int64_t rows, int hidden, float eps, bool f16, hipStream_t stream);
 size_t lsm_workspace_bytes(int64_t rows, int64_t cols);
-int log_softmax_dispatch(const void* x, int64_t ldx, void* out, int64_t ldo, int64_t rows, int64_t cols, void* ws,
-                         size_t ws_bytes, int write_softmax, hipStream_t stream);
+int log_softmax_dispatch(const void* x, int64_t ldx, int in_dtype, void* out, int64_t ldo, int out_dtype, int64_t rows,
+                         int64_t cols, void* ws, size_t ws_bytes, int write_softmax, hipStream_t stream);
 int attention_dispatch(const void* q, const void* k_cache, const void* vt_cache, void* out, const int* q_start,
                        const int* q_len, const int* ctx_len, int batch, int max_q_len, int q_heads, int kv_heads,
                        int head_dim, int max_len, float scale, hipStream_t stream);
@@ -119,8 +119,14 @@ size_t bi_log_softmax_workspace_bytes(int64_t rows, int64_t cols) { return tbik:
 
 int bi_log_softmax_f32(const void* x, int64_t ldx, void* out, int64_t ldo, int64_t rows, int64_t cols, void* workspace,
                        size_t workspace_bytes, int write_softmax, tbik_stream_t stream) {
-  return tbik::log_softmax_dispatch(x, ldx, out, ldo, rows, cols, workspace, workspace_bytes, write_softmax,
+  return tbik::log_softmax_dispatch(x, ldx, 0, out, ldo, 0, rows, cols, workspace, workspace_bytes, write_softmax,
                                     static_cast<hipStream_t>(stream));
+}
+
+int bi_log_softmax(const void* x, int64_t ldx, int in_dtype_code, void* out, int64_t ldo, int out_dtype_code, int64_t rows,
+                   int64_t cols, void* workspace, size_t workspace_bytes, int write_softmax, tbik_stream_t stream) {
+  return tbik::log_softmax_dispatch(x, ldx, in_dtype_code, out, ldo, out_dtype_code, rows, cols, workspace, workspace_bytes,
+                                    write_softmax, static_cast<hipStream_t>(stream));
 }
 
 int bi_mean_dim(const void* x, void* out, int64_t outer, int64_t n, int64_t inner, int dtype_code, tbik_stream_t stream) {

@@ -1,4 +1,4 @@
-// Batch-invariant row reductions for gfx950: RMSNorm (bf16 or fp16), log_softmax / softmax (fp32), mean.
+// Batch-invariant row reductions for gfx950: RMSNorm (bf16 or fp16), log_softmax / softmax (fp32, bf16, fp16), mean.
 //
 // Rule shared by all kernels here: the decomposition of a row into lanes, wavefronts and segments,
 // and the order in which partial sums meet, is a function of the ROW LENGTH only.  The number of rows
@@ -143,67 +143,163 @@ int rmsnorm_dispatch(const void* x, int64_t ldx, const void* res, int64_t ldr, c
 }
 
 // ================================================================================================
-// log_softmax / softmax over the last dimension, fp32.
-// A row is cut into fixed segments of 4096 elements; kernel 1 reduces each segment to (max, sum of
-// exp(x - max)); kernel 2 merges a row's segment pairs in segment order and writes the result.
-// Replaces the one-program-per-row three-pass kernel of the reference
-// (src/bio/batch_invariant_ops.py:200-260): rows no longer limit the parallelism, yet the per-row
-// order stays a function of `cols` alone.
+// log_softmax / softmax over the last dimension; fp32, bf16 or fp16 in, the same type or fp32 out, fp32 arithmetic.
+// Replaces the one-program-per-row three-pass kernel of the reference (src/bio/batch_invariant_ops.py:200-260, which
+// loads the input dtype directly, :263-301).
+//
+// Arithmetic (a function of `cols` alone): a row is cut into fixed segments of 4096 elements.  Inside a segment,
+// thread t of 256 owns the 4-element chunks t, t+256, t+512, t+768; a segment reduces to (max, sum of exp(x - max))
+// by: per-thread sequential, fixed butterfly over the wavefront, four wavefronts joined in order.  The segment pairs
+// of a row are merged by one wavefront (lane l takes segments l, l+64, ... ascending, then the butterfly).
+//
+// Two schedules evaluate exactly this expression, so they give the same bits and the choice may depend on the batch:
+//   * two launches (lsm_partial_kernel + lsm_write_kernel): one work-group per segment; fills the chip for a handful
+//     of rows, but reads the row twice (12 bytes moved per fp32 element for 8 algorithmic);
+//   * one launch (lsm_resident_kernel): one work-group of 512 threads per row keeps the whole row on chip between the
+//     read and the write -- 28 segments in registers (224 of the 256 registers of every thread), the rest in LDS --
+//     so every element is read once and written once.  Rows of up to 154,624 elements fit (a 151,936-entry
+//     vocabulary does).
+// exp is 2^(d * log2 e) on the hardware exponential in both.
 // ================================================================================================
 constexpr int kSeg = 4096;  // elements per segment: 256 threads x 4 chunks x 4 floats
+constexpr int kResidentRegSegs = 28;                          // segments a resident work-group holds in registers
+constexpr int kResidentLdsFloats = (160 * 1024 - 4096) / 4;   // row elements it can hold in LDS behind those
+constexpr int64_t kResidentMaxCols = (int64_t)kResidentRegSegs * kSeg + kResidentLdsFloats;
+
+enum { LSM_F32 = 0, LSM_BF16 = 1, LSM_F16 = 2 };
 
 struct LsmArgs {
-  const float* x;
-  float* out;
+  const void* x;
+  void* out;
   float* ws;  // [rows][segs][2]
   int64_t ldx, ldo;
   int64_t rows, cols;
   int segs;
-  int vec;  // rows allow 16-byte loads/stores
+  int vec;  // rows allow full-width vector loads/stores of a 4-element chunk
   int write_softmax;
 };
 
-// Loads this thread's 16 elements of the segment (chunk q = tid + 256*i holds elements 4q..4q+3 of the
-// segment); out-of-range elements read as `fill`.
-__device__ __forceinline__ void load_seg(const float* row, int64_t base, int64_t cols, int vec, float fill,
-                                         float (&v)[4][4]) {
+__device__ __forceinline__ float fast_exp(float d) { return __builtin_amdgcn_exp2f(d * 1.44269504088896340736f); }
+
+template <int T>
+struct LsmElem;
+template <>
+struct LsmElem<LSM_F32> {
+  typedef float type;
+  static __device__ __forceinline__ void load4(const float* p, float (&v)[4]) {
+    const float4 q = *reinterpret_cast<const float4*>(p);
+    v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+  }
+  static __device__ __forceinline__ float load1(const float* p) { return *p; }
+  static __device__ __forceinline__ void store4(float* p, const float (&v)[4]) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  }
+  static __device__ __forceinline__ void store1(float* p, float v) { *p = v; }
+};
+template <>
+struct LsmElem<LSM_BF16> {
+  typedef uint16_t type;
+  static __device__ __forceinline__ void load4(const uint16_t* p, float (&v)[4]) {
+    const uint2 q = *reinterpret_cast<const uint2*>(p);
+    v[0] = bf16_lo(q.x); v[1] = bf16_hi(q.x); v[2] = bf16_lo(q.y); v[3] = bf16_hi(q.y);
+  }
+  static __device__ __forceinline__ float load1(const uint16_t* p) { return bf16_bits_to_f32(*p); }
+  static __device__ __forceinline__ void store4(uint16_t* p, const float (&v)[4]) {
+    *reinterpret_cast<uint2*>(p) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+  }
+  static __device__ __forceinline__ void store1(uint16_t* p, float v) { *p = f32_to_bf16_bits(v); }
+};
+template <>
+struct LsmElem<LSM_F16> {
+  typedef uint16_t type;
+  static __device__ __forceinline__ void load4(const uint16_t* p, float (&v)[4]) {
+    const uint2 q = *reinterpret_cast<const uint2*>(p);
+    const f16x2 a = __builtin_bit_cast(f16x2, q.x), b = __builtin_bit_cast(f16x2, q.y);
+    v[0] = (float)a[0]; v[1] = (float)a[1]; v[2] = (float)b[0]; v[3] = (float)b[1];
+  }
+  static __device__ __forceinline__ float load1(const uint16_t* p) { return f16_bits_to_f32(*p); }
+  static __device__ __forceinline__ void store4(uint16_t* p, const float (&v)[4]) {
+    *reinterpret_cast<uint2*>(p) = make_uint2(pack_f16x2(v[0], v[1]), pack_f16x2(v[2], v[3]));
+  }
+  static __device__ __forceinline__ void store1(uint16_t* p, float v) { *p = (uint16_t)(pack_f16x2(v, 0.f) & 0xffffu); }
+};
+
+// The 4-element chunk that starts at element e of a row; out-of-range elements read as `fill`.
+template <int IN>
+__device__ __forceinline__ void load_chunk(const typename LsmElem<IN>::type* row, int64_t e, int64_t cols, int vec, float fill,
+                                           float (&v)[4]) {
+  if (vec && e + 3 < cols) {
+    LsmElem<IN>::load4(row + e, v);
+  } else {
 #pragma unroll
-  for (int i = 0; i < 4; i++) {
-    const int64_t e = base + 4 * (int64_t)(threadIdx.x + 256 * i);
-    if (vec && e + 3 < cols) {
-      const float4 q = *reinterpret_cast<const float4*>(row + e);
-      v[i][0] = q.x; v[i][1] = q.y; v[i][2] = q.z; v[i][3] = q.w;
-    } else {
+    for (int j = 0; j < 4; j++) v[j] = (e + j < cols) ? LsmElem<IN>::load1(row + e + j) : fill;
+  }
+}
+template <int OUT>
+__device__ __forceinline__ void store_chunk(typename LsmElem<OUT>::type* row, int64_t e, int64_t cols, int vec, const float (&v)[4]) {
+  if (vec && e + 3 < cols) {
+    LsmElem<OUT>::store4(row + e, v);
+  } else {
 #pragma unroll
-      for (int j = 0; j < 4; j++) v[i][j] = (e + j < cols) ? row[e + j] : fill;
-    }
+    for (int j = 0; j < 4; j++)
+      if (e + j < cols) LsmElem<OUT>::store1(row + e + j, v[j]);
   }
 }
 
-__global__ __launch_bounds__(256) void lsm_partial_kernel(const LsmArgs a) {
-  __shared__ float red[4];
-  const int64_t row = blockIdx.x / a.segs;
-  const int seg = blockIdx.x % a.segs;
-  const float* xr = a.x + row * a.ldx;
-  float v[4][4];
-  load_seg(xr, (int64_t)seg * kSeg, a.cols, a.vec, -INFINITY, v);
+// Thread t (0..255) of a segment's team: its 16 elements (chunk q = t + 256*i holds elements 4q..4q+3 of the segment).
+template <int IN>
+__device__ __forceinline__ void load_seg(const typename LsmElem<IN>::type* row, int64_t base, int t, int64_t cols, int vec,
+                                         float fill, float (&v)[4][4]) {
+#pragma unroll
+  for (int i = 0; i < 4; i++) load_chunk<IN>(row, base + 4 * (int64_t)(t + 256 * i), cols, vec, fill, v[i]);
+}
+
+__device__ __forceinline__ float seg_thread_max(const float (&v)[4][4]) {
   float m = -INFINITY;
 #pragma unroll
   for (int i = 0; i < 4; i++)
 #pragma unroll
     for (int j = 0; j < 4; j++) m = fmaxf(m, v[i][j]);
-  m = wave_max(m);
+  return m;
+}
+__device__ __forceinline__ float seg_thread_expsum(const float (&v)[4][4], float m) {
+  // exp(x - m) = 2^(x * log2 e - m * log2 e): one fused multiply-add and the hardware exponential per element
+  constexpr float kLog2e = 1.44269504088896340736f;
+  const float ml = m * kLog2e;
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++) s += __builtin_amdgcn_exp2f(__builtin_fmaf(v[i][j], kLog2e, -ml));  // 2^(-inf) = 0 for the padding
+  return s;
+}
+
+// The merge of a row's segment pairs by ONE wavefront: lane l takes segments l, l+64, ... in ascending order, then the
+// fixed butterfly.  Returns (global max, log of the global sum) in every lane.
+__device__ __forceinline__ void merge_segments(const float* w, int segs, int lane, float& gmax, float& lg) {
+  float lm = -INFINITY;
+  for (int s = lane; s < segs; s += 64) lm = fmaxf(lm, w[2 * s]);
+  gmax = wave_max(lm);
+  float ls = 0.f;
+  for (int s = lane; s < segs; s += 64) ls += w[2 * s + 1] * expf(w[2 * s] - gmax);
+  lg = logf(wave_sum(ls));
+}
+
+template <int IN>
+__global__ __launch_bounds__(256) void lsm_partial_kernel(const LsmArgs a) {
+  __shared__ float red[4];
+  const int64_t row = blockIdx.x / a.segs;
+  const int seg = blockIdx.x % a.segs;
+  const typename LsmElem<IN>::type* xr = static_cast<const typename LsmElem<IN>::type*>(a.x) + row * a.ldx;
+  float v[4][4];
+  load_seg<IN>(xr, (int64_t)seg * kSeg, threadIdx.x, a.cols, a.vec, -INFINITY, v);
+  float m = wave_max(seg_thread_max(v));
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   if (lane == 0) red[wave] = m;
   __syncthreads();
   m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
   __syncthreads();
-  float s = 0.f;
-#pragma unroll
-  for (int i = 0; i < 4; i++)
-#pragma unroll
-    for (int j = 0; j < 4; j++) s += expf(v[i][j] - m);  // exp(-inf) = 0 for the padding
-  s = wave_sum(s);
+  const float s = wave_sum(seg_thread_expsum(v, m));
   if (lane == 0) red[wave] = s;
   __syncthreads();
   if (threadIdx.x == 0) {
@@ -214,49 +310,183 @@ __global__ __launch_bounds__(256) void lsm_partial_kernel(const LsmArgs a) {
   }
 }
 
+template <int IN, int OUT>
 __global__ __launch_bounds__(256) void lsm_write_kernel(const LsmArgs a) {
   const int64_t row = blockIdx.x / a.segs;
   const int seg = blockIdx.x % a.segs;
-  // The row's segment pairs are merged by the first wavefront only (lane l takes segments l, l+64, ... in
-  // ascending order, then a fixed butterfly): the order is a function of `segs` alone, and the other 192
-  // threads do not repeat the work.
+  // merged by the first wavefront only: the other 192 threads do not repeat the work
   __shared__ float stat[2];
   if (threadIdx.x < 64) {
-    const float* w = a.ws + (int64_t)row * a.segs * 2;
-    float lm = -INFINITY;
-    for (int s = threadIdx.x; s < a.segs; s += 64) lm = fmaxf(lm, w[2 * s]);
-    const float gmax = wave_max(lm);
-    float ls = 0.f;
-    for (int s = threadIdx.x; s < a.segs; s += 64) ls += w[2 * s + 1] * expf(w[2 * s] - gmax);
-    const float gsum = wave_sum(ls);
+    float gmax, lg;
+    merge_segments(a.ws + (int64_t)row * a.segs * 2, a.segs, threadIdx.x, gmax, lg);
     if (threadIdx.x == 0) {
       stat[0] = gmax;
-      stat[1] = logf(gsum);
+      stat[1] = lg;
     }
   }
   __syncthreads();
   const float gm = stat[0], lg = stat[1];
-  const float* xr = a.x + row * a.ldx;
-  float* orow = a.out + row * a.ldo;
+  const typename LsmElem<IN>::type* xr = static_cast<const typename LsmElem<IN>::type*>(a.x) + row * a.ldx;
+  typename LsmElem<OUT>::type* orow = static_cast<typename LsmElem<OUT>::type*>(a.out) + row * a.ldo;
   float v[4][4];
-  load_seg(xr, (int64_t)seg * kSeg, a.cols, a.vec, 0.f, v);
+  load_seg<IN>(xr, (int64_t)seg * kSeg, threadIdx.x, a.cols, a.vec, 0.f, v);
 #pragma unroll
   for (int i = 0; i < 4; i++) {
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-      float y = (v[i][j] - gm) - lg;
-      v[i][j] = a.write_softmax ? expf(y) : y;
+      const float y = (v[i][j] - gm) - lg;
+      v[i][j] = a.write_softmax ? fast_exp(y) : y;
     }
-    const int64_t e = (int64_t)seg * kSeg + 4 * (int64_t)(threadIdx.x + 256 * i);
-    if (a.vec && e + 3 < a.cols) {
-      *reinterpret_cast<float4*>(orow + e) = make_float4(v[i][0], v[i][1], v[i][2], v[i][3]);
-    } else {
-#pragma unroll
-      for (int j = 0; j < 4; j++)
-        if (e + j < a.cols) orow[e + j] = v[i][j];
-    }
+    store_chunk<OUT>(orow, (int64_t)seg * kSeg + 4 * (int64_t)(threadIdx.x + 256 * i), a.cols, a.vec, v[i]);
   }
 }
+
+// One work-group of 512 threads per row: its two halves are the 256-thread teams of two segments at a time
+// (slot k = segments 2k and 2k+1).  The first 28 full segments stay in registers (14 slots of 16 values per thread),
+// what follows (further full segments and the ragged last one) in LDS at its row offset.  Every reduction is the one
+// of the two-launch schedule, value for value.  Rows must allow vector access (a.vec).  The code is kept small on
+// purpose -- branch-free for full segments, run-time loops over the LDS part -- because it runs once per row and has
+// to stay in the instruction cache.
+template <int IN, int OUT, bool SOFTMAX>
+__global__ __launch_bounds__(512) void lsm_resident_kernel(const LsmArgs a) {
+  constexpr int RK = kResidentRegSegs / 2;  // register slots
+  constexpr int MAXSEG = (int)((kResidentMaxCols + kSeg - 1) / kSeg);
+  extern __shared__ __attribute__((aligned(16))) float lds_row[];   // [kResidentLdsFloats] row tail, then the statistics
+  float* red = lds_row + kResidentLdsFloats;                        // [MAXSEG][4] wave partials of a segment
+  float* stat = red + MAXSEG * 4;                                   // [MAXSEG][2] (max, sum) per segment, then 2 row values
+  typedef typename LsmElem<IN>::type in_t;
+  typedef typename LsmElem<OUT>::type out_t;
+  const int tid = threadIdx.x, half = tid >> 8, t = tid & 255, lane = tid & 63, wave = (tid >> 6) & 3;
+  const in_t* xr = static_cast<const in_t*>(a.x) + (int64_t)blockIdx.x * a.ldx;
+  out_t* orow = static_cast<out_t*>(a.out) + (int64_t)blockIdx.x * a.ldo;
+  const int cols = (int)a.cols, segs = a.segs;
+  const int nfull = cols >> 12;                                       // full segments
+  const int nreg = (nfull & ~1) < 2 * RK ? (nfull & ~1) : 2 * RK;     // ... of which in registers (whole slots)
+  const int nslot = nreg >> 1;
+  const int lds0 = nreg * kSeg;                                       // first row element that lives in LDS
+  const int t4 = 4 * t;
+  const int mine = half * kSeg + t4;  // thread's chunk i of slot k starts at row element k*8192 + mine + 1024*i
+
+  auto from_lds = [&](int sg, float (&u)[4][4]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int e = sg * kSeg + t4 + 1024 * i;
+      if (e >= cols) {   // only in the ragged segment: chunks past the end of the row have no place in LDS
+        u[i][0] = u[i][1] = u[i][2] = u[i][3] = -INFINITY;
+      } else {
+        const float4 q = *reinterpret_cast<const float4*>(lds_row + (e - lds0));
+        u[i][0] = q.x; u[i][1] = q.y; u[i][2] = q.z; u[i][3] = q.w;
+      }
+    }
+  };
+  auto finish = [&](int e0, float (&u)[4][4], bool ragged) __attribute__((always_inline)) {
+    const float gm = stat[2 * MAXSEG], lg = stat[2 * MAXSEG + 1];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const float y = (u[i][j] - gm) - lg;
+        u[i][j] = SOFTMAX ? fast_exp(y) : y;
+      }
+      if (!ragged) LsmElem<OUT>::store4(orow + e0 + 1024 * i, u[i]);
+      else store_chunk<OUT>(orow, e0 + 1024 * i, cols, 1, u[i]);
+    }
+  };
+
+  // ---- read the row once.  The part that lives in LDS goes first, four segments per team and round trip through
+  // registers that the register part does not occupy yet (one segment per round trip would cost a memory latency
+  // each); the loads of the register part are then all in flight together and are consumed in order.
+  constexpr int LB = 4;
+  for (int sg0 = nreg + half; sg0 < segs; sg0 += 2 * LB) {
+    float u[LB][4][4];
+#pragma unroll
+    for (int b = 0; b < LB; b++) {
+      const int sg = sg0 + 2 * b;
+      if (sg < nfull) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) LsmElem<IN>::load4(xr + sg * kSeg + t4 + 1024 * i, u[b][i]);
+      } else if (sg < segs) {   // the ragged last segment
+#pragma unroll
+        for (int i = 0; i < 4; i++) load_chunk<IN>(xr, sg * kSeg + t4 + 1024 * i, cols, 1, -INFINITY, u[b][i]);
+      }
+    }
+#pragma unroll
+    for (int b = 0; b < LB; b++) {
+      const int sg = sg0 + 2 * b;
+      if (sg < segs) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const int e = sg * kSeg + t4 + 1024 * i;
+          if (e < cols) *reinterpret_cast<float4*>(lds_row + (e - lds0)) = make_float4(u[b][i][0], u[b][i][1], u[b][i][2], u[b][i][3]);
+        }
+      }
+    }
+  }
+  float v[RK][4][4];
+#pragma unroll
+  for (int k = 0; k < RK; k++)
+    if (k < nslot) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) LsmElem<IN>::load4(xr + k * 2 * kSeg + mine + 1024 * i, v[k][i]);
+    }
+
+  // ---- segment maxima: per thread, butterfly, then the four wavefronts of the team in order
+#pragma unroll
+  for (int k = 0; k < RK; k++)
+    if (k < nslot) {
+      const float m = wave_max(seg_thread_max(v[k]));
+      if (lane == 0) red[(2 * k + half) * 4 + wave] = m;
+    }
+  for (int sg = nreg + half; sg < segs; sg += 2) {
+    float u[4][4];
+    from_lds(sg, u);
+    const float m = wave_max(seg_thread_max(u));
+    if (lane == 0) red[sg * 4 + wave] = m;
+  }
+  __syncthreads();
+  if (tid < segs) stat[2 * tid] = fmaxf(fmaxf(red[4 * tid], red[4 * tid + 1]), fmaxf(red[4 * tid + 2], red[4 * tid + 3]));
+  __syncthreads();
+  // ---- segment sums of exp(x - segment max)
+#pragma unroll
+  for (int k = 0; k < RK; k++)
+    if (k < nslot) {
+      const float sm = wave_sum(seg_thread_expsum(v[k], stat[2 * (2 * k + half)]));
+      if (lane == 0) red[(2 * k + half) * 4 + wave] = sm;
+    }
+  for (int sg = nreg + half; sg < segs; sg += 2) {
+    float u[4][4];
+    from_lds(sg, u);
+    const float sm = wave_sum(seg_thread_expsum(u, stat[2 * sg]));
+    if (lane == 0) red[sg * 4 + wave] = sm;
+  }
+  __syncthreads();
+  if (tid < segs) stat[2 * tid + 1] = ((red[4 * tid] + red[4 * tid + 1]) + red[4 * tid + 2]) + red[4 * tid + 3];
+  __syncthreads();
+  // ---- the row's (max, log sum): first wavefront, as in the two-launch schedule
+  if (tid < 64) {
+    float gmax, lg;
+    merge_segments(stat, segs, tid, gmax, lg);
+    if (tid == 0) {
+      stat[2 * MAXSEG] = gmax;
+      stat[2 * MAXSEG + 1] = lg;
+    }
+  }
+  __syncthreads();
+  // ---- write the row once
+#pragma unroll
+  for (int k = 0; k < RK; k++)
+    if (k < nslot) finish(k * 2 * kSeg + mine, v[k], false);
+  for (int sg = nreg + half; sg < segs; sg += 2) {
+    float u[4][4];
+    from_lds(sg, u);
+    if (sg < nfull) finish(sg * kSeg + t4, u, false);
+    else finish(sg * kSeg + t4, u, true);
+  }
+}
+
+// One launch with the row resident on chip once there are enough rows to occupy the CUs with one work-group each (same
+// bits either way); that schedule does not touch the workspace.
+static bool lsm_resident(int64_t rows, int64_t cols) { return cols <= kResidentMaxCols && rows >= 192; }
 
 size_t lsm_workspace_bytes(int64_t rows, int64_t cols) {
   if (rows <= 0 || cols <= 0) return 0;
@@ -264,34 +494,62 @@ size_t lsm_workspace_bytes(int64_t rows, int64_t cols) {
   return (size_t)rows * (size_t)segs * 2 * sizeof(float);
 }
 
-int log_softmax_dispatch(const void* x, int64_t ldx, void* out, int64_t ldo, int64_t rows, int64_t cols, void* ws,
-                         size_t ws_bytes, int write_softmax, hipStream_t stream) {
+template <int IN, int OUT>
+static int lsm_launch(const LsmArgs& a, bool resident, hipStream_t stream) {
+  if (resident) {
+    constexpr int lds = 160 * 1024;
+    if (a.write_softmax) {
+      static std::atomic<uint64_t> done{0};
+      hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(lsm_resident_kernel<IN, OUT, true>), lds, done);
+      if (e != hipSuccess) return hip_code(e);
+      hipLaunchKernelGGL((lsm_resident_kernel<IN, OUT, true>), dim3((unsigned)a.rows), dim3(512), lds, stream, a);
+    } else {
+      static std::atomic<uint64_t> done{0};
+      hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(lsm_resident_kernel<IN, OUT, false>), lds, done);
+      if (e != hipSuccess) return hip_code(e);
+      hipLaunchKernelGGL((lsm_resident_kernel<IN, OUT, false>), dim3((unsigned)a.rows), dim3(512), lds, stream, a);
+    }
+  } else {
+    const dim3 grid((unsigned)(a.rows * a.segs)), block(256);
+    hipLaunchKernelGGL((lsm_partial_kernel<IN>), grid, block, 0, stream, a);
+    hipLaunchKernelGGL((lsm_write_kernel<IN, OUT>), grid, block, 0, stream, a);
+  }
+  return hip_code(hipGetLastError());
+}
+
+// dtype codes: 0 fp32, 1 bf16, 2 fp16; the output is fp32 or the input's type
+int log_softmax_dispatch(const void* x, int64_t ldx, int in_dtype, void* out, int64_t ldo, int out_dtype, int64_t rows,
+                         int64_t cols, void* ws, size_t ws_bytes, int write_softmax, hipStream_t stream) {
   if (rows < 0 || cols <= 0 || ldx < cols || ldo < cols) return TBIK_ERR_INVALID;
+  if (in_dtype < 0 || in_dtype > 2 || (out_dtype != LSM_F32 && out_dtype != in_dtype)) return TBIK_ERR_UNSUPPORTED;
   if (rows == 0) return TBIK_OK;
   if (!x || !out) return TBIK_ERR_INVALID;
-  if ((reinterpret_cast<uintptr_t>(x) & 3) || (reinterpret_cast<uintptr_t>(out) & 3)) return TBIK_ERR_ALIGNMENT;
-  if (!ws || ws_bytes < lsm_workspace_bytes(rows, cols) || (reinterpret_cast<uintptr_t>(ws) & 3)) return TBIK_ERR_WORKSPACE;
+  const int isz = in_dtype == LSM_F32 ? 4 : 2, osz = out_dtype == LSM_F32 ? 4 : 2;
+  if ((reinterpret_cast<uintptr_t>(x) & (isz - 1)) || (reinterpret_cast<uintptr_t>(out) & (osz - 1))) return TBIK_ERR_ALIGNMENT;
   const int64_t segs = (cols + kSeg - 1) / kSeg;
   if (rows * segs > 0x7fffffff) return TBIK_ERR_INVALID;
+  // the vector and the scalar path read the same elements into the same registers: same order
+  const int vec = ((reinterpret_cast<uintptr_t>(x) & (4 * isz - 1)) == 0 && (reinterpret_cast<uintptr_t>(out) & (4 * osz - 1)) == 0 &&
+                   (ldx & 3) == 0 && (ldo & 3) == 0)
+                      ? 1
+                      : 0;
+  const bool resident = vec && lsm_resident(rows, cols);
+  if (!resident && (!ws || ws_bytes < lsm_workspace_bytes(rows, cols) || (reinterpret_cast<uintptr_t>(ws) & 3))) return TBIK_ERR_WORKSPACE;
   LsmArgs a;
-  a.x = static_cast<const float*>(x);
-  a.out = static_cast<float*>(out);
+  a.x = x;
+  a.out = out;
   a.ws = static_cast<float*>(ws);
   a.ldx = ldx;
   a.ldo = ldo;
   a.rows = rows;
   a.cols = cols;
   a.segs = (int)segs;
-  // the vector and the scalar path read the same elements into the same registers: same order
-  a.vec = ((reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0 && (ldx & 3) == 0 &&
-           (ldo & 3) == 0)
-              ? 1
-              : 0;
+  a.vec = vec;
   a.write_softmax = write_softmax;
-  const dim3 grid((unsigned)(rows * segs)), block(256);
-  hipLaunchKernelGGL(lsm_partial_kernel, grid, block, 0, stream, a);
-  hipLaunchKernelGGL(lsm_write_kernel, grid, block, 0, stream, a);
-  return hip_code(hipGetLastError());
+  if (in_dtype == LSM_F32) return lsm_launch<LSM_F32, LSM_F32>(a, resident, stream);
+  if (in_dtype == LSM_BF16)
+    return out_dtype == LSM_F32 ? lsm_launch<LSM_BF16, LSM_F32>(a, resident, stream) : lsm_launch<LSM_BF16, LSM_BF16>(a, resident, stream);
+  return out_dtype == LSM_F32 ? lsm_launch<LSM_F16, LSM_F32>(a, resident, stream) : lsm_launch<LSM_F16, LSM_F16>(a, resident, stream);
 }
 
 // ================================================================================================

@@ -263,34 +263,46 @@ def _(x, residual, weight, eps):
     return [torch.empty_like(x), torch.empty_like(x)]
 
 
-def _bi_log_softmax_f32_impl(x: torch.Tensor, write_softmax: bool) -> torch.Tensor:
+def _bi_log_softmax_impl(x: torch.Tensor, write_softmax: bool, to_float: bool) -> torch.Tensor:
+    """log_softmax (or softmax) over the last dimension of an fp32 / bf16 / fp16 tensor, in the input's dtype or,
+    with `to_float`, in fp32; the kernel reads the input dtype itself."""
     _require_gpu(x)
+    if x.dtype not in _DTYPE_CODE:
+        raise NotImplementedError(f"bi_log_softmax: unsupported dtype {x.dtype}")
     cols = x.shape[-1]
     x2 = x.reshape(-1, cols)
     if x2.stride(1) != 1 or (x2.shape[0] > 1 and x2.stride(0) < cols):
         x2 = x2.contiguous()
     rows = x2.shape[0]
-    out = torch.empty((rows, cols), device=x.device, dtype=torch.float32)
+    out_dtype = torch.float32 if to_float else x.dtype
+    out = torch.empty((rows, cols), device=x.device, dtype=out_dtype)
     L = _lib.lib()
-    ws = torch.empty((max(L.bi_log_softmax_workspace_bytes(rows, cols), 4) + 3) // 4, device=x.device, dtype=torch.float32)
-    rc = L.bi_log_softmax_f32(x2.data_ptr(), x2.stride(0) if rows > 1 else cols, out.data_ptr(), out.stride(0),
-                              rows, cols, ws.data_ptr(), ws.numel() * 4, int(write_softmax), _stream(x))
-    _lib.check(rc, "bi_log_softmax_f32")
+    nws = L.bi_log_softmax_workspace_bytes(rows, cols)
+    ws = torch.empty((nws + 3) // 4, device=x.device, dtype=torch.float32) if nws else None
+    rc = L.bi_log_softmax(x2.data_ptr(), x2.stride(0) if rows > 1 else cols, _DTYPE_CODE[x.dtype], out.data_ptr(),
+                          out.stride(0), _DTYPE_CODE[out_dtype], rows, cols, None if ws is None else ws.data_ptr(), nws,
+                          int(write_softmax), _stream(x))
+    _lib.check(rc, "bi_log_softmax")
     return out.reshape(x.shape)
 
 
-_bi_log_softmax_f32_op = torch.library.custom_op("tbik::bi_log_softmax_f32", _bi_log_softmax_f32_impl, mutates_args=(), device_types="cuda")
+_bi_log_softmax_op = torch.library.custom_op("tbik::bi_log_softmax", _bi_log_softmax_impl, mutates_args=(), device_types="cuda")
+
+
+def bi_log_softmax(x: torch.Tensor, write_softmax: bool, to_float: bool = False) -> torch.Tensor:
+    if torch.compiler.is_compiling():
+        return _bi_log_softmax_op(x, write_softmax, to_float)
+    return _bi_log_softmax_impl(x, write_softmax, to_float)
+
+
+@_bi_log_softmax_op.register_fake
+def _(x, write_softmax, to_float):
+    return torch.empty_like(x, dtype=torch.float32 if to_float else x.dtype)
 
 
 def bi_log_softmax_f32(x: torch.Tensor, write_softmax: bool) -> torch.Tensor:
-    if torch.compiler.is_compiling():
-        return _bi_log_softmax_f32_op(x, write_softmax)
-    return _bi_log_softmax_f32_impl(x, write_softmax)
-
-
-@_bi_log_softmax_f32_op.register_fake
-def _(x, write_softmax):
-    return torch.empty_like(x)
+    """fp32 in, fp32 out (kept for callers of the earlier name)."""
+    return bi_log_softmax(x.float(), write_softmax)
 
 
 def _bi_mean_dim_impl(x: torch.Tensor, dim: int, keepdim: bool) -> torch.Tensor:

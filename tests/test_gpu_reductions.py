@@ -103,6 +103,51 @@ def test_log_softmax_parity_and_batch_invariance(dev):
     assert bio.log_softmax(yb.to(dev)).dtype == torch.bfloat16
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_log_softmax_reads_16_bit_logits_in_the_kernel(dev, dtype):
+    """bf16 / fp16 logits go to the kernel as they are (no fp32 copy in front): result = the fp64 log_softmax of the
+    16-bit values rounded once to the output type; half_to_float gives the fp32 result of the same arithmetic; rows
+    alone, in a small batch (two launches) and in a large one (row resident on chip) agree bit for bit."""
+    from llm_reproducibility_amd import ops
+    V = 151936
+    g = torch.Generator().manual_seed(3)
+    x = (torch.randn((200, V), generator=g) * 3.0).to(dtype)
+    xd = x.to(dev)
+    full = bio.log_softmax(xd)                       # 200 rows: resident schedule
+    assert full.dtype == dtype
+    want = torch.log_softmax(x[:8].double(), dim=-1)
+    f32 = ops.bi_log_softmax(xd, False, True)
+    assert f32.dtype == torch.float32 and (f32[:8].cpu().double() - want).abs().max() < 2e-5
+    eps = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11       # one unit in the last place, relative
+    assert ((full[:8].cpu().double() - want).abs() <= eps * want.abs() + 1e-6).all()
+    assert torch.equal(full, f32.to(dtype))          # the 16-bit output is the fp32 result rounded once
+    for r in (1, 7, 191, 192):
+        assert torch.equal(bio.log_softmax(xd[:r]), full[:r]), r
+    assert torch.equal(bio.log_softmax(xd[100:101]), full[100:101])
+    sm = ops.bi_log_softmax(xd[:5], True, True)
+    assert (sm.cpu().double() - torch.softmax(x[:5].double(), -1)).abs().max() < 1e-6
+    # strided rows (a column block of a wider tensor), misaligned start, ragged width
+    wide = (torch.randn((260, 5003), generator=g)).to(dtype).to(dev)
+    view = wide[:, 3:5000]
+    got = bio.log_softmax(view)
+    assert ((got.cpu().double() - torch.log_softmax(view.cpu().double(), -1)).abs() <= eps * 12 + 1e-6).all()
+    assert torch.equal(got[:3], bio.log_softmax(view[:3]))
+
+
+def test_log_softmax_schedules_agree_on_widths_around_the_resident_limit(dev):
+    """fp32, 200 rows (one launch, row on chip) against the same rows in batches of 3 (two launches): same bits for
+    widths that end inside the register part, inside the LDS part, on the limit, and beyond it (two launches again)."""
+    g = torch.Generator().manual_seed(5)
+    for cols in (4096, 114688, 114689, 130001, 154624, 154625):
+        x = (torch.randn((200, cols), generator=g) * 2.0).to(dev)
+        big = bio.log_softmax(x)
+        for r0 in (0, 77, 197):
+            assert torch.equal(bio.log_softmax(x[r0:r0 + 3]), big[r0:r0 + 3]), (cols, r0)
+        want = torch.log_softmax(x[:2].cpu().double(), -1)
+        assert (big[:2].cpu().double() - want).abs().max() < 2e-5, cols
+        del x, big
+
+
 def test_mean_parity_and_batch_invariance(dev):
     g = torch.Generator().manual_seed(0)
     x = torch.randn((4096, 4096), generator=g)
