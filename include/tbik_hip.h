@@ -54,9 +54,14 @@ int tbik_tree_params(int K, int leaf_k, int* T, int* flb, int* level_k);
  * C[m,n] depends only on row m of A and column n of B -- not on M, N, the tile configuration or
  * the launch.
  *   A: element (m,k) at A[m*lda + k]                       (K contiguous)
- *   B: element (k,n) at B[k*ldb_k + n*ldb_n]; ldb_k == 1   (the nn.Linear weight [N,K], i.e.
- *      weight.t()) is the native layout; ldb_n == 1 (row-major [K,N]) returns
- *      TBIK_ERR_UNSUPPORTED in this build and is repacked by the caller.
+ *   B: element (k,n) at B[k*ldb_k + n*ldb_n], as the reference passes B's strides to its kernel
+ *      (src/tbik/tree_based_matmul.py:259-264).  ldb_k == 1 (the nn.Linear weight [N,K], i.e. weight.t()) is the
+ *      native layout of every kernel; ldb_n == 1 (row-major [K,N], what simple_matmul.py:11-14 hands over) is
+ *      consumed in place by the tiled kernels, which transpose 8x8 blocks in registers on the way to LDS -- same
+ *      MFMA chain, same bits, no copy (the large-M pipeline is built for [N,K] only, so big row-major problems run
+ *      slower than their [N,K] form).  The contiguous dimension's partner stride must be a multiple of 8 elements;
+ *      neither stride equal to 1 returns TBIK_ERR_UNSUPPORTED.
+ *      For ldb_n == 1 the workspace size is tbik_gemm_workspace_bytes_rowmajor_b(M,N,K,leaf_k,f16).
  *   C: element (m,n) at C[m*ldc + n]
  *   workspace: at least tbik_gemm_workspace_bytes(M,N,K,leaf_k) bytes, 16-byte aligned (may be NULL when 0)
  * Replaces: matmul_tp_persistent + matmul_kernel_tp_persistent,
@@ -77,6 +82,8 @@ int tbik_gemm_bf16(const void* A, int64_t lda,
  * Replaces: the in-register tensor `S` of the reference kernel, src/tbik/tree_based_matmul.py:85.
  */
 size_t tbik_gemm_workspace_bytes(int M, int N, int K, int leaf_k);
+/* The same for a row-major B[K,N] (ldb_n == 1); f16 != 0: for tbik_gemm_f16. */
+size_t tbik_gemm_workspace_bytes_rowmajor_b(int M, int N, int K, int leaf_k, int f16);
 
 /*
  * tbik_gemm_bf16 for callers that cannot allocate device memory: code under HIP graph capture, tight serving loops,

@@ -6,7 +6,7 @@ namespace tbik {
 int gemm_dispatch(bool tree, bool f16, const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C,
                   int64_t ldc, int M, int N, int K, int leaf_k, const void* bias, void* ws, size_t ws_bytes,
                   hipStream_t stream);
-size_t gemm_workspace_bytes(int M, int N, int K, int leaf_k, bool f16);
+size_t gemm_workspace_bytes(int M, int N, int K, int leaf_k, bool f16, bool rowmajor_b = false);
 int tree_combine_dispatch(const void* const* parts, int nparts, void* out, int64_t numel, bool f16, hipStream_t stream);
 int tree_combine_f32_dispatch(const void* const* parts, int nparts, void* out, int64_t numel, hipStream_t stream);
 int rmsnorm_dispatch(const void* x, int64_t ldx, const void* res, int64_t ldr, const void* w, void* out, int64_t ldo,
@@ -62,6 +62,9 @@ int tbik_tree_params(int K, int leaf_k, int* T, int* flb, int* level_k) {
 
 size_t tbik_gemm_workspace_bytes(int M, int N, int K, int leaf_k) { return tbik::gemm_workspace_bytes(M, N, K, leaf_k, false); }
 size_t tbik_gemm_f16_workspace_bytes(int M, int N, int K, int leaf_k) { return tbik::gemm_workspace_bytes(M, N, K, leaf_k, true); }
+size_t tbik_gemm_workspace_bytes_rowmajor_b(int M, int N, int K, int leaf_k, int f16) {
+  return tbik::gemm_workspace_bytes(M, N, K, leaf_k, f16 != 0, true);
+}
 
 int tbik_gemm_bf16(const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C, int64_t ldc, int M,
                    int N, int K, int leaf_k, const void* bias_or_null, void* workspace, size_t workspace_bytes,

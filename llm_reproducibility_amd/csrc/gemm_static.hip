@@ -8,7 +8,7 @@ namespace tbik {
 int gemm_dispatch(bool tree, bool f16, const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C,
                   int64_t ldc, int M, int N, int K, int leaf_k, const void* bias, void* ws, size_t ws_bytes,
                   hipStream_t stream);
-size_t gemm_workspace_bytes(int M, int N, int K, int leaf_k, bool f16);
+size_t gemm_workspace_bytes(int M, int N, int K, int leaf_k, bool f16, bool rowmajor_b = false);
 }  // namespace tbik
 
 // Every GPU the library runs on holds its own copy of this array, at its own address, until the process ends.  In host
@@ -46,7 +46,7 @@ extern "C" int tbik_gemm_bf16_static(const void* A, int64_t lda, const void* B, 
                                      tbik_stream_t stream) {
   if (M < 0 || N < 0 || K <= 0) return TBIK_ERR_INVALID;
   if (M == 0 || N == 0) return TBIK_OK;
-  const size_t need = tbik::gemm_workspace_bytes(M, N, K, leaf_k, false);
+  const size_t need = tbik::gemm_workspace_bytes(M, N, K, leaf_k, false, ldb_k != 1);
   if (need > (size_t)TBIK_STATIC_SCRATCH_BYTES) return TBIK_ERR_SCRATCH_LIMIT;  // before anything is launched
   void* ws = nullptr;
   if (need > 0) {

@@ -16,6 +16,12 @@
 //
 // Operand roles: W ([N,K], K contiguous) feeds the MFMA "A" port and X ([M,K]) the "B" port, so an
 // output lane holds 4 consecutive n of one m and stores them as one 8-byte word.
+//
+// WT = true: the weight operand is given row-major as B[K,N] (N contiguous, row stride ldw) -- what a plain
+// `x @ B` hands over (simple_matmul.py:11-14 of the reference; the reference kernel takes B's strides as they are,
+// src/tbik/tree_based_matmul.py:259-264).  It is consumed in place: a thread loads an 8(k) x 8(n) block as eight
+// 16-byte rows, transposes it in registers (v_perm_b32) and writes eight K-contiguous 16-byte chunks into the same
+// LDS tile layout, so fragments, MFMA chain and bits are those of the [N,K] form.
 #include "common.h"
 #include "gemm_args.h"
 
@@ -43,14 +49,15 @@ constexpr int BK = 64;  // K elements per LDS stage (8 chunks of 16 bytes per ro
 // The XOR spreads the 16 rows an MFMA fragment read touches over all banks.
 __device__ __forceinline__ int lds_off(int r, int c) { return r * BK + ((c ^ (r & 7)) << 3); }
 
-template <int WAVES_M, int WAVES_N, int TM, int TN, int LS, int LBMAX, bool TREE, bool F16>
+template <int WAVES_M, int WAVES_N, int TM, int TN, int LS, int LBMAX, bool TREE, bool F16, bool WT = false>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmArgs p) {
   using Num = Num16<F16>;
   constexpr int NT = WAVES_M * WAVES_N * 64;
   constexpr int BM = WAVES_M * TM * 16;
   constexpr int BN = WAVES_N * TN * 16;
   constexpr int XCH = (BM * 8 + NT - 1) / NT;  // 16-byte chunks of the X tile per thread
-  constexpr int WCH = (BN * 8 + NT - 1) / NT;
+  constexpr int WCH = WT ? 8 : (BN * 8 + NT - 1) / NT;  // WT: the eight k rows of this thread's 8x8 block
+  static_assert(!WT || NT >= BN, "one 8x8 block of the W tile per thread");
 
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
   constexpr int STAGE = (BM + BN) * BK;  // elements per LDS stage: X tile, then W tile
@@ -81,7 +88,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
   const int n0 = pid_n * BN;
 
   const uint16_t* Xs = p.X + blockIdx.y * p.k_shard;
-  const uint16_t* Ws = p.W + blockIdx.y * p.k_shard;
+  const uint16_t* Ws = p.W + blockIdx.y * p.k_shard * (WT ? p.ldw : 1);
   uint16_t* Cs = p.C + blockIdx.y * p.c_shard;
 
   // ---- global -> register staging (rows past the edge are clamped: their results are never stored)
@@ -96,13 +103,23 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
     xptr[i] = Xs + (int64_t)gr * p.ldx + c * 8;
     xdst[i] = lds_off(r, c);
   }
+  // WT: thread b < BN owns the block of k rows 8*(b%8) .. +7 and columns 8*(b/8) .. +7 of the tile (eight lanes
+  // that differ in the k block read one full 128-byte line of each of eight k rows and write one LDS row)
+  const int wt_kb = tid & 7, wt_nb = tid >> 3;
+  const bool wt_active = WT && tid < BN;
+  const bool wt_full = WT && (n0 + wt_nb * 8 + 8 <= p.N);   // else: the block crosses the edge, loaded element-wise
 #pragma unroll
   for (int i = 0; i < WCH; i++) {
-    const int q = tid + i * NT;
-    const int r = (q >> 3) % BN, c = q & 7;
-    const int gr = min(n0 + r, p.N - 1);
-    wptr[i] = Ws + (int64_t)gr * p.ldw + c * 8;
-    wdst[i] = lds_off(r, c);
+    if (WT) {
+      wptr[i] = Ws + (int64_t)(wt_kb * 8 + i) * p.ldw + n0 + wt_nb * 8;
+      wdst[i] = lds_off(wt_nb * 8 + i, wt_kb);   // destination of the transposed chunk for column 8*nb + i
+    } else {
+      const int q = tid + i * NT;
+      const int r = (q >> 3) % BN, c = q & 7;
+      const int gr = min(n0 + r, p.N - 1);
+      wptr[i] = Ws + (int64_t)gr * p.ldw + c * 8;
+      wdst[i] = lds_off(r, c);
+    }
   }
   // Staging registers.  Large tree tiles load one stage ahead (their merge stack needs the registers); the
   // single-accumulator mm (no K split, so often a small grid in which every work-group is a chain of memory round
@@ -124,13 +141,37 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
           xreg[i] = u32x4{0, 0, 0, 0};
       }
     }
+    if (WT) {
+      if (wt_active) {
+        const bool k_ok = TREE || k0 + wt_kb * 8 < p.K;   // K is a multiple of 8: a block is inside or outside
 #pragma unroll
-    for (int i = 0; i < WCH; i++) {
-      if ((BN * 8) % NT == 0 || tid + i * NT < BN * 8) {
-        if (TREE || k0 + (tid & 7) * 8 < p.K)
-          wreg[i] = *reinterpret_cast<const u32x4*>(wptr[i] + k0);
-        else
-          wreg[i] = u32x4{0, 0, 0, 0};
+        for (int i = 0; i < WCH; i++) {
+          const uint16_t* src = wptr[i] + (int64_t)k0 * p.ldw;
+          if (!k_ok) {
+            wreg[i] = u32x4{0, 0, 0, 0};
+          } else if (wt_full) {
+            wreg[i] = *reinterpret_cast<const u32x4*>(src);
+          } else {
+            uint32_t w4[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              const int c0 = min(n0 + wt_nb * 8 + 2 * e, p.N - 1) - (n0 + wt_nb * 8);      // clamped: never stored
+              const int c1 = min(n0 + wt_nb * 8 + 2 * e + 1, p.N - 1) - (n0 + wt_nb * 8);
+              w4[e] = (uint32_t)src[c0] | ((uint32_t)src[c1] << 16);
+            }
+            wreg[i] = u32x4{w4[0], w4[1], w4[2], w4[3]};
+          }
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < WCH; i++) {
+        if ((BN * 8) % NT == 0 || tid + i * NT < BN * 8) {
+          if (TREE || k0 + (tid & 7) * 8 < p.K)
+            wreg[i] = *reinterpret_cast<const u32x4*>(wptr[i] + k0);
+          else
+            wreg[i] = u32x4{0, 0, 0, 0};
+        }
       }
     }
   };
@@ -140,9 +181,24 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
 #pragma unroll
     for (int i = 0; i < XCH; i++)
       if ((BM * 8) % NT == 0 || tid + i * NT < BM * 8) *reinterpret_cast<u32x4*>(smem + buf * STAGE + xdst[i]) = xreg[i];
+    if (WT) {
+      if (wt_active) {
+        // 8x8 transpose of 16-bit elements: column j of the block = (row 0..7).half[j]; word w of the output pairs
+        // k rows 2w and 2w+1 (low half = the even row)
 #pragma unroll
-    for (int i = 0; i < WCH; i++)
-      if ((BN * 8) % NT == 0 || tid + i * NT < BN * 8) *reinterpret_cast<u32x4*>(smem + buf * STAGE + BM * BK + wdst[i]) = wreg[i];
+        for (int j = 0; j < 8; j++) {
+          u32x4 o;
+#pragma unroll
+          for (int w = 0; w < 4; w++)
+            o[w] = __builtin_amdgcn_perm(wreg[2 * w + 1][j >> 1], wreg[2 * w][j >> 1], (j & 1) ? 0x07060302u : 0x05040100u);
+          *reinterpret_cast<u32x4*>(smem + buf * STAGE + BM * BK + wdst[j]) = o;
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < WCH; i++)
+        if ((BN * 8) % NT == 0 || tid + i * NT < BN * 8) *reinterpret_cast<u32x4*>(smem + buf * STAGE + BM * BK + wdst[i]) = wreg[i];
+    }
   };
 
   // ---- fragment addressing: lane l reads row (l%16), 16-byte chunk kk*4 + l/16
@@ -301,13 +357,13 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
 // ------------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------------
-template <int WAVES_M, int WAVES_N, int TM, int TN, int LS, int LBMAX, bool TREE, bool F16>
+template <int WAVES_M, int WAVES_N, int TM, int TN, int LS, int LBMAX, bool TREE, bool F16, bool WT = false>
 static int launch(const GemmArgs& a, int split, hipStream_t stream) {
   constexpr int NT = WAVES_M * WAVES_N * 64;
   constexpr int BM = WAVES_M * TM * 16;
   constexpr int BN = WAVES_N * TN * 16;
   constexpr size_t smem = (size_t)2 * (BM + BN) * BK * sizeof(uint16_t);
-  auto kern = gemm_kernel<WAVES_M, WAVES_N, TM, TN, LS, LBMAX, TREE, F16>;
+  auto kern = gemm_kernel<WAVES_M, WAVES_N, TM, TN, LS, LBMAX, TREE, F16, WT>;
   if (smem > 48 * 1024) {
     static std::atomic<uint64_t> done{0};
     hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), (int)smem, done);
@@ -332,6 +388,13 @@ static int launch_by_m(const GemmArgs& a, int split, hipStream_t stream) {
   return launch<2, 2, 4, 4, LS, LBMAX, TREE, F16>(a, split, stream);
 }
 
+// Row-major B[K,N]: two tile shapes (16 and 64 rows), the deepest merge stack
+template <int LS, int LBMAX, bool TREE, bool F16>
+static int launch_rowmajor_b(const GemmArgs& a, int split, hipStream_t stream) {
+  if (a.M <= 16) return launch<1, 4, 1, 1, LS, LBMAX, TREE, F16, true>(a, split, stream);
+  return launch<1, 4, 4, 2, LS, LBMAX, TREE, F16, true>(a, split, stream);
+}
+
 template <int LS, bool F16>
 static int launch_tree(const GemmArgs& a, int split, hipStream_t stream) {
   if (a.lb <= 2) return launch_by_m<LS, 2, true, F16>(a, split, stream);
@@ -352,7 +415,7 @@ struct Plan {
   size_t partial_bytes, parked_bytes;
 };
 
-static bool make_plan(int M, int N, int K, int leaf_k, bool f16, Plan* pl) {
+static bool make_plan(int M, int N, int K, int leaf_k, bool f16, Plan* pl, bool rowmajor_b = false) {
   int T, flb, level_k;
   if (M <= 0 || N <= 0 || tbik_tree_params(K, leaf_k, &T, &flb, &level_k) != TBIK_OK) return false;
   const int lb = level_k - 1;
@@ -360,7 +423,7 @@ static bool make_plan(int M, int N, int K, int leaf_k, bool f16, Plan* pl) {
   const int64_t wide_tiles = (int64_t)((M + 127) / 128) * ((N + 255) / 256);
   int split = 1;
   bool wide = false;
-  if (M >= 64 && !f16) {  // the wide kernel exists for bf16 only
+  if (M >= 64 && !f16 && !rowmajor_b) {  // the wide kernel exists for bf16 and [N,K] weights only
     // Estimated time of the wide kernel for each legal split: work-group rounds on 256 CUs times the K extent of
     // one shard, plus the shard-combine pass over (split + 1) [M,N] arrays.  Constants are measured on MI355X
     // (17 ns per k per round; 5 TB/s and 4 us for the combine).
@@ -378,7 +441,7 @@ static bool make_plan(int M, int N, int K, int leaf_k, bool f16, Plan* pl) {
     wide = wide_tiles * split >= 64;
   }
   if (!wide) {
-    const int bm = M <= 16 ? 16 : (M <= 64 ? 64 : 128), bn = M <= 16 ? 64 : 128;
+    const int bm = M <= 16 ? 16 : ((M <= 64 || rowmajor_b) ? 64 : 128), bn = M <= 16 ? 64 : 128;
     const int64_t tiles = (int64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
     split = 1;
     while (tiles * split < 512 && split < max_split && split < 8) split *= 2;
@@ -396,9 +459,10 @@ static bool make_plan(int M, int N, int K, int leaf_k, bool f16, Plan* pl) {
   return true;
 }
 
-size_t gemm_workspace_bytes(int M, int N, int K, int leaf_k, bool f16) {
+size_t gemm_workspace_bytes(int M, int N, int K, int leaf_k, bool f16, bool rowmajor_b) {
   Plan pl;
-  if (!make_plan(M, N, K, leaf_k, f16, &pl)) return 0;
+  if (!make_plan(M, N, K, leaf_k, f16, &pl, rowmajor_b)) return 0;
+  if (rowmajor_b) return pl.partial_bytes;
   if (gemm_tree_strip_waves(M, N, K, pl.lb + (pl.split > 1 ? __builtin_ctz((unsigned)pl.split) : 0))) return 0;  // no workspace on that path
   return pl.partial_bytes + pl.parked_bytes;
 }
@@ -409,9 +473,13 @@ int gemm_dispatch(bool tree, bool f16, const void* A, int64_t lda, const void* B
   if (M < 0 || N < 0 || K <= 0) return TBIK_ERR_INVALID;
   if (M == 0 || N == 0) return TBIK_OK;  // nothing to do (empty tensors may come with null pointers)
   if (!A || !B || !C) return TBIK_ERR_INVALID;
-  if (ldb_k != 1) return TBIK_ERR_UNSUPPORTED;  // row-major [K,N] weights are repacked by the caller
-  if (lda < K || ldb_n < K || ldc < N) return TBIK_ERR_INVALID;
-  if (!aligned16(A) || !aligned16(B) || (lda & 7) || (ldb_n & 7) || (K & 7)) return TBIK_ERR_ALIGNMENT;
+  // B[K,N] row-major (ldb_n == 1) is consumed in place by the tiled kernels; [N,K] K-contiguous (ldb_k == 1, the
+  // nn.Linear weight) is the native layout of all of them
+  const bool rowmajor_b = ldb_k != 1;
+  if (rowmajor_b && ldb_n != 1) return TBIK_ERR_UNSUPPORTED;  // neither dimension contiguous
+  const int64_t ldw = rowmajor_b ? ldb_k : ldb_n;
+  if (lda < K || ldw < (rowmajor_b ? N : K) || ldc < N) return TBIK_ERR_INVALID;
+  if (!aligned16(A) || !aligned16(B) || (lda & 7) || (ldw & 7) || (K & 7)) return TBIK_ERR_ALIGNMENT;
   if (reinterpret_cast<uintptr_t>(C) & 1) return TBIK_ERR_ALIGNMENT;
 
   GemmArgs a;
@@ -420,7 +488,7 @@ int gemm_dispatch(bool tree, bool f16, const void* A, int64_t lda, const void* B
   a.C = static_cast<uint16_t*>(C);
   a.bias = static_cast<const uint16_t*>(bias);
   a.ldx = lda;
-  a.ldw = ldb_n;
+  a.ldw = ldw;
   a.ldc = ldc;
   a.M = M;
   a.N = N;
@@ -431,6 +499,8 @@ int gemm_dispatch(bool tree, bool f16, const void* A, int64_t lda, const void* B
   a.vec_store = ((reinterpret_cast<uintptr_t>(C) & 7) == 0 && (ldc & 3) == 0) ? 1 : 0;
   a.k_shard = 0;
   a.c_shard = 0;
+  if (!tree && rowmajor_b)
+    return f16 ? launch_rowmajor_b<4, 0, false, true>(a, 1, stream) : launch_rowmajor_b<4, 0, false, false>(a, 1, stream);
   if (!tree) {
     // large problems whose K is a whole number of 64-wide slices take the one-wave-per-SIMD pipeline (same MFMA
     // chain per element, so the same bits as the tiled kernel)
@@ -455,7 +525,7 @@ int gemm_dispatch(bool tree, bool f16, const void* A, int64_t lda, const void* B
   }
 
   if (leaf_k != 256 && leaf_k != 128) return TBIK_ERR_UNSUPPORTED;
-  {
+  if (!rowmajor_b) {
     // a handful of rows: one launch, K cut over the waves of a work-group, nothing goes through the workspace
     int T, flb, level_k;
     if (tbik_tree_params(K, leaf_k, &T, &flb, &level_k) != TBIK_OK) return TBIK_ERR_INVALID;
@@ -466,7 +536,7 @@ int gemm_dispatch(bool tree, bool f16, const void* A, int64_t lda, const void* B
     }
   }
   Plan pl;
-  if (!make_plan(M, N, K, leaf_k, f16, &pl)) return TBIK_ERR_INVALID;
+  if (!make_plan(M, N, K, leaf_k, f16, &pl, rowmajor_b)) return TBIK_ERR_INVALID;
   const size_t need = pl.partial_bytes + pl.parked_bytes;
   if (need > 0 && (!ws || ws_bytes < need || !aligned16(ws))) return TBIK_ERR_WORKSPACE;
   uint8_t* wsb = static_cast<uint8_t*>(ws);
@@ -484,7 +554,11 @@ int gemm_dispatch(bool tree, bool f16, const void* A, int64_t lda, const void* B
     a.bias = nullptr;
   }
   int rc;
-  if (pl.wide) {
+  if (rowmajor_b) {
+    if (a.lb > 6) return TBIK_ERR_UNSUPPORTED;
+    if (f16) rc = leaf_k == 256 ? launch_rowmajor_b<4, 6, true, true>(a, pl.split, stream) : launch_rowmajor_b<2, 6, true, true>(a, pl.split, stream);
+    else rc = leaf_k == 256 ? launch_rowmajor_b<4, 6, true, false>(a, pl.split, stream) : launch_rowmajor_b<2, 6, true, false>(a, pl.split, stream);
+  } else if (pl.wide) {
     WideArgs w{a.X, a.W, a.C, a.bias, reinterpret_cast<u32x4*>(wsb + pl.partial_bytes), a.ldx, a.ldw, a.ldc, M, N, a.K,
                a.T, a.flb, a.lb, a.vec_store, a.k_shard, a.c_shard};
     rc = gemm_tree_wide_launch(w, leaf_k, pl.split, stream);

@@ -89,10 +89,19 @@ def _rows16(t: torch.Tensor):
     return c, c.shape[1]
 
 
-def _weight_nk(B: torch.Tensor):
-    """The [N,K] K-contiguous form of a [K,N] operand (the nn.Linear weight layout) and its leading
-    dimension; `weight.t()` is used as it is, a row-major [K,N] operand is repacked."""
-    return _rows16(B.t())
+def _weight_operand(B: torch.Tensor):
+    """How a [K,N] operand is handed to the kernels without a copy: (tensor whose data_ptr is passed, ldb_k, ldb_n).
+
+    `weight.t()` of an nn.Linear weight ([N,K], K contiguous) is the native layout (ldb_k = 1); a row-major [K,N]
+    operand (N contiguous: a plain `x @ B`) is consumed in place too (ldb_n = 1).  Anything else -- neither dimension
+    contiguous, rows not 16-byte aligned -- is repacked once into the native layout."""
+    K, N = B.shape
+    if B.stride(0) == 1 and _aligned16(B) and K % 8 == 0 and (N == 1 or (B.stride(1) >= K and B.stride(1) % 8 == 0)):
+        return B, 1, (K if N == 1 else B.stride(1))
+    if B.stride(1) == 1 and _aligned16(B) and B.stride(0) >= N and B.stride(0) % 8 == 0:
+        return B, B.stride(0), 1
+    w, ldw = _rows16(B.t())
+    return w, 1, ldw
 
 
 # --------------------------------------------------------------------------------------------
@@ -105,14 +114,17 @@ def _gemm_tree_impl(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.Tenso
     M, K = A.shape
     N = B.shape[1]
     a, lda = _rows16(A)
-    w, ldw = _weight_nk(B)
+    w, ldb_k, ldb_n = _weight_operand(B)
     b = None if bias is None else bias.contiguous()
     f16 = _is_f16(A, B, bias)
     C = torch.empty((M, N), device=A.device, dtype=A.dtype)
     L = _lib.lib()
-    ws_bytes = (L.tbik_gemm_f16_workspace_bytes if f16 else L.tbik_gemm_workspace_bytes)(M, N, K, leaf_k)
+    if ldb_k != 1:
+        ws_bytes = L.tbik_gemm_workspace_bytes_rowmajor_b(M, N, K, leaf_k, int(f16))
+    else:
+        ws_bytes = (L.tbik_gemm_f16_workspace_bytes if f16 else L.tbik_gemm_workspace_bytes)(M, N, K, leaf_k)
     ws = torch.empty(ws_bytes, device=A.device, dtype=torch.uint8) if ws_bytes else None
-    rc = (L.tbik_gemm_f16 if f16 else L.tbik_gemm_bf16)(a.data_ptr(), lda, w.data_ptr(), 1, ldw, C.data_ptr(), C.stride(0),
+    rc = (L.tbik_gemm_f16 if f16 else L.tbik_gemm_bf16)(a.data_ptr(), lda, w.data_ptr(), ldb_k, ldb_n, C.data_ptr(), C.stride(0),
                           M, N, K, leaf_k, None if b is None else b.data_ptr(),
                           None if ws is None else ws.data_ptr(), ws_bytes, _stream(A))
     _lib.check(rc, "tbik_gemm_bf16")
@@ -180,11 +192,11 @@ def _bi_gemm_impl(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.Tensor]
         B = torch.nn.functional.pad(B, (0, 0, 0, pad))
         K += pad
     a, lda = _rows16(A)
-    w, ldw = _weight_nk(B)
+    w, ldb_k, ldb_n = _weight_operand(B)
     b = None if bias is None else bias.contiguous()
     C = torch.empty((M, N), device=A.device, dtype=A.dtype)
     L = _lib.lib()
-    rc = (L.bi_gemm_f16 if _is_f16(A, B, bias) else L.bi_gemm_bf16)(a.data_ptr(), lda, w.data_ptr(), 1, ldw, C.data_ptr(), C.stride(0),
+    rc = (L.bi_gemm_f16 if _is_f16(A, B, bias) else L.bi_gemm_bf16)(a.data_ptr(), lda, w.data_ptr(), ldb_k, ldb_n, C.data_ptr(), C.stride(0),
                                  M, N, K, None if b is None else b.data_ptr(), _stream(A))
     _lib.check(rc, "bi_gemm")
     return C

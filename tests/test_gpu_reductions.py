@@ -256,6 +256,31 @@ def test_single_accumulator_mm_c_abi_strided_and_misaligned_output(dev, M, N, K)
         assert bool((wide[:, :shift] == 7).all()) and bool((wide[:, shift + N:] == 7).all()), "wrote outside its block"
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 100, 200), (7, 64, 4096), (33, 1000, 328), (200, 520, 1024)])
+def test_single_accumulator_mm_row_major_b_in_place(dev, M, N, K):
+    """mm_batch_invariant on a plain row-major [K,N] operand (what `x @ W` hands to the aten override, backward
+    matmuls included): no copy of B, integer inputs bit-exact vs the oracle, rows independent of the batch."""
+    from llm_reproducibility_amd import _lib
+    L = _lib.lib()
+    a = O.integer_bf16((M, K), -9, 9, 1)
+    bw = O.integer_bf16((K, N + (-N) % 8), -7, 7, 2)
+    b = bw[:, :N]
+    bias = O.integer_bf16((N,), -300, 300, 3)
+    want = O.matmul_single_acc(a, b, bias)
+    ad, bd, biasd = a.to(dev), bw.to(dev), bias.to(dev)
+    C = torch.empty((M, N), device=dev, dtype=torch.bfloat16)
+    rc = L.bi_gemm_bf16(ad.data_ptr(), K, bd.data_ptr(), bw.shape[1], 1, C.data_ptr(), N, M, N, K, biasd.data_ptr(),
+                        torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, rc
+    torch.cuda.synchronize()
+    assert torch.equal(C.cpu(), want)
+    got = bio.matmul_persistent(ad, bd[:, :N], biasd)
+    assert torch.equal(got.cpu(), want)
+    assert torch.equal(bio.matmul_persistent(ad[:1], bd[:, :N], biasd), got[:1])
+    with bio.set_batch_invariant_mode(True):
+        assert torch.equal((ad @ bd[:, :N]).cpu(), O.matmul_single_acc(a, b))
+
+
 def test_single_accumulator_mm_fp16(dev):
     a = O.gaussian_bf16((300, 1000), 1.0, 0).to(torch.float16)
     w = O.gaussian_bf16((200, 1000), 0.05, 1).to(torch.float16)

@@ -150,6 +150,56 @@ def test_bias_strided_a_and_row_major_b(dev):
     assert_bitwise(matmul_tp_persistent(odd, B.to(dev)), O.matmul_tree(A_wide[:, 3:3 + K], B), "misaligned A")
 
 
+# (M, N, K, leaf): row-major B[K,N] consumed in place -- both tile shapes, column tails that cut an 8-wide block
+# (N = 100, 1001 elements... with a row stride that is a multiple of 8), the K-cut path, leaf 128, deep trees
+ROWMAJOR_SHAPES = [(1, 64, 512, 256), (16, 104, 768, 256), (17, 200, 1536, 256), (70, 136, 2048, 256), (300, 1000, 1024, 256),
+                   (33, 96, 3200, 128), (8, 24, 8192, 256), (130, 4096, 12288, 256), (64, 72, 6400, 128)]
+
+
+@pytest.mark.parametrize("M,N,K,leaf", ROWMAJOR_SHAPES)
+def test_row_major_b_is_consumed_in_place_bitwise(dev, M, N, K, leaf):
+    """The C ABI with ldb_n == 1 (B[K,N], N contiguous, the layout of simple_matmul.py): no repack anywhere -- the raw
+    entry point is called on the row-major buffer -- and the bits equal the oracle's and the [N,K] path's."""
+    from llm_reproducibility_amd import _lib
+    L = _lib.lib()
+    print("case", M, N, K, leaf, flush=True)
+    A = O.integer_bf16((M, K), -9, 9, 50 + M)
+    ldb = N + (-N) % 8 + 8                                   # row stride: a multiple of 8, wider than N
+    Bw = O.integer_bf16((K, ldb), -7, 7, 60 + N % 89)
+    B = Bw[:, :N]
+    bias = O.integer_bf16((N,), -300, 300, 7)
+    want = O.matmul_tree(A, B, bias, leaf=leaf)
+    Ad, Bd, bd = A.to(dev), Bw.to(dev), bias.to(dev)
+    nws = L.tbik_gemm_workspace_bytes_rowmajor_b(M, N, K, leaf, 0)
+    ws = torch.empty(max(nws, 1), device=dev, dtype=torch.uint8)
+    C = torch.empty((M, N), device=dev, dtype=torch.bfloat16)
+    rc = L.tbik_gemm_bf16(Ad.data_ptr(), K, Bd.data_ptr(), ldb, 1, C.data_ptr(), N, M, N, K, leaf, bd.data_ptr(),
+                          ws.data_ptr() if nws else None, nws, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, rc
+    torch.cuda.synchronize()
+    assert_bitwise(C, want, "row-major B through the C ABI")
+    # the wrapper hands a row-major view over as it is (same bits as the [N,K] form, which runs other kernels)
+    got = matmul_tp_persistent(Ad, Bd[:, :N], bd, leaf_k=leaf)
+    assert_bitwise(got, want, "row-major B through the wrapper")
+    assert_bitwise(matmul_tp_persistent(Ad, Bd[:, :N].t().contiguous().t(), bd, leaf_k=leaf), want, "[N,K] form")
+    if leaf == 256 and M <= 70:
+        h = matmul_tp_persistent(Ad.to(torch.float16), Bd[:, :N].to(torch.float16), leaf_k=leaf)
+        assert_bitwise(h, O.matmul_tree(A.to(torch.float16), B.to(torch.float16), leaf=leaf), "fp16, row-major B")
+
+
+def test_row_major_b_simulated_tp_as_the_reference_script_runs_it(dev):
+    """simple_matmul.py:23-43 on its own layout: A[M,K] and B[K,N] both row-major, K cut into shards by slicing rows of
+    B (still row-major views), shard outputs combined in the tree: bitwise equal to the unsplit product."""
+    M, K, N = 96, 6144, 520
+    A = O.gaussian_bf16((M, K), 1.0, 0).to(dev)
+    B = O.gaussian_bf16((K, N), 1.0, 1).to(dev)
+    full = matmul_tp_persistent(A, B)
+    for p in (2, 4, 8):
+        assert_bitwise(sim_tp(A, B, p, 256), full, f"TP={p}")
+    assert_bitwise(matmul_tp_persistent(A[:7], B), full[:7], "batch prefix")
+    assert_close_to_oracle(full, O.matmul_tree(A.cpu(), B.cpu()), "row-major B, Gaussian")
+
+
 @pytest.mark.parametrize("M,N,K", [(256, 4096, 4096), (128, 512, 12288), (16, 256, 12288), (1, 128, 8192)])
 def test_gaussian_inputs_within_one_ulp_of_oracle(dev, M, N, K):
     print("case", M, N, K, flush=True)

@@ -49,7 +49,11 @@ def test_host_argument_checks_fire_before_any_launch():
     p = ctypes.addressof(buf)
     p16 = (p + 15) & ~15
     assert L.tbik_gemm_bf16(p16, 300, p16, 1, 300, p16, 8, 1, 8, 300, 256, None, None, 0, None) == _lib.TBIK_ERR_ALIGNMENT
-    assert L.tbik_gemm_bf16(p16, 512, p16, 512, 1, p16, 8, 1, 8, 512, 256, None, None, 0, None) == _lib.TBIK_ERR_UNSUPPORTED
+    # B with neither dimension contiguous is not taken; a row-major B (ldb_n == 1) is, so its checks fire instead
+    assert L.tbik_gemm_bf16(p16, 512, p16, 512, 2, p16, 8, 1, 8, 512, 256, None, None, 0, None) == _lib.TBIK_ERR_UNSUPPORTED
+    assert L.tbik_gemm_bf16(p16, 512, p16, 4, 1, p16, 8, 1, 8, 512, 256, None, None, 0, None) == _lib.TBIK_ERR_INVALID      # ldb_k < N
+    assert L.tbik_gemm_bf16(p16, 512, p16, 12, 1, p16, 8, 1, 8, 512, 256, None, None, 0, None) == _lib.TBIK_ERR_ALIGNMENT  # ldb_k % 8
+    assert L.tbik_gemm_workspace_bytes_rowmajor_b(128, 4096, 12288, 256, 0) > 0
     assert L.tbik_gemm_bf16(p16 + 2, 512, p16, 1, 512, p16, 8, 1, 8, 512, 256, None, None, 0, None) == _lib.TBIK_ERR_ALIGNMENT
     assert L.tbik_gemm_bf16(p16, 384, p16, 1, 384, p16, 8, 1, 8, 384, 256, None, None, 0, None) == _lib.TBIK_ERR_INVALID
     arr = (ctypes.c_void_p * 3)(p16, p16, p16)
