@@ -126,8 +126,9 @@ def ceiling(settle_ms):
     return res
 
 
-def table(steps, warmup, hot=False):
-    """Per-shape figures.  Unless `hot`, every case cycles through enough distinct input sets (more than 768 MB in
+def table(steps, warmup, hot=False, settle_ms=20.0):
+    """Per-shape figures, each after `settle_ms` of the same call run back to back (the settled rate, as for the
+    headline).  Unless `hot`, every case cycles through enough distinct input sets (more than 768 MB in
     all) that nothing it reads is still in the 256 MB memory-side cache from the previous call: the GB/s are HBM
     figures, as in a model whose every layer has its own weights."""
     import torch
@@ -152,7 +153,7 @@ def table(steps, warmup, hot=False):
         def make():
             return (torch.randn((M, K), device=dev).to(torch.bfloat16), (torch.randn((N, K), device=dev) * 0.02).to(torch.bfloat16))
         fl, by = 2.0 * M * N * K, 2.0 * (M * K + K * N + M * N)
-        ms, _ = hip_time_ms(cycling(make, by, lambda X, W: matmul_tp_persistent(X, W.t(), leaf_k=leaf)), steps, warmup)
+        ms, _ = hip_time_ms(cycling(make, by, lambda X, W: matmul_tp_persistent(X, W.t(), leaf_k=leaf)), steps, warmup, settle_ms)
         rows.append((name, ms * 1e3, fl / ms / 1e9, by / ms / 1e6))
 
     for M in (1, 16, 128, 2048):
@@ -162,7 +163,7 @@ def table(steps, warmup, hot=False):
         def make():
             return (torch.randn((M, K), device=dev).to(torch.bfloat16), (torch.randn((N, K), device=dev) * 0.02).to(torch.bfloat16))
         fl, by = 2.0 * M * N * K, 2.0 * (M * K + K * N + M * N)
-        ms, _ = hip_time_ms(cycling(make, by, lambda X, W: torch.matmul(X, W.t())), steps, warmup)
+        ms, _ = hip_time_ms(cycling(make, by, lambda X, W: torch.matmul(X, W.t())), steps, warmup, settle_ms)
         rows.append((f"  [torch.matmul, not invariant] M={M} K={K} N={N}", ms * 1e3, fl / ms / 1e9, by / ms / 1e6))
 
     for M in (1, 128, 2048):
@@ -183,34 +184,39 @@ def table(steps, warmup, hot=False):
         def make(M=M, K=K, N=N):
             return (torch.randn((M, K), device=dev).to(torch.bfloat16), (torch.randn((N, K), device=dev) * 0.02).to(torch.bfloat16))
         by = 2.0 * (M * K + K * N + M * N)
-        ms, _ = hip_time_ms(cycling(make, by, lambda X, W: bio.matmul_persistent(X, W.t())), steps, warmup)
+        ms, _ = hip_time_ms(cycling(make, by, lambda X, W: bio.matmul_persistent(X, W.t())), steps, warmup, settle_ms)
         rows.append((f"batch-invariant mm {name} M={M} K={K} N={N}", ms * 1e3, 2.0 * M * N * K / ms / 1e9, by / ms / 1e6))
     for p in (2, 4, 8):
         by = (p + 1) * 2048 * 4096 * 2
         make = lambda p=p: ([torch.randn((2048, 4096), device=dev).to(torch.bfloat16) for _ in range(p)],)  # noqa: E731
-        ms, _ = hip_time_ms(cycling(make, by, tree_combine), steps, warmup)
+        ms, _ = hip_time_ms(cycling(make, by, tree_combine), steps, warmup, settle_ms)
         rows.append((f"tree_combine p={p} [2048,4096]", ms * 1e3, 0.0, by / ms / 1e6))
     w = torch.ones(4096, device=dev, dtype=torch.bfloat16)
     for r in (1, 7, 256, 4096):
         by = r * 4096 * 4 + 8192
         make = lambda r=r: (torch.randn((r, 4096), device=dev).to(torch.bfloat16),)  # noqa: E731
-        ms, _ = hip_time_ms(cycling(make, by, lambda x: bio.rms_norm(x, w, 1e-6)), steps, warmup)
+        ms, _ = hip_time_ms(cycling(make, by, lambda x: bio.rms_norm(x, w, 1e-6)), steps, warmup, settle_ms)
         rows.append((f"rmsnorm rows={r} hidden=4096", ms * 1e3, 0.0, by / ms / 1e6))
     for r in (1, 7, 256, 4096):
         by = r * 151936 * 8
         make = lambda r=r: (torch.randn((r, 151936), device=dev),)  # noqa: E731
-        ms, _ = hip_time_ms(cycling(make, by, bio.log_softmax), max(steps // 4, 3), warmup)
+        ms, _ = hip_time_ms(cycling(make, by, bio.log_softmax), max(steps // 4, 3), warmup, settle_ms)
         rows.append((f"log_softmax rows={r} vocab=151936 (8 B/elem)", ms * 1e3, 0.0, by / ms / 1e6))
+    for r in (256, 4096):
+        by = r * 151936 * 4
+        make = lambda r=r: (torch.randn((r, 151936), device=dev).to(torch.bfloat16),)  # noqa: E731
+        ms, _ = hip_time_ms(cycling(make, by, bio.log_softmax), max(steps // 4, 3), warmup, settle_ms)
+        rows.append((f"log_softmax bf16 in/out rows={r} vocab=151936 (4 B/elem)", ms * 1e3, 0.0, by / ms / 1e6))
     for r in (1, 7, 256, 4096):
         by = r * 4096 * 4
         make = lambda r=r: (torch.randn((r, 4096), device=dev),)  # noqa: E731
-        ms, _ = hip_time_ms(cycling(make, 2 * by, lambda x: bio.mean_dim(x, -1)), steps, warmup)
+        ms, _ = hip_time_ms(cycling(make, 2 * by, lambda x: bio.mean_dim(x, -1)), steps, warmup, settle_ms)
         rows.append((f"mean rows={r} n=4096", ms * 1e3, 0.0, by / ms / 1e6))
     from llm_reproducibility_amd import ops
     for r in (1, 256, 4096):
         by = r * 12288 * 6
         make = lambda r=r: (torch.randn((r, 2 * 12288), device=dev).to(torch.bfloat16),)  # noqa: E731
-        ms, _ = hip_time_ms(cycling(make, by, ops.bi_silu_mul), steps, warmup)
+        ms, _ = hip_time_ms(cycling(make, by, ops.bi_silu_mul), steps, warmup, settle_ms)
         rows.append((f"silu_mul rows={r} inter=12288 (6 B/elem)", ms * 1e3, 0.0, by / ms / 1e6))
     # fixed-order attention (Qwen3-8B heads: 32 query, 8 key/value, head_dim 128)
     Hq, Hkv, D = 32, 8, 128
@@ -228,7 +234,7 @@ def table(steps, warmup, hot=False):
                     torch.randn((B, Hkv, L, D), device=dev).to(torch.bfloat16),
                     torch.randn((B, Hkv, D, L), device=dev).to(torch.bfloat16))
         ms, _ = hip_time_ms(cycling(make, byts, lambda q, kc, vt: ops.bi_attention_bf16(q, kc, vt, qs, ql, cl, qlen, D ** -0.5)),
-                            max(steps // 2, 3), warmup)
+                            max(steps // 2, 3), warmup, settle_ms)
         rows.append((f"attention {name}", ms * 1e3, 4.0 * pairs * D / ms / 1e9, byts / ms / 1e6))
     print("inputs " + ("reused by every call (hot in the memory-side cache)" if hot else
                        "cycled through more than 768 MB of distinct buffers (cold in the 256 MB memory-side cache)"), file=sys.stderr)
@@ -335,7 +341,7 @@ def main():
         context["ceiling"] = ceiling(args.settle_ms)
     out["context"] = context
     if args.table:
-        table(max(args.steps // 2, 5), max(args.warmup // 2, 2), hot=args.table_hot)
+        table(max(args.steps // 2, 5), max(args.warmup // 2, 2), hot=args.table_hot, settle_ms=min(args.settle_ms, 20.0))
     print(json.dumps(out))
 
 
