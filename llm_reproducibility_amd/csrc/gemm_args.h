@@ -20,6 +20,9 @@ struct WideArgs {
 };
 size_t wide_workspace_bytes(int M, int N, int lb, int split);
 int gemm_tree_wide_launch(const WideArgs& a, int leaf_k, int split, hipStream_t stream);
+// gemm_tree_wide_deep.hip: the same tile and bits for leaves of 256 with two binary levels in registers (a.lb >= 2 uses
+// both); takes the same arguments and at most the workspace that wide_workspace_bytes() reports
+int gemm_tree_deep_launch(const WideArgs& a, int split, hipStream_t stream);
 
 // gemm_single_acc_quad.hip: single-accumulator bf16 GEMM, one wave per SIMD
 struct QuadArgs {

@@ -561,7 +561,10 @@ int gemm_dispatch(bool tree, bool f16, const void* A, int64_t lda, const void* B
   } else if (pl.wide) {
     WideArgs w{a.X, a.W, a.C, a.bias, reinterpret_cast<u32x4*>(wsb + pl.partial_bytes), a.ldx, a.ldw, a.ldc, M, N, a.K,
                a.T, a.flb, a.lb, a.vec_store, a.k_shard, a.c_shard};
-    rc = gemm_tree_wide_launch(w, leaf_k, pl.split, stream);
+    // deep trees (four or more binary levels per shard) go to the kernel that keeps two of them in registers: it
+    // parks and re-reads less than half as often; on shallower trees its branchy loop body loses a few percent
+    rc = (leaf_k == 256 && a.lb >= 4) ? gemm_tree_deep_launch(w, pl.split, stream)
+                                      : gemm_tree_wide_launch(w, leaf_k, pl.split, stream);
   } else {
     if (f16) rc = leaf_k == 256 ? launch_tree<4, true>(a, pl.split, stream) : launch_tree<2, true>(a, pl.split, stream);
     else rc = leaf_k == 256 ? launch_tree<4, false>(a, pl.split, stream) : launch_tree<2, false>(a, pl.split, stream);

@@ -1,0 +1,28 @@
+// Inline-asm memory operations shared by the 128x256-tile GEMM kernels: the direct global->LDS load and a store with a
+// wave-uniform base.  The compiler cannot see inside an asm statement, so each statement carries its own wait states.
+#pragma once
+#include "common.h"
+
+namespace tbik {
+
+// One 16-byte-per-lane direct global->LDS load: lane l's 16 bytes land at lds_addr + 16*l.
+// The compiler cannot see inside the statement, so the statement carries its own wait states: a vector-memory
+// instruction must not read a scalar register less than five states after a vector instruction wrote it (which is
+// how a spilled scalar comes back: v_readlane_b32), and the load must not follow the write of m0 directly.  m0 is
+// declared clobbered so that the compiler never keeps a value of its own there.
+__device__ __forceinline__ void dma16(uint32_t lds_addr, uint32_t voff, const void* base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(base)
+               : "memory", "m0");
+}
+
+// 16-byte-per-lane store to (wave-uniform base) + voff, scalar-base addressing: no per-lane 64-bit pointer.
+__device__ __forceinline__ void store16_sbase(void* base, uint32_t voff, u32x4 v) {
+  // the wait states behind the store keep the next instruction from overwriting the data registers while the store
+  // still reads them, the ones in front of it cover a scalar base that a vector instruction has just written
+  // (hazards the compiler handles for its own instructions, but cannot see inside an asm statement)
+  asm volatile("s_nop 4\n\tglobal_store_dwordx4 %0, %1, %2\n\ts_nop 1" : : "v"(voff), "v"(v), "s"(base) : "memory");
+}
+
+}  // namespace tbik
