@@ -415,6 +415,14 @@ struct Plan {
   size_t partial_bytes, parked_bytes;
 };
 
+// Which of the two 128x256-tile kernels runs a shard whose tree has groups of `flb` leaves and `lb` binary levels.  The
+// kernel that keeps two binary levels in registers parks and re-reads a level less than half as often, which pays when
+// levels are parked often: groups of two leaves from two levels on (13 % at K = 8192), any tree from four levels on;
+// on the other trees its branchy loop body loses about 3 %.
+static bool wide_uses_deep_kernel(int leaf_k, int flb, int lb) {
+  return leaf_k == 256 && (lb >= 4 || (flb == 2 && lb >= 2));
+}
+
 static bool make_plan(int M, int N, int K, int leaf_k, bool f16, Plan* pl, bool rowmajor_b = false) {
   int T, flb, level_k;
   if (M <= 0 || N <= 0 || tbik_tree_params(K, leaf_k, &T, &flb, &level_k) != TBIK_OK) return false;
@@ -423,15 +431,18 @@ static bool make_plan(int M, int N, int K, int leaf_k, bool f16, Plan* pl, bool 
   const int64_t wide_tiles = (int64_t)((M + 127) / 128) * ((N + 255) / 256);
   int split = 1;
   bool wide = false;
-  if (M >= 64 && !f16 && !rowmajor_b) {  // the wide kernel exists for bf16 and [N,K] weights only
-    // Estimated time of the wide kernel for each legal split: work-group rounds on 256 CUs times the K extent of
-    // one shard, plus the shard-combine pass over (split + 1) [M,N] arrays.  Constants are measured on MI355X
-    // (17 ns per k per round; 5 TB/s and 4 us for the combine).
+  if (M >= 64 && !f16 && !rowmajor_b) {  // the wide kernels exist for bf16 and [N,K] weights only
+    // Estimated time of the 128x256-tile kernels for each legal split: rounds of work-groups on 256 CUs, each round a
+    // fixed part (pipeline fill, last merges, store) plus the K extent of one shard at the rate of the kernel that
+    // shard would run on, plus the shard-combine pass over (split + 1) [M,N] arrays.  Constants measured on MI355X:
+    // 5.5 us per round; 16.5 ns per k (15.0 on the kernel for deep trees); 5 TB/s and 4 us for the combine.
     double best = 0;
-    for (int sp = 1; sp <= max_split; sp *= 2) {
+    int ls = 0;
+    for (int sp = 1; sp <= max_split; sp *= 2, ls++) {
       if (sp > 8 && wide_tiles * sp > 256) break;  // finer cuts only while the whole grid still runs as one round
       const double rounds = (double)((wide_tiles * sp + 255) / 256);
-      double t = rounds * ((double)K / sp) * 0.0173;
+      const double ns_per_k = wide_uses_deep_kernel(leaf_k, flb, lb - ls) ? 0.0150 : 0.0165;
+      double t = rounds * (5.5 + ((double)K / sp) * ns_per_k);
       if (sp > 1) t += 4.0 + (double)(sp + 1) * M * N * 2.0 / 5.0e6;
       if (sp == 1 || t < best) {
         best = t;
@@ -561,10 +572,8 @@ int gemm_dispatch(bool tree, bool f16, const void* A, int64_t lda, const void* B
   } else if (pl.wide) {
     WideArgs w{a.X, a.W, a.C, a.bias, reinterpret_cast<u32x4*>(wsb + pl.partial_bytes), a.ldx, a.ldw, a.ldc, M, N, a.K,
                a.T, a.flb, a.lb, a.vec_store, a.k_shard, a.c_shard};
-    // deep trees (four or more binary levels per shard) go to the kernel that keeps two of them in registers: it
-    // parks and re-reads less than half as often; on shallower trees its branchy loop body loses a few percent
-    rc = (leaf_k == 256 && a.lb >= 4) ? gemm_tree_deep_launch(w, pl.split, stream)
-                                      : gemm_tree_wide_launch(w, leaf_k, pl.split, stream);
+    rc = wide_uses_deep_kernel(leaf_k, a.flb, a.lb) ? gemm_tree_deep_launch(w, pl.split, stream)
+                                                    : gemm_tree_wide_launch(w, leaf_k, pl.split, stream);
   } else {
     if (f16) rc = leaf_k == 256 ? launch_tree<4, true>(a, pl.split, stream) : launch_tree<2, true>(a, pl.split, stream);
     else rc = leaf_k == 256 ? launch_tree<4, false>(a, pl.split, stream) : launch_tree<2, false>(a, pl.split, stream);

@@ -79,6 +79,27 @@ def test_integer_inputs_match_oracle_bitwise(dev, M, N, K, leaf):
     assert_bitwise(got, want, f"{M}x{N}x{K}")
 
 
+# (M, N, K, leaf): grids of 128x256 tiles.  Both large-M kernels (one binary level in registers / two, the latter for
+# groups of two leaves from two levels on and for any tree from four levels on), with and without a K split in front,
+# leaves of 256 and 128, ragged tiles in M and N
+LARGE_TILE_SHAPES = [
+    (1000, 4000, 8192, 256), (520, 2100, 12288, 256), (1024, 2048, 6400, 128), (2048, 2048, 2048, 256),
+    (300, 5000, 4096, 256), (640, 1024, 16384, 256),
+]
+
+
+@pytest.mark.parametrize("M,N,K,leaf", LARGE_TILE_SHAPES)
+def test_large_tile_kernels_match_oracle_bitwise(dev, M, N, K, leaf):
+    print("case", M, N, K, leaf, flush=True)
+    A_wide = O.integer_bf16((M, K + 8), -9, 9, 50 + M % 89)
+    A = A_wide[:, 8:]                       # a strided view (row stride K + 8)
+    Wnk = O.integer_bf16((N, K), -7, 7, 60 + N % 97)
+    bias = O.integer_bf16((N,), -300, 300, 6)
+    Ad, Wd = A_wide.to(dev)[:, 8:], Wnk.to(dev)
+    assert_bitwise(matmul_tp_persistent(Ad, Wd.t(), leaf_k=leaf), O.matmul_tree(A, Wnk.t(), leaf=leaf), f"{M}x{N}x{K}")
+    assert_bitwise(matmul_tp_persistent(Ad, Wd.t(), bias.to(dev), leaf_k=leaf), O.matmul_tree(A, Wnk.t(), bias, leaf=leaf), "bias")
+
+
 # (M, N, K, leaf): a few rows (up to 16 when the tree has at most four aligned subtrees) and a grid of 16-column strips that loads every CU alike: the one-launch kernel that
 # cuts K over the waves of a work-group (2/4/8 waves, FLB in {1,2,3,5,25}, up to three binary levels inside a wave,
 # a ragged last strip)
