@@ -22,7 +22,7 @@ if ROOT not in sys.path:
 M_, K_, N_ = 2048, 12288, 4096
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
-TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "gemm_tree_wide_headline_counters.txt")
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "gemm_tree_deep_headline_counters.txt")
 
 
 def traffic_from_profile():
@@ -320,7 +320,7 @@ def main():
         "algorithmic_GBps": round(algo_bytes / (ms * 1e-3) / 1e9, 1),
         "roofline": {"bound": "mfma", "achieved": round(tflops, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(tflops / PEAK_BF16_TFLOPS, 4), "traffic": traffic_from_profile(),
-                     "traffic_source": "profiles/gemm_tree_wide_headline_counters.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
+                     "traffic_source": "profiles/gemm_tree_deep_headline_counters.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
                                        "scaled by a copy of known size; a figure of that profile, not of this run)",
                      "kernel_avg_us": round(ms * 1e3, 2)},
     }
@@ -337,6 +337,11 @@ def main():
     lib_ms, _ = hip_time_ms(lambda: torch.matmul(X, Wt), args.steps, args.warmup, args.settle_ms)
     context["vendor_gemm_same_operands_TFLOPs"] = round(flops / (lib_ms * 1e-3) / 1e12, 2)
     context["note"] = "torch.matmul (vendor library), reduction order not fixed, no tree"
+    # this library's own matmul without the tree (one fp32 accumulator over all of K, the batch-invariant mm) on the
+    # same operands: the same tile, ring and MFMA chain, so the difference to `value` is what the tree order costs
+    from llm_reproducibility_amd.bio import batch_invariant_ops as bio
+    mm_ms, _ = hip_time_ms(lambda: bio.matmul_persistent(X, Wt), args.steps, args.warmup, args.settle_ms)
+    context["single_accumulator_mm_same_operands_TFLOPs"] = round(flops / (mm_ms * 1e-3) / 1e12, 2)
     if args.ceiling:
         context["ceiling"] = ceiling(args.settle_ms)
     out["context"] = context

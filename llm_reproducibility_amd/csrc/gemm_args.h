@@ -18,10 +18,12 @@ struct WideArgs {
   int vec_store;
   int64_t k_shard, c_shard;  // K split over gridDim.y shards: operand column offset and partial-output offset per shard
 };
-size_t wide_workspace_bytes(int M, int N, int lb, int split);
+// bytes of parked tree levels: one slab of 16 B per lane per level beyond those the kernel keeps in registers (1 for
+// gemm_tree_wide.hip, 2 for gemm_tree_wide_deep.hip; both kernels use the same tile grid and the same slab layout)
+size_t wide_workspace_bytes(int M, int N, int lb, int split, int levels_in_registers);
 int gemm_tree_wide_launch(const WideArgs& a, int leaf_k, int split, hipStream_t stream);
 // gemm_tree_wide_deep.hip: the same tile and bits for leaves of 256 with two binary levels in registers (a.lb >= 2 uses
-// both); takes the same arguments and at most the workspace that wide_workspace_bytes() reports
+// both); takes the same arguments
 int gemm_tree_deep_launch(const WideArgs& a, int split, hipStream_t stream);
 
 // gemm_single_acc_quad.hip: single-accumulator bf16 GEMM, one wave per SIMD

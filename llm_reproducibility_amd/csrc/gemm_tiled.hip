@@ -466,7 +466,7 @@ static bool make_plan(int M, int N, int K, int leaf_k, bool f16, Plan* pl, bool 
   pl->lb = lb - ls;
   pl->partial_bytes = split > 1 ? (size_t)split * M * N * sizeof(uint16_t) : 0;
   pl->partial_bytes = (pl->partial_bytes + 255) & ~(size_t)255;
-  pl->parked_bytes = wide ? wide_workspace_bytes(M, N, pl->lb, split) : 0;
+  pl->parked_bytes = wide ? wide_workspace_bytes(M, N, pl->lb, split, wide_uses_deep_kernel(leaf_k, flb, pl->lb) ? 2 : 1) : 0;
   return true;
 }
 

@@ -41,11 +41,11 @@ constexpr int MAXLB = 16;
 enum Kind { K_NONE = 0, K_ADD = 1, K_P0 = 2, K_P1 = 3, K_P2 = 4 };
 }  // namespace wide
 
-size_t wide_workspace_bytes(int M, int N, int lb, int split) {
+size_t wide_workspace_bytes(int M, int N, int lb, int split, int levels_in_registers) {
   using namespace wide;
-  if (lb <= RL) return 0;
+  if (lb <= levels_in_registers) return 0;
   const size_t tiles = (size_t)((M + BM - 1) / BM) * ((N + BN - 1) / BN) * (size_t)split;
-  return (size_t)(lb - RL) * tiles * (NT / 64) * 8 * 64 * sizeof(u32x4);
+  return (size_t)(lb - levels_in_registers) * tiles * (NT / 64) * 8 * 64 * sizeof(u32x4);
 }
 
 // TREE = false: the same pipeline with ONE fp32 accumulator run over all of K (the batch-invariant mm); T counts

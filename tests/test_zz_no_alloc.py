@@ -48,11 +48,16 @@ def test_static_scratch_entry_point_matches_the_workspace_entry_point(dev):
     print("case third call 96x5120x6400 leaf 128", flush=True)
     got3, want3, _, _, _ = _both(L, dev, 96, 5120, 6400, 128, 9, True)
     assert torch.equal(got3.view(torch.int16), want3.view(torch.int16))
+    # the headline shape parks two tree levels of 16 MiB each: exactly the size of the array
+    print("case fourth call 2048x4096x12288 (fills the scratch array to the last byte)", flush=True)
+    got4, want4, nws4, _, _ = _both(L, dev, 2048, 4096, 12288, 256, 13, False)
+    assert nws4 == _lib.STATIC_SCRATCH_BYTES
+    assert torch.equal(got4.view(torch.int16), want4.view(torch.int16))
 
 
 def test_static_scratch_entry_point_rejects_what_does_not_fit(dev):
     L = _lib.lib()
-    M, N, K = 2048, 4096, 12288
+    M, N, K = 4096, 5120, 8192
     assert L.tbik_gemm_workspace_bytes(M, N, K, 256) > _lib.STATIC_SCRATCH_BYTES
     C = torch.full((8,), 3.0, device=dev, dtype=torch.bfloat16)                 # never written: the call must not launch
     A = torch.zeros((8,), device=dev, dtype=torch.bfloat16)
