@@ -5,7 +5,7 @@
 
 namespace tbik {
 
-// gemm_tree_wide.hip: tree-ordered bf16 GEMM, 128x256 tiles
+// gemm_tree_wide.hip: tree-ordered bf16 / fp16 GEMM, 128x256 tiles
 struct WideArgs {
   const uint16_t* X;   // [M,K], row stride ldx
   const uint16_t* W;   // [N,K], row stride ldw
@@ -21,7 +21,7 @@ struct WideArgs {
 // bytes of parked tree levels: one slab of 16 B per lane per level beyond those the kernel keeps in registers (1 for
 // gemm_tree_wide.hip, 2 for gemm_tree_wide_deep.hip; both kernels use the same tile grid and the same slab layout)
 size_t wide_workspace_bytes(int M, int N, int lb, int split, int levels_in_registers);
-int gemm_tree_wide_launch(const WideArgs& a, int leaf_k, int split, hipStream_t stream);
+int gemm_tree_wide_launch(const WideArgs& a, int leaf_k, bool f16, int split, hipStream_t stream);
 // gemm_tree_wide_deep.hip: the same tile and bits for leaves of 256 with two binary levels in registers (a.lb >= 2 uses
 // both); takes the same arguments
 int gemm_tree_deep_launch(const WideArgs& a, int split, hipStream_t stream);

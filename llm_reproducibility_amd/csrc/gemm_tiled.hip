@@ -418,9 +418,10 @@ struct Plan {
 // Which of the two 128x256-tile kernels runs a shard whose tree has groups of `flb` leaves and `lb` binary levels.  The
 // kernel that keeps two binary levels in registers parks and re-reads a level less than half as often, which pays when
 // levels are parked often: groups of two leaves from two levels on (13 % at K = 8192), any tree from four levels on;
-// on the other trees its branchy loop body loses about 3 %.
-static bool wide_uses_deep_kernel(int leaf_k, int flb, int lb) {
-  return leaf_k == 256 && (lb >= 4 || (flb == 2 && lb >= 2));
+// on the other trees its branchy loop body loses about 3 %.  (bf16 only: an fp16 node is a single packed add, so there
+// is little to save.)
+static bool wide_uses_deep_kernel(int leaf_k, bool f16, int flb, int lb) {
+  return leaf_k == 256 && !f16 && (lb >= 4 || (flb == 2 && lb >= 2));
 }
 
 static bool make_plan(int M, int N, int K, int leaf_k, bool f16, Plan* pl, bool rowmajor_b = false) {
@@ -431,7 +432,7 @@ static bool make_plan(int M, int N, int K, int leaf_k, bool f16, Plan* pl, bool 
   const int64_t wide_tiles = (int64_t)((M + 127) / 128) * ((N + 255) / 256);
   int split = 1;
   bool wide = false;
-  if (M >= 64 && !f16 && !rowmajor_b) {  // the wide kernels exist for bf16 and [N,K] weights only
+  if (M >= 64 && !rowmajor_b) {  // the wide kernels exist for [N,K] weights only
     // Estimated time of the 128x256-tile kernels for each legal split: rounds of work-groups on 256 CUs, each round a
     // fixed part (pipeline fill, last merges, store) plus the K extent of one shard at the rate of the kernel that
     // shard would run on, plus the shard-combine pass over (split + 1) [M,N] arrays.  Constants measured on MI355X:
@@ -441,7 +442,7 @@ static bool make_plan(int M, int N, int K, int leaf_k, bool f16, Plan* pl, bool 
     for (int sp = 1; sp <= max_split; sp *= 2, ls++) {
       if (sp > 8 && wide_tiles * sp > 256) break;  // finer cuts only while the whole grid still runs as one round
       const double rounds = (double)((wide_tiles * sp + 255) / 256);
-      const double ns_per_k = wide_uses_deep_kernel(leaf_k, flb, lb - ls) ? 0.0150 : 0.0165;
+      const double ns_per_k = wide_uses_deep_kernel(leaf_k, f16, flb, lb - ls) ? 0.0150 : 0.0165;
       double t = rounds * (5.5 + ((double)K / sp) * ns_per_k);
       if (sp > 1) t += 4.0 + (double)(sp + 1) * M * N * 2.0 / 5.0e6;
       if (sp == 1 || t < best) {
@@ -466,7 +467,7 @@ static bool make_plan(int M, int N, int K, int leaf_k, bool f16, Plan* pl, bool 
   pl->lb = lb - ls;
   pl->partial_bytes = split > 1 ? (size_t)split * M * N * sizeof(uint16_t) : 0;
   pl->partial_bytes = (pl->partial_bytes + 255) & ~(size_t)255;
-  pl->parked_bytes = wide ? wide_workspace_bytes(M, N, pl->lb, split, wide_uses_deep_kernel(leaf_k, flb, pl->lb) ? 2 : 1) : 0;
+  pl->parked_bytes = wide ? wide_workspace_bytes(M, N, pl->lb, split, wide_uses_deep_kernel(leaf_k, f16, flb, pl->lb) ? 2 : 1) : 0;
   return true;
 }
 
@@ -572,8 +573,8 @@ int gemm_dispatch(bool tree, bool f16, const void* A, int64_t lda, const void* B
   } else if (pl.wide) {
     WideArgs w{a.X, a.W, a.C, a.bias, reinterpret_cast<u32x4*>(wsb + pl.partial_bytes), a.ldx, a.ldw, a.ldc, M, N, a.K,
                a.T, a.flb, a.lb, a.vec_store, a.k_shard, a.c_shard};
-    rc = wide_uses_deep_kernel(leaf_k, a.flb, a.lb) ? gemm_tree_deep_launch(w, pl.split, stream)
-                                                    : gemm_tree_wide_launch(w, leaf_k, pl.split, stream);
+    rc = wide_uses_deep_kernel(leaf_k, f16, a.flb, a.lb) ? gemm_tree_deep_launch(w, pl.split, stream)
+                                                         : gemm_tree_wide_launch(w, leaf_k, f16, pl.split, stream);
   } else {
     if (f16) rc = leaf_k == 256 ? launch_tree<4, true>(a, pl.split, stream) : launch_tree<2, true>(a, pl.split, stream);
     else rc = leaf_k == 256 ? launch_tree<4, false>(a, pl.split, stream) : launch_tree<2, false>(a, pl.split, stream);

@@ -48,11 +48,11 @@ size_t wide_workspace_bytes(int M, int N, int lb, int split, int levels_in_regis
   return (size_t)(lb - levels_in_registers) * tiles * (NT / 64) * 8 * 64 * sizeof(u32x4);
 }
 
-// TREE = false: the same pipeline with ONE fp32 accumulator run over all of K (the batch-invariant mm); T counts
-// 256-wide spans of K, nothing is merged, and a bias is added in fp32 before the single rounding.
-template <int LS, bool TREE = true>
+// F16: the operands and the tree nodes are fp16 instead of bf16 (same tile, ring and order; a node is one packed add).
+template <int LS, bool F16 = false>
 __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs p) {
   using namespace wide;
+  using NUM = Num16<F16>;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
   const int tid = threadIdx.x;
@@ -146,8 +146,8 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
         const u32x4 a = *w0, b = *w1;
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-          t[8 * q + e] = add_bf16x2(a[e], t[8 * q + e]);
-          t[8 * q + 4 + e] = add_bf16x2(b[e], t[8 * q + 4 + e]);
+          t[8 * q + e] = NUM::add(a[e], t[8 * q + e]);
+          t[8 * q + 4 + e] = NUM::add(b[e], t[8 * q + 4 + e]);
         }
       } else {
         store16_sbase(ws_base(l, 2 * q), lane16, u32x4{t[8 * q], t[8 * q + 1], t[8 * q + 2], t[8 * q + 3]});
@@ -172,10 +172,8 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
   auto merge_quarter = [&](auto kind_c, int q) __attribute__((always_inline)) {
     constexpr int KIND = decltype(kind_c)::value;
     if (KIND == K_NONE) {
-      if (TREE) {
 #pragma unroll
-        for (int e = 0; e < 8; e++) s0[8 * q + e] = t[8 * q + e];
-      }
+      for (int e = 0; e < 8; e++) s0[8 * q + e] = t[8 * q + e];
       return;
     }
     u32x4 pf[2];
@@ -192,11 +190,11 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
 #pragma unroll
     for (int e = 0; e < 8; e++) {
       const int r = 8 * q + e;
-      const uint32_t l0 = add_bf16x2(s0[r], t[r]);
+      const uint32_t l0 = NUM::add(s0[r], t[r]);
       if (KIND == K_ADD) s0[r] = l0;
       if (KIND == K_P0) sb0[r] = l0;
-      if (KIND == K_P1) t[r] = add_bf16x2(sb0[r], l0);
-      if (KIND == K_P2) t[r] = add_bf16x2(pf[e >> 2][e & 3], add_bf16x2(sb0[r], l0));
+      if (KIND == K_P1) t[r] = NUM::add(sb0[r], l0);
+      if (KIND == K_P2) t[r] = NUM::add(pf[e >> 2][e & 3], NUM::add(sb0[r], l0));
     }
     if (KIND == K_P1) {
       store16_sbase(ws_base(RL, 2 * q), lane16, u32x4{t[8 * q], t[8 * q + 1], t[8 * q + 2], t[8 * q + 3]});
@@ -216,8 +214,8 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
   auto pack_row = [&](int a) __attribute__((always_inline)) {
 #pragma unroll
     for (int b = 0; b < TN; b++) {
-      t[(a * TN + b) * 2] = pack_bf16x2(acc[a][b][0], acc[a][b][1]);
-      t[(a * TN + b) * 2 + 1] = pack_bf16x2(acc[a][b][2], acc[a][b][3]);
+      t[(a * TN + b) * 2] = NUM::pack(acc[a][b][0], acc[a][b][1]);
+      t[(a * TN + b) * 2 + 1] = NUM::pack(acc[a][b][2], acc[a][b][3]);
     }
   };
   // One leaf: LS slices of MFMAs, with the pending leaf merged a quarter (LS=4) or a half (LS=2) per slice.
@@ -251,12 +249,12 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
 #pragma unroll
           for (int b = 0; b < TN; b++) {
             const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-            acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[b], fx[a], (i == 0 && kk == 0 && (TREE || j == 0)) ? zero : acc[a][b], 0, 0, 0);
+            acc[a][b] = NUM::mfma(fw[b], fx[a], (i == 0 && kk == 0) ? zero : acc[a][b]);
           }
           // The finished leaf is rounded to bf16 (into the pending buffer) one MFMA row behind the row that
           // completes it, so the rounding never waits for the MFMA pipeline; rows whose pending registers are
           // merged only at the end of this slice follow after that merge.
-          if (TREE && i == LS - 1 && kk == 1 && a >= 1 && a - 1 < EARLY_ROWS) pack_row(a - 1);
+          if (i == LS - 1 && kk == 1 && a >= 1 && a - 1 < EARLY_ROWS) pack_row(a - 1);
           const int d = kk * TM + a;  // 0..7: loads 0..5 go out after MFMA rows 0..5
           if (d < NDMA) {
             __builtin_amdgcn_sched_barrier(0);
@@ -267,7 +265,7 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
       }
 #pragma unroll
       for (int q = i * (4 / LS); q < (i + 1) * (4 / LS); q++) merge_quarter(kind_c, q);
-      if (TREE && i == LS - 1) {
+      if (i == LS - 1) {
 #pragma unroll
         for (int a = EARLY_ROWS; a < TM; a++) pack_row(a);
       }
@@ -277,10 +275,6 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
 
   int kind = K_NONE;
   for (int j = 0; j < p.T; j++) {
-    if (!TREE) {
-      leaf_body(std::integral_constant<int, K_NONE>{}, j);
-      continue;
-    }
     switch (kind) {
       case K_NONE: leaf_body(std::integral_constant<int, K_NONE>{}, j); break;
       case K_ADD: leaf_body(std::integral_constant<int, K_ADD>{}, j); break;
@@ -307,15 +301,15 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
   }
 
   // ---- the last leaf: every level carries, t ends as the root
-  if (TREE && c0 != 0) {
+  if (c0 != 0) {
 #pragma unroll
-    for (int r = 0; r < NREG; r++) t[r] = add_bf16x2(s0[r], t[r]);
+    for (int r = 0; r < NREG; r++) t[r] = NUM::add(s0[r], t[r]);
   }
-  if (TREE && p.lb > 0) {
+  if (p.lb > 0) {
 #pragma unroll
-    for (int r = 0; r < NREG; r++) t[r] = add_bf16x2(sb0[r], t[r]);
+    for (int r = 0; r < NREG; r++) t[r] = NUM::add(sb0[r], t[r]);
   }
-  if (TREE && p.lb > RL) {
+  if (p.lb > RL) {
 #pragma unroll
     for (int q = 0; q < 4; q++) chain_parked(q, RL, g);
   }
@@ -332,19 +326,12 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
       if (p.bias) {
 #pragma unroll
         for (int e = 0; e < 4; e++)
-          if (n + e < p.N) bv[e] = bf16_bits_to_f32(p.bias[n + e]);
+          if (n + e < p.N) bv[e] = NUM::to_f32(p.bias[n + e]);
       }
-      uint32_t lo, hi;
-      if (TREE) {
-        lo = t[(a * TN + b) * 2];
-        hi = t[(a * TN + b) * 2 + 1];
-        if (p.bias) {
-          lo = add_bf16x2(lo, pack_bf16x2(bv[0], bv[1]));
-          hi = add_bf16x2(hi, pack_bf16x2(bv[2], bv[3]));
-        }
-      } else {
-        lo = pack_bf16x2(acc[a][b][0] + bv[0], acc[a][b][1] + bv[1]);
-        hi = pack_bf16x2(acc[a][b][2] + bv[2], acc[a][b][3] + bv[3]);
+      uint32_t lo = t[(a * TN + b) * 2], hi = t[(a * TN + b) * 2 + 1];
+      if (p.bias) {
+        lo = NUM::add(lo, NUM::pack(bv[0], bv[1]));
+        hi = NUM::add(hi, NUM::pack(bv[2], bv[3]));
       }
       uint16_t* dst = p.C + shard * p.c_shard + (int64_t)m * p.ldc + n;
       if (p.vec_store && n + 3 < p.N) {
@@ -359,34 +346,26 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
   }
 }
 
-int gemm_tree_wide_launch(const WideArgs& a, int leaf_k, int split, hipStream_t stream) {
+template <int LS, bool F16>
+static int wide_launch(const WideArgs& a, unsigned tiles, int split, hipStream_t stream) {
   using namespace wide;
   constexpr size_t smem = (size_t)NSLOT * STAGE_BYTES + 16384;  // 144 KiB ring + 16 KiB staging
+  auto kern = gemm_tree_wide_kernel<LS, F16>;
+  static std::atomic<uint64_t> done{0};
+  hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), (int)smem, done);
+  if (e != hipSuccess) return hip_code(e);
+  hipLaunchKernelGGL(kern, dim3(tiles, (unsigned)split), dim3(NT), smem, stream, a);
+  return hip_code(hipGetLastError());
+}
+
+int gemm_tree_wide_launch(const WideArgs& a, int leaf_k, bool f16, int split, hipStream_t stream) {
+  using namespace wide;
   const int64_t tiles = (int64_t)((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
   if (tiles <= 0 || tiles > 0x7fffffff || a.lb > MAXLB) return TBIK_ERR_UNSUPPORTED;
   if (a.ldx >= (1 << 22) || a.ldw >= (1 << 22)) return TBIK_ERR_UNSUPPORTED;  // 32-bit in-tile byte offsets
-  if (leaf_k == 256) {
-    auto kern = gemm_tree_wide_kernel<4>;
-    static std::atomic<uint64_t> done{0};
-    hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), (int)smem, done);
-    if (e != hipSuccess) return hip_code(e);
-    hipLaunchKernelGGL(kern, dim3((unsigned)tiles, (unsigned)split), dim3(NT), smem, stream, a);
-  } else if (leaf_k == 0) {  // single accumulator over K (a multiple of 256)
-    auto kern = gemm_tree_wide_kernel<4, false>;
-    static std::atomic<uint64_t> done{0};
-    hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), (int)smem, done);
-    if (e != hipSuccess) return hip_code(e);
-    hipLaunchKernelGGL(kern, dim3((unsigned)tiles, 1u), dim3(NT), smem, stream, a);
-  } else if (leaf_k == 128) {
-    auto kern = gemm_tree_wide_kernel<2>;
-    static std::atomic<uint64_t> done{0};
-    hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), (int)smem, done);
-    if (e != hipSuccess) return hip_code(e);
-    hipLaunchKernelGGL(kern, dim3((unsigned)tiles, (unsigned)split), dim3(NT), smem, stream, a);
-  } else {
-    return TBIK_ERR_UNSUPPORTED;
-  }
-  return hip_code(hipGetLastError());
+  if (leaf_k == 256) return f16 ? wide_launch<4, true>(a, (unsigned)tiles, split, stream) : wide_launch<4, false>(a, (unsigned)tiles, split, stream);
+  if (leaf_k == 128) return f16 ? wide_launch<2, true>(a, (unsigned)tiles, split, stream) : wide_launch<2, false>(a, (unsigned)tiles, split, stream);
+  return TBIK_ERR_UNSUPPORTED;
 }
 
 }  // namespace tbik

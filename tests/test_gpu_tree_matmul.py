@@ -98,6 +98,9 @@ def test_large_tile_kernels_match_oracle_bitwise(dev, M, N, K, leaf):
     Ad, Wd = A_wide.to(dev)[:, 8:], Wnk.to(dev)
     assert_bitwise(matmul_tp_persistent(Ad, Wd.t(), leaf_k=leaf), O.matmul_tree(A, Wnk.t(), leaf=leaf), f"{M}x{N}x{K}")
     assert_bitwise(matmul_tp_persistent(Ad, Wd.t(), bias.to(dev), leaf_k=leaf), O.matmul_tree(A, Wnk.t(), bias, leaf=leaf), "bias")
+    # fp16 operands on the same grids (the first of the two kernels, instantiated for fp16)
+    h = matmul_tp_persistent(Ad.to(torch.float16), Wd.to(torch.float16).t(), bias.to(dev).to(torch.float16), leaf_k=leaf)
+    assert_bitwise(h, O.matmul_tree(A.to(torch.float16), Wnk.to(torch.float16).t(), bias.to(torch.float16), leaf=leaf), "fp16")
 
 
 # (M, N, K, leaf): a few rows (up to 16 when the tree has at most four aligned subtrees) and a grid of 16-column strips that loads every CU alike: the one-launch kernel that
