@@ -103,6 +103,32 @@ def test_large_tile_kernels_match_oracle_bitwise(dev, M, N, K, leaf):
     assert_bitwise(h, O.matmul_tree(A.to(torch.float16), Wnk.to(torch.float16).t(), bias.to(torch.float16), leaf=leaf), "fp16")
 
 
+def test_large_tile_kernels_seeded_sweep_of_random_shapes(dev):
+    """Random grids of 128x256 tiles (64 or more rows, ragged edges, trees of every depth and group size the leaf count
+    allows, leaves of 128 and 256, bf16 and fp16, with and without bias): bit-exact against the oracle on integer inputs."""
+    import random
+    rng = random.Random(2024)
+    for it in range(14):
+        leaf = rng.choice([256, 256, 256, 128])
+        T = rng.choice([2, 3, 4, 6, 8, 12, 16, 20, 24, 32, 40, 48, 64, 96])
+        M = rng.choice([64, 100, 128, 200, 333, 512, 777, 1024, 1500])
+        N = rng.choice([256, 520, 1000, 1536, 2048, 3000, 4096, 5120])
+        K = leaf * T
+        if M * N * K > 1.2e11:
+            N = 1024
+        f16 = rng.random() < 0.3
+        use_bias = rng.random() < 0.5
+        print("case", it, M, N, K, leaf, "fp16" if f16 else "bf16", "bias" if use_bias else "", flush=True)
+        A = O.integer_bf16((M, K), -9, 9, 100 + it)
+        Wnk = O.integer_bf16((N, K), -3, 3, 200 + it)
+        bias = O.integer_bf16((N,), -64, 64, 300 + it) if use_bias else None
+        if f16:
+            A, Wnk, bias = A.to(torch.float16), Wnk.to(torch.float16), (bias.to(torch.float16) if use_bias else None)
+        want = O.matmul_tree(A, Wnk.t(), bias, leaf=leaf)
+        got = matmul_tp_persistent(A.to(dev), Wnk.to(dev).t(), bias.to(dev) if use_bias else None, leaf_k=leaf)
+        assert_bitwise(got, want, f"case {it}: {M}x{N}x{K} leaf {leaf}")
+
+
 # (M, N, K, leaf): a few rows (up to 16 when the tree has at most four aligned subtrees) and a grid of 16-column strips that loads every CU alike: the one-launch kernel that
 # cuts K over the waves of a work-group (2/4/8 waves, FLB in {1,2,3,5,25}, up to three binary levels inside a wave,
 # a ragged last strip)
