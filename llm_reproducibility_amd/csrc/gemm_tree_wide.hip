@@ -1,5 +1,6 @@
-// Tree-ordered bf16 GEMM for gfx950, large-M path: 128x256 output tile per work-group, 8 wavefronts
-// (2 per SIMD) of 64x64 each, K streamed through a 3-slot LDS ring in 64-element slices.
+// Tree-ordered bf16 / fp16 GEMM for gfx950, large-M path: 128x256 output tile per work-group, 8 wavefronts
+// (2 per SIMD) of 64x64 each, K streamed through a 3-slot LDS ring in 64-element slices.  Leaves of 256 or 128;
+// trees of leaves of 256 that carry often run on the sibling kernel in gemm_tree_wide_deep.hip (same bits).
 //
 // Same arithmetic contract as gemm_tiled.hip (and therefore the same bits): per leaf a chain of
 // 16x16x32 bf16 MFMAs over k in ascending order into a zeroed fp32 accumulator, one rounding to bf16,
@@ -18,6 +19,8 @@
 //     (which frees it for the next leaf's first MFMA); a quarter of the tiles is merged in each of the
 //     next leaf's K slices.  The leaf body is instantiated once per merge kind so that every slice is
 //     straight-line code and the VALU work can issue in the shadow of the MFMAs.
+// Compiled with -structurizecfg-skip-uniform-regions: the switch between the leaf bodies is wave-uniform; structurized,
+// it becomes a chain of flow blocks whose preambles copy every live array whether or not a body runs.
 #include <type_traits>
 
 #include "common.h"

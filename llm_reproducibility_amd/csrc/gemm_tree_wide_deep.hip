@@ -1,22 +1,21 @@
-// Tree-ordered bf16 GEMM for gfx950, large-M path for deep merge trees (leaf 256, four or more binary levels): the same
-// tile, ring and arithmetic as gemm_tree_wide.hip (128x256 output tile per work-group, 8 wavefronts of 64x64, K streamed
-// through a 3-slot LDS ring in 64-element slices, one chain of 16x16x32 bf16 MFMAs per leaf, one rounding per leaf, every
-// tree node rounded to bf16), so the bits are the same; what differs is where the merge tree lives:
+// Tree-ordered bf16 GEMM for gfx950, large-M path for trees that carry often (leaf 256; four or more binary levels, or
+// two or more when a group has two leaves): the same tile, ring and arithmetic as gemm_tree_wide.hip (128x256 output
+// tile per work-group, 8 wavefronts of 64x64, K streamed through a 3-slot LDS ring in 64-element slices, one chain of
+// 16x16x32 bf16 MFMAs per leaf, one rounding per leaf, every tree node rounded to bf16), so the bits are the same;
+// what differs is where the merge tree lives:
 //   * TWO binary levels stay in registers next to the level-0 running sum (the other kernel keeps one), so a tree of 16
 //     groups parks a level in the workspace 3 times instead of 7 and meets a parked level once instead of 3 times;
 //   * ONE loop body serves every leaf: what happens to the previous leaf (nothing / add to the running sum / one of
 //     the carries) is decided by wave-uniform branches around the merge code of each slice, and a leaf that opens a
 //     group is rounded straight into the running-sum registers.  With a single body the register allocator keeps every
 //     array in place across the loop (no copies at the joins of per-kind bodies), which is what makes room for the
-//     second level inside the 256 registers of a wave; the price is a few scalar branches per slice, so trees with
-//     fewer levels stay on the other kernel.
+//     second level inside the 256 registers of a wave; the price is a few scalar branches per slice, so trees that
+//     carry less often stay on the other kernel.
 // Replaces matmul_kernel_tp_persistent, src/tbik/tree_based_matmul.py:50-187.
 //
 // This file is compiled with -structurizecfg-skip-uniform-regions: the branches in the K loop are wave-uniform, and
 // leaving them unstructured keeps the compiler from turning them into chains of flow blocks with a copy per live
 // register.
-#include <type_traits>
-
 #include "common.h"
 #include "gemm_args.h"
 #include "lds_direct.h"
@@ -153,7 +152,7 @@ __global__ __launch_bounds__(deep::NT) void gemm_tree_deep_kernel(const WideArgs
   int pos = 0, kind = K_NONE, g = 0, g_pending = 0;
 
   // merge of quarter q (MFMA row q of the wave's tile: registers 8q..8q+7 of every level)
-  auto lump_simple = [&](int q) __attribute__((always_inline)) {
+  auto merge_in_registers = [&](int q) __attribute__((always_inline)) {
     if (kind == K_ADD) {
 #pragma unroll
       for (int e = 0; e < 8; e++) s0[8 * q + e] = add_bf16x2(s0[8 * q + e], t[8 * q + e]);
@@ -165,7 +164,7 @@ __global__ __launch_bounds__(deep::NT) void gemm_tree_deep_kernel(const WideArgs
       for (int e = 0; e < 8; e++) sb1[8 * q + e] = add_bf16x2(sb0[8 * q + e], add_bf16x2(s0[8 * q + e], t[8 * q + e]));
     }
   };
-  auto lump_park = [&](int q) __attribute__((always_inline)) {
+  auto merge_through_workspace = [&](int q) __attribute__((always_inline)) {
     // bits 0 and 1 of the group counter are set: t = sb1 + (sb0 + (s0 + t)); bit 2 decides whether that value is
     // parked at level 2 or meets the value parked there (staged in LDS since the start of this slice) and carries on
 #pragma unroll
@@ -246,7 +245,7 @@ __global__ __launch_bounds__(deep::NT) void gemm_tree_deep_kernel(const WideArgs
         // where it covers the latency of those loads
         if (kk == 1 && simple) {
           __builtin_amdgcn_sched_barrier(0);
-          lump_simple(i);
+          merge_in_registers(i);
           __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
@@ -266,7 +265,7 @@ __global__ __launch_bounds__(deep::NT) void gemm_tree_deep_kernel(const WideArgs
           }
         }
       }
-      if (park) lump_park(i);
+      if (park) merge_through_workspace(i);
       if (i == LS - 1) {
         if (park) {
 #pragma unroll
