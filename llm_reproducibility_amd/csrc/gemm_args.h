@@ -38,6 +38,7 @@ struct QuadArgs {
 };
 int gemm_single_acc_quad_launch(const QuadArgs& a, hipStream_t stream);
 int gemm_single_acc_slab_launch(const QuadArgs& a, hipStream_t stream);  // at most 128 rows; TBIK_ERR_UNSUPPORTED: use another kernel
+int gemm_single_acc_balanced_launch(const QuadArgs& a, hipStream_t stream);  // any row count: tile width from a cost model
 
 // gemm_single_acc_stream.hip: single-accumulator 16-bit GEMM for at most 64 rows, weights streamed from global memory
 struct StreamArgs {

@@ -35,9 +35,9 @@ __device__ __forceinline__ void quad_dma16(uint32_t lds_addr, uint32_t voff, con
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(base) : "memory", "m0");
 }
 
-// TN = 8: the 128x256 tile of the large shapes.  TN = 1..4: the same pipeline on 128x32 .. 128x128 tiles for 33..128
-// rows, where the call is one pass over the weights and the tile width is chosen so that every CU gets the same
-// number of work-groups.
+// TN = 8: the 128x256 tile of the large shapes.  TN = 1..4 and 6: the same pipeline on 128x32 .. 128x192 tiles for
+// grids that the wide tile would not spread over the chip: the width is chosen per call so that the CUs get the same
+// number of work-groups (gemm_single_acc_balanced_launch).
 template <int TN>
 __global__ __launch_bounds__(quad::NT) void gemm_single_acc_quad_kernel(const QuadArgs p) {
   using namespace quad;
@@ -116,18 +116,19 @@ __global__ __launch_bounds__(quad::NT) void gemm_single_acc_quad_kernel(const Qu
       // The MFMAs of a k step go out in groups; behind every group follow two fragment reads of the next k step
       // ((s,1) from this slot, or (s+1,0) from the next slot, which the mid-slice barrier has made visible) and one
       // direct load: slice s+3 goes into the slot slice s vacates at the mid-slice barrier (first half of its loads
-      // in the second k step of s, second half in the first k step of s+1).  The 256-wide tile has eight groups of
-      // four MFMAs (half a row of tiles each), the narrow tiles four groups of one row.
-      constexpr int NG = TN == 8 ? 8 : 4;
+      // in the second k step of s, second half in the first k step of s+1).  Tiles wider than 128 columns have eight
+      // groups of half a row of MFMAs each, the narrow tiles four groups of one row.
+      constexpr int NG = TN > 4 ? 8 : 4;
       constexpr int H1 = (NDMA + 1) / 2, H2 = NDMA - H1;
       static_assert(H1 <= NG && TM + TN <= 2 * NG, "schedule does not fit the groups");
 #pragma unroll
       for (int q = 0; q < NG; q++) {
         const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-        if constexpr (TN == 8) {
+        if constexpr (TN > 4) {
+          static_assert(TN % 2 == 0, "tiles wider than 128 columns are issued in half rows");
 #pragma unroll
-          for (int bb = 0; bb < 4; bb++) {
-            const int a = q >> 1, b = (q & 1) * 4 + bb;
+          for (int bb = 0; bb < TN / 2; bb++) {
+            const int a = q >> 1, b = (q & 1) * (TN / 2) + bb;
             acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[kk][b], fx[kk][a], (s == 0 && kk == 0) ? zero : acc[a][b], 0, 0, 0);
           }
         } else {
@@ -228,6 +229,58 @@ int gemm_single_acc_slab_launch(const QuadArgs& a, hipStream_t stream) {
     case 2: return quad_launch<2>(a, stream);
     case 1: return quad_launch<1>(a, stream);
     default: return TBIK_ERR_UNSUPPORTED;
+  }
+}
+
+// More than 128 rows on a grid that 128x256 tiles would not spread over the chip: the tile width is chosen by a small
+// cost model (constants measured on MI355X).  The mm cannot cut K (one accumulator), so a work-group's time is a pass
+// over K at a per-slice rate that grows with the tile width, 0.185 + 0.0665 us per 32 columns, and by up to 16 % with
+// the share of the CUs that are busy (the chip is power-bound); narrow tiles fit two work-groups on a CU, which then
+// both run at 1.7 times the single rate; rounds after the first overlap the one before by about a tenth; and no
+// schedule beats one pass over the weights at 3.5 TB/s.  Every width issues the same MFMA chain per element, so the
+// choice never changes a bit.  Examples (us, before -> after, vendor library GEMM in brackets): qkv [M,4096]x[4096,6144]
+// at M=256 39 -> 24 (37), M=512 54 -> 31 (34); gate_up (N=24576) M=384 101 -> 85 (70); 8192x8192 at M=256 83 -> 42 (68).
+int gemm_single_acc_balanced_launch(const QuadArgs& a, hipStream_t stream) {
+  if (a.M <= 0 || a.N <= 0 || a.K < quad::BK || (a.K % quad::BK) != 0) return TBIK_ERR_UNSUPPORTED;
+  const double nsl = (double)(a.K / quad::BK);
+  const int64_t tm = ((int64_t)a.M + quad::BM - 1) / quad::BM;
+  const double floor_us = (double)a.N * a.K * 2.0 / 3.5e6;
+  static const int widths[6] = {8, 6, 4, 3, 2, 1};
+  int best = 8;
+  double best_t = 0.0;
+  for (int i = 0; i < 6; i++) {
+    const int tn = widths[i];
+    const int64_t tiles = tm * (((int64_t)a.N + 32 * tn - 1) / (32 * tn));
+    const double s0 = 0.185 + 0.0665 * tn;
+    double t;
+    if (tn <= 2) {  // up to two work-groups per CU
+      if (tiles <= 256) {
+        t = 3.0 + nsl * s0 * (1.0 + 0.16 * (double)tiles / 256.0);
+      } else {
+        const double rounds = (double)((tiles + 511) / 512);
+        t = (3.0 + nsl * s0 * 1.7) * (1.0 + 0.9 * (rounds - 1.0));
+      }
+    } else {
+      t = 0.0;
+      int64_t left = tiles;
+      for (int r = 0; left > 0; r++, left -= 256) {
+        const double fill = (double)(left < 256 ? left : 256) / 256.0;
+        t += (r == 0 ? 1.0 : 0.9) * (3.0 + nsl * s0 * (1.0 + 0.16 * fill));
+      }
+    }
+    if (t < floor_us) t = floor_us + 1e-3 * t;  // memory-bound either way: keep the order of the compute estimates
+    if (i == 0 || t < best_t) {
+      best_t = t;
+      best = tn;
+    }
+  }
+  switch (best) {
+    case 8: return quad_launch<8>(a, stream);
+    case 6: return quad_launch<6>(a, stream);
+    case 4: return quad_launch<4>(a, stream);
+    case 3: return quad_launch<3>(a, stream);
+    case 2: return quad_launch<2>(a, stream);
+    default: return quad_launch<1>(a, stream);
   }
 }
 

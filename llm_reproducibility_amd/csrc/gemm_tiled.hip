@@ -524,6 +524,11 @@ int gemm_dispatch(bool tree, bool f16, const void* A, int64_t lda, const void* B
       const int rc = gemm_single_acc_slab_launch(qa, stream);
       if (rc != TBIK_ERR_UNSUPPORTED) return rc;
     }
+    // more rows: the same pipeline with the tile width that spreads the grid over the chip (128x256 on large shapes)
+    if (!f16 && M > 128 && (K & 63) == 0 && lda < (1 << 22) && ldb_n < (1 << 22)) {
+      QuadArgs qa{a.X, a.W, a.C, a.bias, a.ldx, a.ldw, a.ldc, M, N, K, a.vec_store};
+      return gemm_single_acc_balanced_launch(qa, stream);
+    }
     if (!f16 && M > 64 && wide_tiles >= 128 && (K & 63) == 0 && lda < (1 << 22) && ldb_n < (1 << 22)) {
       QuadArgs qa{a.X, a.W, a.C, a.bias, a.ldx, a.ldw, a.ldc, M, N, K, a.vec_store};
       return gemm_single_acc_quad_launch(qa, stream);

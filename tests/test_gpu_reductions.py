@@ -202,6 +202,28 @@ def test_single_accumulator_mm_large_and_small_kernels_agree_bitwise(dev):
     assert torch.equal(bio.matmul_persistent(ai.to(dev), wi.to(dev).t()).cpu(), O.matmul_single_acc(ai, wi.t()))
 
 
+# (M, N, K) -> tile width the cost model picks: 64 / 96 / 192 / 128 / 256 / 32 columns, ragged edges in M and N
+@pytest.mark.parametrize("M,N,K", [(200, 6144, 1024), (500, 6100, 512), (700, 6144, 1024), (384, 8192, 2048), (1100, 8200, 256),
+                                   (130, 40, 512), (257, 24576, 320)])
+def test_single_accumulator_mm_balanced_tiles_match_oracle_bitwise(dev, M, N, K):
+    """More than 128 rows: 128-row tiles whose width is chosen to spread the grid over the chip.  Integer inputs, so the
+    oracle's bits are the only right answer; a row alone (streaming kernel) and inside the batch agree bitwise."""
+    print("case", M, N, K, flush=True)
+    a = O.integer_bf16((M, K), -9, 9, 31)
+    w = O.integer_bf16((N, K), -7, 7, 32)
+    bias = O.integer_bf16((N,), -5, 5, 33)
+    ad, wd, bd = a.to(dev), w.to(dev), bias.to(dev)
+    got = bio.matmul_persistent(ad, wd.t(), bd)
+    assert torch.equal(got.cpu(), O.matmul_single_acc(a, w.t(), bias))
+    assert torch.equal(bio.matmul_persistent(ad[M - 1:M], wd.t(), bd), got[M - 1:M])
+    assert torch.equal(bio.matmul_persistent(ad[:129], wd.t(), bd), got[:129])
+    g = O.gaussian_bf16((M, K), 1.0, 34)
+    gw = O.gaussian_bf16((N, K), 0.05, 35)
+    full = bio.matmul_persistent(g.to(dev), gw.to(dev).t())
+    assert torch.equal(bio.matmul_persistent(g[:64].to(dev), gw.to(dev).t()), full[:64])
+    assert not O.outside_tolerance(full, O.matmul_single_acc(g, gw.t())).any()
+
+
 @pytest.mark.parametrize("M,N,K", [(128, 6144, 4096), (65, 8200, 1024), (33, 24576, 512), (100, 16384, 512), (128, 16400, 256), (40, 12296, 1088)])
 def test_single_accumulator_mm_one_round_tiles_match_oracle_bitwise(dev, M, N, K):
     """33..128 rows on a grid of 128-row tiles that is resident at once (tile widths 32, 64, 96 and 128, ragged last
