@@ -1,0 +1,231 @@
+// Batch-invariant bf16 GEMM (one fp32 accumulator per element, K strictly ascending) for gfx950, path of the shapes
+// with many rounds of tiles: 256x256 output tile per work-group, 4 wavefronts (one per SIMD) of 128x128 each, K
+// streamed in 64-element slices through a ring of ten 16 KiB blocks that fills the 160 KiB of LDS.  Replaces
+// matmul_kernel_persistent, src/bio/batch_invariant_ops.py:42-124, where the 128x256 tile of
+// gemm_single_acc_quad.hip would make six or more rounds; per element it issues the same MFMA chain
+// (v_mfma_f32_16x16x32_bf16 over k ascending into one accumulator) as every other single-accumulator kernel of this
+// library, so the bits are the same and a row never sees M.
+//
+// Why a second tile shape: a 128x128 wave tile needs 16 fragment reads and 8 KiB of direct loads per 64 MFMAs where
+// the 64x128 tile needs 24 and 12 KiB, and a work-group has half the barriers per flop.
+//
+// Ring: a slice of the tile is four blocks of 128 rows x 128 B (X rows of the upper and of the lower pair of waves,
+// W rows of the left and of the right pair); a row is one full cache line, so the direct loads ask the L2 for whole
+// lines (a ring of 32-wide units with 64 B rows doubled the L2 requests and was 8-12 % slower).  Two slices and a
+// half fit: block g of the stream sits at position g mod 10.  All four blocks of slice s are free once every wave
+// has read its fragments of the second k step of s, which the one barrier per slice, between its two k steps,
+// establishes; into them go the W blocks of slice s+2 (issued during the second k step of s) and the X blocks of
+// slice s+3 (issued during the first k step of s+1), so every load has at least the length of one k step to land
+// and half of them a slice and a half.
+//
+// Schedule: fragment reads run one k step ahead of the MFMAs; every non-MFMA instruction sits alone behind one MFMA
+// (a wave issues in order: a cluster of LDS reads and loads behind a row of MFMAs would leave the MFMA pipe idle
+// while it issues).  The 16-byte chunk c of row r sits at position c ^ (r & 7); a lane of a direct load fetches the
+// global chunk that belongs at its linear LDS position, which realises that swizzle on the source side.
+#include "common.h"
+#include "gemm_args.h"
+#include "lds_direct.h"
+
+namespace tbik {
+
+namespace sq {
+constexpr int BM = 256, BN = 256, BK = 64, NT = 256, NWAVE = 4, TM = 8, TN = 8;
+constexpr int BLOCK_ROWS = 128, BLOCK_BYTES = BLOCK_ROWS * BK * 2;  // 16 KiB
+constexpr int NBLOCK = 10;                                         // ring positions: 160 KiB
+constexpr int BDMA = BLOCK_ROWS / 8 / NWAVE;                       // direct loads per wave per block: 4 (8 rows each)
+__device__ __forceinline__ int wrap(int pos) { return pos >= NBLOCK ? pos - NBLOCK : pos; }
+}  // namespace sq
+
+// The 64 accumulator tiles of a wave are 256 registers, the whole accumulation register file.  Left to the compiler, all
+// MFMA accumulators go there and, with nothing to spare, half of them are shuttled through the other file in every trip
+// of the loop (two moves per MFMA).  So the MFMAs are opaque statements that pin their accumulator: seven columns of
+// tiles in accumulation registers, the eighth in ordinary vector registers.  The compiler cannot see the hazards of
+// such a statement: inside the loop an accumulator is touched by nothing but its own MFMA (the next one 64 MFMAs
+// later), the fragment registers are written by LDS reads that the compiler orders itself, and the epilogue waits
+// before anything else reads the results (mfma_results_ready).
+__device__ __forceinline__ void mfma_in_agprs(f32x4& acc, const bf16x8& a, const bf16x8& b) {
+  asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mfma_in_vgprs(f32x4& acc, const bf16x8& a, const bf16x8& b) {
+  asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
+}
+__device__ __forceinline__ void mfma_results_ready() {
+  // an 8-pass MFMA needs up to 18 wait states before another kind of instruction may read its result; the scheduling
+  // fence keeps every later instruction behind the wait
+  asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+}
+
+__global__ __launch_bounds__(sq::NT) void gemm_single_acc_256_kernel(const QuadArgs p) {
+  using namespace sq;
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+
+  const int tiles_m = (p.M + BM - 1) / BM;
+  const int tiles_n = (p.N + BN - 1) / BN;
+  int lid = blockIdx.x;
+  {
+    const int nwg = gridDim.x;
+    if ((nwg & 7) == 0) lid = (lid & 7) * (nwg >> 3) + (lid >> 3);  // consecutive ids share an XCD
+  }
+  constexpr int GROUP = 4;
+  const int per_group = GROUP * tiles_n;
+  const int group_id = lid / per_group;
+  const int first_m = group_id * GROUP;
+  const int gsz = min(tiles_m - first_m, GROUP);
+  const int pid_m = first_m + (lid % per_group) % gsz;
+  const int pid_n = (lid % per_group) / gsz;
+  const int m0 = pid_m * BM, n0 = pid_n * BN;
+
+  const uint8_t* xbase = reinterpret_cast<const uint8_t*>(p.X + (int64_t)m0 * p.ldx);
+  const uint8_t* wbase = reinterpret_cast<const uint8_t*>(p.W + (int64_t)n0 * p.ldw);
+  // byte offsets of this lane's direct loads inside the tile's operands: [half][load]; rows past the edge are clamped
+  uint32_t voffx[2 * BDMA], voffw[2 * BDMA];
+  {
+    const int r = lane >> 3, c = (lane & 7) ^ r;
+#pragma unroll
+    for (int i = 0; i < 2 * BDMA; i++) {
+      const int row = (i / BDMA) * BLOCK_ROWS + ((i % BDMA) * NWAVE + wave) * 8 + r;
+      voffx[i] = (uint32_t)(((min(m0 + row, p.M - 1) - m0) * p.ldx + c * 8) * 2);
+      voffw[i] = (uint32_t)(((min(n0 + row, p.N - 1) - n0) * p.ldw + c * 8) * 2);
+    }
+  }
+  const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
+  const int nslices = p.K / BK;
+  // load i (0..7: half i / 4, rows of load i % 4) of the X or W blocks of slice s into ring position pos of that half;
+  // slices past the end of K load the last one again (never read): the count of loads in flight stays the same
+  auto dma_x = [&](int s, int pos, int i) __attribute__((always_inline)) {
+    dma16(lds0 + pos * BLOCK_BYTES + ((i % BDMA) * NWAVE + wave) * 1024, voffx[i],
+          xbase + (int64_t)min(s, nslices - 1) * (BK * 2));
+  };
+  auto dma_w = [&](int s, int pos, int i) __attribute__((always_inline)) {
+    dma16(lds0 + pos * BLOCK_BYTES + ((i % BDMA) * NWAVE + wave) * 1024, voffw[i],
+          wbase + (int64_t)min(s, nslices - 1) * (BK * 2));
+  };
+  const int frow = lane & 15, fchk = lane >> 4;
+  const uint32_t frag = (frow * BK + ((fchk ^ (frow & 7)) << 3)) * 2;  // inside a block, row a * 16 + frow, k step 0
+
+  f32x4 acc[TM][TN];
+  bf16x8 fx[2][TM], fw[2][TN];
+  auto read_frag = [&](int buf, int xpos, int wpos, int kk, int f) __attribute__((always_inline)) {
+    if (f < TM) fx[buf][f] = *reinterpret_cast<const bf16x8*>(smem + xpos * BLOCK_BYTES + (frag ^ (kk * 64)) + f * 16 * BK * 2);
+    else fw[buf][f - TM] = *reinterpret_cast<const bf16x8*>(smem + wpos * BLOCK_BYTES + (frag ^ (kk * 64)) + (f - TM) * 16 * BK * 2);
+  };
+
+  // prologue: slices 0 and 1 and the X blocks of slice 2 fill the ten positions; slice 0 visible, fragments of its
+  // first k step in registers
+#pragma unroll
+  for (int s = 0; s < 2; s++) {
+#pragma unroll
+    for (int i = 0; i < 2 * BDMA; i++) dma_x(s, 4 * s + i / BDMA, i);
+#pragma unroll
+    for (int i = 0; i < 2 * BDMA; i++) dma_w(s, 4 * s + 2 + i / BDMA, i);
+  }
+#pragma unroll
+  for (int i = 0; i < 2 * BDMA; i++) dma_x(2, 8 + i / BDMA, i);
+#pragma unroll
+  for (int a = 0; a < TM; a++)
+#pragma unroll
+    for (int b = 0; b < TN; b++) {
+      // zero here, long before the first MFMA, and opaque from here on: a zero that the compiler knows to be zero is
+      // written again right in front of the first MFMA, closer than an MFMA may follow a write of its accumulator
+      acc[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (b < TN - 1) asm volatile("" : "+a"(acc[a][b]));
+      else asm volatile("" : "+v"(acc[a][b]));
+    }
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(6 * BDMA) : "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+#pragma unroll
+  for (int f = 0; f < TM + TN; f++) read_frag(0, wm, 2 + wn, 0, f);
+
+  int px = 0;  // ring position of the first block of slice s
+  for (int s = 0; s < nslices; s++) {
+    const int px1 = wrap(px + 4);
+    const int xpos = wrap(px + wm), wpos = wrap(px + 2 + wn);      // this wave's blocks of slice s
+    const int xpos1 = wrap(px1 + wm), wpos1 = wrap(px1 + 2 + wn);  // and of slice s+1
+#pragma unroll
+    for (int kk = 0; kk < 2; kk++) {
+#pragma unroll
+      for (int q = 0; q < TM; q++) {
+#pragma unroll
+        for (int b = 0; b < TN; b++) {
+          if (b < TN - 1) mfma_in_agprs(acc[q][b], fw[kk][b], fx[kk][q]);
+          else mfma_in_vgprs(acc[q][b], fw[kk][b], fx[kk][q]);
+          if (b == 0 || b == 2) {
+            // fragments of the next k step: the second of this slice, or the first of the next slice (behind the
+            // last slice that reads blocks whose loads have landed and are never used)
+            if (kk == 0) read_frag(1, xpos, wpos, 1, 2 * q + (b >> 1));
+            else read_frag(0, xpos1, wpos1, 0, 2 * q + (b >> 1));
+          }
+          if (b == 4) {
+            // first k step: X blocks of slice s+2 into the positions of the W blocks of slice s-1 (the prologue has
+            // issued those of slice 2); second k step: W blocks of slice s+2 into the positions of the X blocks of s
+            if (kk == 0) {
+              if (s > 0) dma_x(s + 2, wrap(px + 8 + q / BDMA), q);
+            } else {
+              dma_w(s + 2, wrap(px + q / BDMA), q);
+            }
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      if (kk == 0) {
+        // between the k steps: slice s+1 has landed (this wave's share: the X loads of s+2 may still fly) and every
+        // fragment read of slice s is done
+        asm volatile("s_waitcnt vmcnt(%0)" : : "n"(2 * BDMA) : "memory");
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+      }
+    }
+    px = px1;
+  }
+
+  mfma_results_ready();
+#pragma unroll
+  for (int a = 0; a < TM; a++) {
+    const int m = m0 + (wm * TM + a) * 16 + frow;
+#pragma unroll
+    for (int b = 0; b < TN; b++) {
+      const int n = n0 + (wn * TN + b) * 16 + fchk * 4;
+      if (m >= p.M || n >= p.N) continue;
+      float bv[4] = {0.f, 0.f, 0.f, 0.f};
+      if (p.bias) {
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+          if (n + e < p.N) bv[e] = bf16_bits_to_f32(p.bias[n + e]);
+      }
+      const uint32_t lo = pack_bf16x2(acc[a][b][0] + bv[0], acc[a][b][1] + bv[1]);
+      const uint32_t hi = pack_bf16x2(acc[a][b][2] + bv[2], acc[a][b][3] + bv[3]);
+      uint16_t* dst = p.C + (int64_t)m * p.ldc + n;
+      if (p.vec_store && n + 3 < p.N) {
+        *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);
+      } else {
+        const uint16_t v[4] = {(uint16_t)(lo & 0xffff), (uint16_t)(lo >> 16), (uint16_t)(hi & 0xffff), (uint16_t)(hi >> 16)};
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+          if (n + e < p.N) dst[e] = v[e];
+      }
+    }
+  }
+  // the direct loads past the end of K have an address in this work-group's LDS: they must land before it is released
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
+int gemm_single_acc_256_launch(const QuadArgs& a, hipStream_t stream) {
+  using namespace sq;
+  constexpr size_t smem = (size_t)NBLOCK * BLOCK_BYTES;  // 160 KiB: all of a CU's LDS
+  const int64_t tiles = (int64_t)((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
+  if (tiles <= 0 || tiles > 0x7fffffff || a.K < BK || (a.K % BK) != 0) return TBIK_ERR_UNSUPPORTED;
+  if (a.ldx >= (1 << 22) || a.ldw >= (1 << 22)) return TBIK_ERR_UNSUPPORTED;  // 32-bit in-tile byte offsets
+  static std::atomic<uint64_t> done{0};
+  hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(gemm_single_acc_256_kernel), (int)smem, done);
+  if (e != hipSuccess) return hip_code(e);
+  hipLaunchKernelGGL(gemm_single_acc_256_kernel, dim3((unsigned)tiles), dim3(NT), smem, stream, a);
+  return hip_code(hipGetLastError());
+}
+
+}  // namespace tbik

@@ -14,6 +14,7 @@
 //     ahead of the MFMAs, also across the barrier; scheduling fences keep that order in the generated code.
 #include "common.h"
 #include "gemm_args.h"
+#include "lds_direct.h"
 
 namespace tbik {
 
@@ -28,12 +29,6 @@ struct Shape {
   static constexpr int NDMA = ROWS / 8 / NWAVE;   // direct loads per wave per slice: 12 for the 256-wide tile
 };
 }  // namespace quad
-
-__device__ __forceinline__ void quad_dma16(uint32_t lds_addr, uint32_t voff, const void* base) {
-  // wait states inside the statement (the compiler cannot see the instructions): five between a vector instruction
-  // that wrote a scalar operand and the load that reads it, one between the write of m0 and the load; m0 is clobbered
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(base) : "memory", "m0");
-}
 
 // TN = 8: the 128x256 tile of the large shapes.  TN = 1..4 and 6: the same pipeline on 128x32 .. 128x192 tiles for
 // grids that the wide tile would not spread over the chip: the width is chosen per call so that the CUs get the same
@@ -79,7 +74,7 @@ __global__ __launch_bounds__(quad::NT) void gemm_single_acc_quad_kernel(const Qu
   const int nstages = p.K / BK;
   auto dma_one = [&](int s, int slot, int i) __attribute__((always_inline)) {
     const uint8_t* b = (i < XDMA ? xbase : wbase) + (int64_t)min(s, nstages - 1) * (BK * 2);
-    quad_dma16(lds0 + slot * STAGE_BYTES + (i * NWAVE + wave) * 1024, voff[i], b);
+    dma16(lds0 + slot * STAGE_BYTES + (i * NWAVE + wave) * 1024, voff[i], b);
   };
   const int frow = lane & 15, fchk = lane >> 4;
   const uint32_t xfrag = ((wm * TM * 16 + frow) * BK + ((fchk ^ (frow & 7)) << 3)) * 2;
@@ -273,6 +268,21 @@ int gemm_single_acc_balanced_launch(const QuadArgs& a, hipStream_t stream) {
       best_t = t;
       best = tn;
     }
+  }
+  // Many rounds of tiles: the 256x256 tile halves the L2 traffic and the LDS reads per flop.  A round of it costs
+  // 6 us + 1.44 us per slice against 3 us + 0.83 us per slice of the 128x256 tile, which makes twice the rounds;
+  // from six rounds on the estimate above (fitted on grids of few rounds) is below what the 128x256 tile sustains,
+  // so the comparison uses its sustained rate there.  gate_up [M,4096]x[4096,24576]: M=2048 366 -> 301 us,
+  // M=8192 1402 -> 1175 (vendor library 272 / 1048); down [M,12288]x[12288,4096] at M=4096 319 -> 274 (259).
+  {
+    const int64_t tiles8 = tm * (((int64_t)a.N + 255) / 256);
+    const int64_t tiles256 = (((int64_t)a.M + 255) / 256) * (((int64_t)a.N + 255) / 256);
+    const double rounds8 = (double)((tiles8 + 255) / 256);
+    double t256 = (double)((tiles256 + 255) / 256) * (6.0 + nsl * 1.44);
+    if (t256 < floor_us) t256 = floor_us + 1e-3 * t256;
+    const double t128 = rounds8 >= 6.0 ? rounds8 * (3.0 + nsl * 0.83) : best_t;
+    if (tiles8 > 256 && t256 < t128)
+      return gemm_single_acc_256_launch(a, stream);
   }
   switch (best) {
     case 8: return quad_launch<8>(a, stream);

@@ -6,13 +6,16 @@
 namespace tbik {
 
 // One 16-byte-per-lane direct global->LDS load: lane l's 16 bytes land at lds_addr + 16*l.
-// The compiler cannot see inside the statement, so the statement carries its own wait states: a vector-memory
-// instruction must not read a scalar register less than five states after a vector instruction wrote it (which is
-// how a spilled scalar comes back: v_readlane_b32), and the load must not follow the write of m0 directly.  m0 is
-// declared clobbered so that the compiler never keeps a value of its own there.
+// The compiler cannot see inside the statement, so the statement takes care of its own hazards without idle wait
+// states: the load must not follow the write of m0 directly, and a vector-memory instruction must not read a scalar
+// register less than five states after a VECTOR instruction wrote it (which is how a spilled scalar comes back:
+// v_readlane_b32).  The scalar copy of the base address between the write of m0 and the load settles both: it is the
+// one state behind m0, and the load then reads a register that a scalar instruction has written.  m0 is declared
+// clobbered so that the compiler never keeps a value of its own there.
 __device__ __forceinline__ void dma16(uint32_t lds_addr, uint32_t voff, const void* base) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %1, %2"
-               :
+  const void* base_copy;
+  asm volatile("s_mov_b32 m0, %1\n\ts_mov_b64 %0, %3\n\tglobal_load_lds_dwordx4 %2, %0"
+               : "=&s"(base_copy)
                : "s"(lds_addr), "v"(voff), "s"(base)
                : "memory", "m0");
 }

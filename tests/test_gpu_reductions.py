@@ -224,6 +224,32 @@ def test_single_accumulator_mm_balanced_tiles_match_oracle_bitwise(dev, M, N, K)
     assert not O.outside_tolerance(full, O.matmul_single_acc(g, gw.t())).any()
 
 
+# grids of many rounds, where the cost model picks the 256x256 tile: one round of 256 tiles with ragged edges in M and N,
+# an odd number of 64-wide slices, five rounds with a last column of tiles eight columns wide
+@pytest.mark.parametrize("M,N,K", [(2040, 8190, 1024), (4096, 4090, 2112), (8192, 8200, 1024), (2048, 8192, 768)])
+def test_single_accumulator_mm_256_tiles_match_oracle_bitwise(dev, M, N, K):
+    """256x256 tiles (accumulators pinned by hand in both register files, ten-block LDS ring): integer inputs, so the
+    oracle's bits are the only right answer; rows alone (streaming kernel), the first 129 rows (128-row tiles) and the
+    whole batch agree bitwise; Gaussian inputs stay inside the tolerance and agree with the 128-row tiles bitwise."""
+    print("case", M, N, K, flush=True)
+    a = O.integer_bf16((M, K), -9, 9, 41)
+    w = O.integer_bf16((N, K), -7, 7, 42)
+    bias = O.integer_bf16((N,), -5, 5, 43)
+    ad, wd, bd = a.to(dev), w.to(dev), bias.to(dev)
+    got = bio.matmul_persistent(ad, wd.t(), bd)
+    assert torch.equal(got.cpu(), O.matmul_single_acc(a, w.t(), bias))
+    assert torch.equal(bio.matmul_persistent(ad[M - 1:M], wd.t(), bd), got[M - 1:M])
+    assert torch.equal(bio.matmul_persistent(ad[:129], wd.t(), bd), got[:129])
+    g = O.gaussian_bf16((M, K), 1.0, 44)
+    gw = O.gaussian_bf16((N, K), 0.05, 45)
+    gd, gwd = g.to(dev), gw.to(dev)
+    full = bio.matmul_persistent(gd, gwd.t())
+    for lo in range(0, M, 640):  # pieces of at most 640 rows take the 128-row tiles: same MFMA chain, same bits
+        assert torch.equal(bio.matmul_persistent(gd[lo:lo + 640], gwd.t()), full[lo:lo + 640]), lo
+    assert not O.outside_tolerance(full[:512], O.matmul_single_acc(g[:512], gw.t())).any()
+    assert torch.equal(bio.matmul_persistent(gd, gwd.t()), full)  # and the same bits on a second launch
+
+
 @pytest.mark.parametrize("M,N,K", [(128, 6144, 4096), (65, 8200, 1024), (33, 24576, 512), (100, 16384, 512), (128, 16400, 256), (40, 12296, 1088)])
 def test_single_accumulator_mm_one_round_tiles_match_oracle_bitwise(dev, M, N, K):
     """33..128 rows on a grid of 128-row tiles that is resident at once (tile widths 32, 64, 96 and 128, ragged last
