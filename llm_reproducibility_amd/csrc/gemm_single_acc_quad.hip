@@ -119,26 +119,30 @@ __global__ __launch_bounds__(quad::NT) void gemm_single_acc_quad_kernel(const Qu
 #pragma unroll
       for (int q = 0; q < NG; q++) {
         const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-        if constexpr (TN > 4) {
-          static_assert(TN % 2 == 0, "tiles wider than 128 columns are issued in half rows");
-#pragma unroll
-          for (int bb = 0; bb < TN / 2; bb++) {
-            const int a = q >> 1, b = (q & 1) * (TN / 2) + bb;
-            acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[kk][b], fx[kk][a], (s == 0 && kk == 0) ? zero : acc[a][b], 0, 0, 0);
-          }
-        } else {
-#pragma unroll
-          for (int b = 0; b < TN; b++)
-            acc[q][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[kk][b], fx[kk][q], (s == 0 && kk == 0) ? zero : acc[q][b], 0, 0, 0);
-        }
         const int rslot = kk == 0 ? slot : nslot;
+        // the group's other instructions, each alone behind one MFMA where the group has enough of them (a wave
+        // issues in order: a cluster of LDS reads and a load behind the group leaves the MFMA pipe idle meanwhile)
+        auto other = [&](int j) __attribute__((always_inline)) {
+          if (j < 2) {
+            const int f = 2 * q + j;
+            if (f < TM) read_x(kk ^ 1, rslot, kk ^ 1, f);
+            else if (f - TM < TN) read_w(kk ^ 1, rslot, kk ^ 1, f - TM);
+          } else {
+            if (kk == 1 && q < H1) dma_one(s + 3, slot, q);
+            if (kk == 0 && q < H2 && s > 0) dma_one(s + 2, pslot, H1 + q);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        };
+        constexpr int GM = TN > 4 ? TN / 2 : TN;  // MFMAs of a group
+        static_assert(TN <= 4 || TN % 2 == 0, "tiles wider than 128 columns are issued in half rows");
 #pragma unroll
-        for (int f = 2 * q; f < 2 * q + 2; f++) {
-          if (f < TM) read_x(kk ^ 1, rslot, kk ^ 1, f);
-          else if (f - TM < TN) read_w(kk ^ 1, rslot, kk ^ 1, f - TM);
+        for (int j = 0; j < GM; j++) {
+          const int a = TN > 4 ? q >> 1 : q, b = TN > 4 ? (q & 1) * (TN / 2) + j : j;
+          acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[kk][b], fx[kk][a], (s == 0 && kk == 0) ? zero : acc[a][b], 0, 0, 0);
+          if (j < 3) other(j);
         }
-        if (kk == 1 && q < H1) dma_one(s + 3, slot, q);
-        if (kk == 0 && q < H2 && s > 0) dma_one(s + 2, pslot, H1 + q);
+#pragma unroll
+        for (int j = GM; j < 3; j++) other(j);
         __builtin_amdgcn_sched_barrier(0);
       }
       if (kk == 0) {
