@@ -177,7 +177,9 @@ def table(steps, warmup, hot=False, settle_ms=20.0):
     library_row(4096, 8192, 5120)
     library_row(4096, 25600, 5120)
     library_row(2048, 4096, 24576)
-    for name, M, K, N in (("qkv 8B", 2048, 4096, 6144), ("gate_up 8B", 2048, 4096, 24576), ("lm_head 8B", 128, 4096, 151936),
+    library_row(8192, 4096, 24576)
+    for name, M, K, N in (("qkv 8B", 2048, 4096, 6144), ("gate_up 8B", 2048, 4096, 24576), ("gate_up 8B", 8192, 4096, 24576),
+                          ("lm_head 8B", 128, 4096, 151936),
                           ("qkv 8B", 1, 4096, 6144), ("qkv 8B", 32, 4096, 6144), ("qkv 8B", 128, 4096, 6144),
                           ("gate_up 8B", 1, 4096, 24576), ("gate_up 8B", 32, 4096, 24576), ("gate_up 8B", 128, 4096, 24576),
                           ("lm_head 8B", 1, 4096, 151936), ("lm_head 8B", 32, 4096, 151936)):
