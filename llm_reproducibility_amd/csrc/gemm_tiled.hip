@@ -22,6 +22,8 @@
 // src/tbik/tree_based_matmul.py:259-264).  It is consumed in place: a thread loads an 8(k) x 8(n) block as eight
 // 16-byte rows, transposes it in registers (v_perm_b32) and writes eight K-contiguous 16-byte chunks into the same
 // LDS tile layout, so fragments, MFMA chain and bits are those of the [N,K] form.
+#include <algorithm>
+
 #include "common.h"
 #include "gemm_args.h"
 
@@ -424,6 +426,58 @@ static bool wide_uses_deep_kernel(int leaf_k, bool f16, int flb, int lb) {
   return leaf_k == 256 && !f16 && (lb >= 4 || (flb == 2 && lb >= 2));
 }
 
+// Estimated time of the 128x256-tile kernels over the legal K splits of one problem, and the best split: rounds of
+// work-groups on 256 CUs, each round a fixed part (pipeline fill, last merges, store) plus the K extent of one shard at
+// the rate of the kernel that shard would run on, plus the shard-combine pass over (split + 1) [M,N] arrays.  Constants
+// measured on MI355X: 5.5 us per round; 16.5 ns per k (15.0 on the kernel for deep trees); 5 TB/s and 4 us for the
+// combine.
+static double wide_cost_us(int M, int N, int K, int leaf_k, bool f16, int flb, int lb, int* best_split) {
+  const int max_split = lb >= 5 ? 32 : (1 << lb);
+  const int64_t wide_tiles = (int64_t)((M + 127) / 128) * ((N + 255) / 256);
+  double best = 0;
+  int split = 1, ls = 0;
+  for (int sp = 1; sp <= max_split; sp *= 2, ls++) {
+    if (sp > 8 && wide_tiles * sp > 256) break;  // finer cuts only while the whole grid still runs as one round
+    const double rounds = (double)((wide_tiles * sp + 255) / 256);
+    const double ns_per_k = wide_uses_deep_kernel(leaf_k, f16, flb, lb - ls) ? 0.0150 : 0.0165;
+    double t = rounds * (5.5 + ((double)K / sp) * ns_per_k);
+    if (sp > 1) t += 4.0 + (double)(sp + 1) * M * N * 2.0 / 5.0e6;
+    if (sp == 1 || t < best) {
+      best = t;
+      split = sp;
+    }
+  }
+  *best_split = split;
+  return best;
+}
+
+// Column regions.  A grid of 128x256 tiles rarely fills whole rounds of 256 work-groups, and one K split serves the
+// whole problem; cut into the columns [0, NA) and [NA, N), each part gets the split that fills ITS rounds (o_proj 32B
+// at M=4096: 512 tiles unsplit = two full rounds, then 128 tiles cut in two = one round of half the length, instead of
+// three rounds: 395 -> 350 us; at M=512: 64 tiles cut in four and 16 tiles cut in sixteen, 74 -> 69 us).  The parts
+// run one after the other as problems of their own, so every element is still computed by the same leaf and shard
+// trees: the bits do not change.  Returns NA (a multiple of 256), or 0 when the whole problem in one piece is
+// estimated within 5 % of the best pair.
+static int column_regions(int M, int N, int K, int leaf_k, bool f16) {
+  int T, flb, level_k;
+  if (M < 64 || N <= 256 || tbik_tree_params(K, leaf_k, &T, &flb, &level_k) != TBIK_OK) return 0;
+  const int tiles_n = (N + 255) / 256;
+  if (tiles_n > 64) return 0;
+  int sp;
+  const double whole = wide_cost_us(M, N, K, leaf_k, f16, flb, level_k - 1, &sp);
+  double best = whole * 0.95;
+  int best_na = 0;
+  for (int na = 1; na < tiles_n; na++) {
+    const double t = wide_cost_us(M, na * 256, K, leaf_k, f16, flb, level_k - 1, &sp) +
+                     wide_cost_us(M, N - na * 256, K, leaf_k, f16, flb, level_k - 1, &sp);
+    if (t < best) {
+      best = t;
+      best_na = na * 256;
+    }
+  }
+  return best_na;
+}
+
 static bool make_plan(int M, int N, int K, int leaf_k, bool f16, Plan* pl, bool rowmajor_b = false) {
   int T, flb, level_k;
   if (M <= 0 || N <= 0 || tbik_tree_params(K, leaf_k, &T, &flb, &level_k) != TBIK_OK) return false;
@@ -433,23 +487,7 @@ static bool make_plan(int M, int N, int K, int leaf_k, bool f16, Plan* pl, bool 
   int split = 1;
   bool wide = false;
   if (M >= 64 && !rowmajor_b) {  // the wide kernels exist for [N,K] weights only
-    // Estimated time of the 128x256-tile kernels for each legal split: rounds of work-groups on 256 CUs, each round a
-    // fixed part (pipeline fill, last merges, store) plus the K extent of one shard at the rate of the kernel that
-    // shard would run on, plus the shard-combine pass over (split + 1) [M,N] arrays.  Constants measured on MI355X:
-    // 5.5 us per round; 16.5 ns per k (15.0 on the kernel for deep trees); 5 TB/s and 4 us for the combine.
-    double best = 0;
-    int ls = 0;
-    for (int sp = 1; sp <= max_split; sp *= 2, ls++) {
-      if (sp > 8 && wide_tiles * sp > 256) break;  // finer cuts only while the whole grid still runs as one round
-      const double rounds = (double)((wide_tiles * sp + 255) / 256);
-      const double ns_per_k = wide_uses_deep_kernel(leaf_k, f16, flb, lb - ls) ? 0.0150 : 0.0165;
-      double t = rounds * (5.5 + ((double)K / sp) * ns_per_k);
-      if (sp > 1) t += 4.0 + (double)(sp + 1) * M * N * 2.0 / 5.0e6;
-      if (sp == 1 || t < best) {
-        best = t;
-        split = sp;
-      }
-    }
+    wide_cost_us(M, N, K, leaf_k, f16, flb, lb, &split);
     wide = wide_tiles * split >= 64;
   }
   if (!wide) {
@@ -471,7 +509,18 @@ static bool make_plan(int M, int N, int K, int leaf_k, bool f16, Plan* pl, bool 
   return true;
 }
 
+static size_t region_workspace_bytes(int M, int N, int K, int leaf_k, bool f16) {
+  Plan pl;
+  if (!make_plan(M, N, K, leaf_k, f16, &pl)) return 0;
+  return pl.partial_bytes + pl.parked_bytes;
+}
+
 size_t gemm_workspace_bytes(int M, int N, int K, int leaf_k, bool f16, bool rowmajor_b) {
+  if (!rowmajor_b) {
+    // the two column regions run one after the other and share the workspace
+    if (const int na = column_regions(M, N, K, leaf_k, f16))
+      return std::max(region_workspace_bytes(M, na, K, leaf_k, f16), region_workspace_bytes(M, N - na, K, leaf_k, f16));
+  }
   Plan pl;
   if (!make_plan(M, N, K, leaf_k, f16, &pl, rowmajor_b)) return 0;
   if (rowmajor_b) return pl.partial_bytes;
@@ -479,9 +528,19 @@ size_t gemm_workspace_bytes(int M, int N, int K, int leaf_k, bool f16, bool rowm
   return pl.partial_bytes + pl.parked_bytes;
 }
 
+static int gemm_dispatch_impl(bool tree, bool f16, const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n,
+                              void* C, int64_t ldc, int M, int N, int K, int leaf_k, const void* bias, void* ws,
+                              size_t ws_bytes, hipStream_t stream, bool whole_problem);
+
 int gemm_dispatch(bool tree, bool f16, const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C,
                   int64_t ldc, int M, int N, int K, int leaf_k, const void* bias, void* ws, size_t ws_bytes,
                   hipStream_t stream) {
+  return gemm_dispatch_impl(tree, f16, A, lda, B, ldb_k, ldb_n, C, ldc, M, N, K, leaf_k, bias, ws, ws_bytes, stream, true);
+}
+
+static int gemm_dispatch_impl(bool tree, bool f16, const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n,
+                              void* C, int64_t ldc, int M, int N, int K, int leaf_k, const void* bias, void* ws,
+                              size_t ws_bytes, hipStream_t stream, bool whole_problem) {
   if (M < 0 || N < 0 || K <= 0) return TBIK_ERR_INVALID;
   if (M == 0 || N == 0) return TBIK_OK;  // nothing to do (empty tensors may come with null pointers)
   if (!A || !B || !C) return TBIK_ERR_INVALID;
@@ -550,6 +609,19 @@ int gemm_dispatch(bool tree, bool f16, const void* A, int64_t lda, const void* B
     if (waves) {
       StripArgs sa{a.X, a.W, a.C, a.bias, a.ldx, a.ldw, a.ldc, M, N, K, flb, level_k - 1, a.vec_store};
       return gemm_tree_strip_launch(sa, leaf_k, waves, f16, stream);
+    }
+  }
+  if (whole_problem && !rowmajor_b) {
+    if (const int na = column_regions(M, N, K, leaf_k, f16)) {
+      // columns [0, na) and [na, N) as problems of their own, one after the other on the stream, sharing the workspace
+      const size_t esz = sizeof(uint16_t);
+      const int rc = gemm_dispatch_impl(tree, f16, A, lda, B, ldb_k, ldb_n, C, ldc, M, na, K, leaf_k, bias, ws, ws_bytes,
+                                        stream, false);
+      if (rc != TBIK_OK) return rc;
+      return gemm_dispatch_impl(tree, f16, A, lda, static_cast<const uint8_t*>(B) + (size_t)na * ldb_n * esz, ldb_k, ldb_n,
+                                static_cast<uint8_t*>(C) + (size_t)na * esz, ldc, M, N - na, K, leaf_k,
+                                bias ? static_cast<const uint8_t*>(bias) + (size_t)na * esz : nullptr, ws, ws_bytes,
+                                stream, false);
     }
   }
   Plan pl;
