@@ -25,6 +25,18 @@ int gemm_tree_wide_launch(const WideArgs& a, int leaf_k, bool f16, int split, hi
 // gemm_tree_wide_deep.hip: the same tile and bits for leaves of 256 with two binary levels in registers (a.lb >= 2 uses
 // both); takes the same arguments
 int gemm_tree_deep_launch(const WideArgs& a, int split, hipStream_t stream);
+// Two problems in ONE launch of either kernel (column regions of one GEMM, each with a K split of its own): the
+// work-groups of `first` come first in the grid (give it the longer shards, so that the short work-groups of `second`
+// fill the CUs that finish early), then those of `second`; every work-group computes what it would compute in a launch
+// of its problem alone.
+struct WidePair {
+  WideArgs first, second;
+  int split_first, split_second;
+};
+template <bool PAIR> struct WideKernelArgs { using type = WideArgs; };
+template <> struct WideKernelArgs<true> { using type = WidePair; };
+int gemm_tree_wide_pair_launch(const WidePair& a, int leaf_k, bool f16, hipStream_t stream);
+int gemm_tree_deep_pair_launch(const WidePair& a, hipStream_t stream);
 
 // gemm_single_acc_quad.hip: single-accumulator bf16 GEMM, one wave per SIMD
 struct QuadArgs {

@@ -509,17 +509,35 @@ static bool make_plan(int M, int N, int K, int leaf_k, bool f16, Plan* pl, bool 
   return true;
 }
 
-static size_t region_workspace_bytes(int M, int N, int K, int leaf_k, bool f16) {
-  Plan pl;
-  if (!make_plan(M, N, K, leaf_k, f16, &pl)) return 0;
-  return pl.partial_bytes + pl.parked_bytes;
+// The two column regions of a problem (column_regions): when both run on the same 128x256-tile kernel they go out as
+// ONE launch (the short work-groups of one region fill the CUs that the long ones of the other leave early) and each
+// needs a workspace of its own; otherwise they run one after the other and share it.
+struct RegionPlan {
+  int na;     // columns of the first region; 0: the problem runs in one piece
+  bool pair;  // one launch for both
+  Plan a, b;
+  size_t bytes_a, bytes_b, bytes;
+};
+
+static bool plan_regions(int M, int N, int K, int leaf_k, bool f16, RegionPlan* rp) {
+  rp->na = column_regions(M, N, K, leaf_k, f16);
+  if (!rp->na) return false;
+  if (!make_plan(M, rp->na, K, leaf_k, f16, &rp->a) || !make_plan(M, N - rp->na, K, leaf_k, f16, &rp->b)) {
+    rp->na = 0;
+    return false;
+  }
+  rp->bytes_a = (rp->a.partial_bytes + rp->a.parked_bytes + 255) & ~(size_t)255;
+  rp->bytes_b = (rp->b.partial_bytes + rp->b.parked_bytes + 255) & ~(size_t)255;
+  rp->pair = rp->a.wide && rp->b.wide &&
+             wide_uses_deep_kernel(leaf_k, f16, rp->a.flb, rp->a.lb) == wide_uses_deep_kernel(leaf_k, f16, rp->b.flb, rp->b.lb);
+  rp->bytes = rp->pair ? rp->bytes_a + rp->bytes_b : std::max(rp->bytes_a, rp->bytes_b);
+  return true;
 }
 
 size_t gemm_workspace_bytes(int M, int N, int K, int leaf_k, bool f16, bool rowmajor_b) {
   if (!rowmajor_b) {
-    // the two column regions run one after the other and share the workspace
-    if (const int na = column_regions(M, N, K, leaf_k, f16))
-      return std::max(region_workspace_bytes(M, na, K, leaf_k, f16), region_workspace_bytes(M, N - na, K, leaf_k, f16));
+    RegionPlan rp;
+    if (plan_regions(M, N, K, leaf_k, f16, &rp)) return rp.bytes;
   }
   Plan pl;
   if (!make_plan(M, N, K, leaf_k, f16, &pl, rowmajor_b)) return 0;
@@ -611,18 +629,57 @@ static int gemm_dispatch_impl(bool tree, bool f16, const void* A, int64_t lda, c
       return gemm_tree_strip_launch(sa, leaf_k, waves, f16, stream);
     }
   }
-  if (whole_problem && !rowmajor_b) {
-    if (const int na = column_regions(M, N, K, leaf_k, f16)) {
+  RegionPlan rp;
+  if (whole_problem && !rowmajor_b && plan_regions(M, N, K, leaf_k, f16, &rp)) {
+    const size_t esz = sizeof(uint16_t);
+    const int na = rp.na;
+    const void* Bb = static_cast<const uint8_t*>(B) + (size_t)na * ldb_n * esz;
+    void* Cb = static_cast<uint8_t*>(C) + (size_t)na * esz;
+    const void* bias_b = bias ? static_cast<const uint8_t*>(bias) + (size_t)na * esz : nullptr;
+    if (!rp.pair) {
       // columns [0, na) and [na, N) as problems of their own, one after the other on the stream, sharing the workspace
-      const size_t esz = sizeof(uint16_t);
       const int rc = gemm_dispatch_impl(tree, f16, A, lda, B, ldb_k, ldb_n, C, ldc, M, na, K, leaf_k, bias, ws, ws_bytes,
                                         stream, false);
       if (rc != TBIK_OK) return rc;
-      return gemm_dispatch_impl(tree, f16, A, lda, static_cast<const uint8_t*>(B) + (size_t)na * ldb_n * esz, ldb_k, ldb_n,
-                                static_cast<uint8_t*>(C) + (size_t)na * esz, ldc, M, N - na, K, leaf_k,
-                                bias ? static_cast<const uint8_t*>(bias) + (size_t)na * esz : nullptr, ws, ws_bytes,
+      return gemm_dispatch_impl(tree, f16, A, lda, Bb, ldb_k, ldb_n, Cb, ldc, M, N - na, K, leaf_k, bias_b, ws, ws_bytes,
                                 stream, false);
     }
+    if (rp.bytes > 0 && (!ws || ws_bytes < rp.bytes || !aligned16(ws))) return TBIK_ERR_WORKSPACE;
+    uint8_t* wsa = static_cast<uint8_t*>(ws);
+    uint8_t* wsb2 = wsa + rp.bytes_a;
+    // the kernel arguments of one region: its shards write [M, n] partials into its workspace when K is cut
+    auto region_args = [&](const Plan& pl, const void* Bw, void* Cr, const void* bias_r, int n, uint8_t* w) {
+      WideArgs r{a.X, static_cast<const uint16_t*>(Bw), static_cast<uint16_t*>(Cr), static_cast<const uint16_t*>(bias_r),
+                 reinterpret_cast<u32x4*>(w + pl.partial_bytes), a.ldx, a.ldw, a.ldc, M, n, K / pl.split, pl.T, pl.flb, pl.lb,
+                 ((reinterpret_cast<uintptr_t>(Cr) & 7) == 0 && (ldc & 3) == 0) ? 1 : 0, (int64_t)(K / pl.split), 0};
+      if (pl.split > 1) {
+        r.C = reinterpret_cast<uint16_t*>(w);
+        r.ldc = n;
+        r.c_shard = (int64_t)M * n;
+        r.vec_store = (n & 3) == 0 ? 1 : 0;
+        r.bias = nullptr;
+      }
+      return r;
+    };
+    const WideArgs ra = region_args(rp.a, B, C, bias, na, wsa);
+    const WideArgs rb = region_args(rp.b, Bb, Cb, bias_b, N - na, wsb2);
+    // the region with the longer shards first
+    const bool a_first = ra.K >= rb.K;
+    const WidePair pair{a_first ? ra : rb, a_first ? rb : ra, a_first ? rp.a.split : rp.b.split, a_first ? rp.b.split : rp.a.split};
+    int rc = wide_uses_deep_kernel(leaf_k, f16, rp.a.flb, rp.a.lb) ? gemm_tree_deep_pair_launch(pair, stream)
+                                                                   : gemm_tree_wide_pair_launch(pair, leaf_k, f16, stream);
+    if (rc != TBIK_OK) return rc;
+    const void* parts[32];
+    if (rp.a.split > 1) {
+      for (int i = 0; i < rp.a.split; i++) parts[i] = wsa + (size_t)i * M * na * esz;
+      rc = tree_combine_bias_dispatch(parts, rp.a.split, C, (int64_t)M * na, bias, na, f16, stream, ldc);
+      if (rc != TBIK_OK) return rc;
+    }
+    if (rp.b.split > 1) {
+      for (int i = 0; i < rp.b.split; i++) parts[i] = wsb2 + (size_t)i * M * (N - na) * esz;
+      rc = tree_combine_bias_dispatch(parts, rp.b.split, Cb, (int64_t)M * (N - na), bias_b, N - na, f16, stream, ldc);
+    }
+    return rc;
   }
   Plan pl;
   if (!make_plan(M, N, K, leaf_k, f16, &pl, rowmajor_b)) return TBIK_ERR_INVALID;

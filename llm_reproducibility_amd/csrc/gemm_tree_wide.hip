@@ -52,8 +52,8 @@ size_t wide_workspace_bytes(int M, int N, int lb, int split, int levels_in_regis
 }
 
 // F16: the operands and the tree nodes are fp16 instead of bf16 (same tile, ring and order; a node is one packed add).
-template <int LS, bool F16 = false>
-__global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs p) {
+template <int LS, bool F16 = false, bool PAIR = false>
+__global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const typename WideKernelArgs<PAIR>::type pp) {
   using namespace wide;
   using NUM = Num16<F16>;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -64,13 +64,26 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
   const int wm = wave >> 2;  // 0..1
   const int wn = wave & 3;   // 0..3
 
+  // one problem per launch, or two (WidePair): the block index decides which one this work-group belongs to
+  WideArgs p;
+  int wg = blockIdx.x, nwg = gridDim.x, shard = blockIdx.y, nshards = gridDim.y;
+  if constexpr (PAIR) {
+    const int tiles_first = ((pp.first.M + BM - 1) / BM) * ((pp.first.N + BN - 1) / BN);
+    const int wg_second = tiles_first * pp.split_first;
+    const bool second = (int)blockIdx.x >= wg_second;  // wave-uniform
+    p = second ? pp.second : pp.first;
+    nshards = second ? pp.split_second : pp.split_first;
+    nwg = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
+    wg = second ? blockIdx.x - wg_second : blockIdx.x;
+    shard = wg / nwg;
+    wg -= shard * nwg;
+  } else {
+    p = pp;
+  }
   const int tiles_m = (p.M + BM - 1) / BM;
   const int tiles_n = (p.N + BN - 1) / BN;
-  int lid = blockIdx.x;
-  {
-    const int nwg = gridDim.x;
-    if ((nwg & 7) == 0) lid = (lid & 7) * (nwg >> 3) + (lid >> 3);  // consecutive ids share an XCD
-  }
+  int lid = wg;
+  if ((nwg & 7) == 0) lid = (lid & 7) * (nwg >> 3) + (lid >> 3);  // consecutive ids share an XCD
   constexpr int GROUP = 8;
   const int per_group = GROUP * tiles_n;
   const int group_id = lid / per_group;
@@ -80,9 +93,8 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
   const int pid_n = (lid % per_group) / gsz;
   const int m0 = pid_m * BM;
   const int n0 = pid_n * BN;
-  const int shard = blockIdx.y;
   const int tile_id = (shard * tiles_m + pid_m) * tiles_n + pid_n;
-  const int ntiles = tiles_m * tiles_n * gridDim.y;
+  const int ntiles = tiles_m * tiles_n * nshards;
 
   // ---- direct global->LDS loads.  Wave w's i-th load of a slice fills LDS rows [8*(8i+w), +8): lane l
   // lands at row 8*(8i+w) + l/8, physical 16-byte chunk l%8, so it fetches logical chunk (l%8)^(l/8).
@@ -349,25 +361,44 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const WideArgs
   }
 }
 
-template <int LS, bool F16>
-static int wide_launch(const WideArgs& a, unsigned tiles, int split, hipStream_t stream) {
+static int wide_check(const WideArgs& a, int64_t* tiles) {
+  using namespace wide;
+  *tiles = (int64_t)((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
+  if (*tiles <= 0 || *tiles > 0x7fffffff || a.lb > MAXLB) return TBIK_ERR_UNSUPPORTED;
+  if (a.ldx >= (1 << 22) || a.ldw >= (1 << 22)) return TBIK_ERR_UNSUPPORTED;  // 32-bit in-tile byte offsets
+  return TBIK_OK;
+}
+
+template <int LS, bool F16, bool PAIR>
+static int wide_launch(const typename WideKernelArgs<PAIR>::type& a, dim3 grid, hipStream_t stream) {
   using namespace wide;
   constexpr size_t smem = (size_t)NSLOT * STAGE_BYTES + 16384;  // 144 KiB ring + 16 KiB staging
-  auto kern = gemm_tree_wide_kernel<LS, F16>;
+  auto kern = gemm_tree_wide_kernel<LS, F16, PAIR>;
   static std::atomic<uint64_t> done{0};
   hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), (int)smem, done);
   if (e != hipSuccess) return hip_code(e);
-  hipLaunchKernelGGL(kern, dim3(tiles, (unsigned)split), dim3(NT), smem, stream, a);
+  hipLaunchKernelGGL(kern, grid, dim3(NT), smem, stream, a);
   return hip_code(hipGetLastError());
 }
 
 int gemm_tree_wide_launch(const WideArgs& a, int leaf_k, bool f16, int split, hipStream_t stream) {
-  using namespace wide;
-  const int64_t tiles = (int64_t)((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
-  if (tiles <= 0 || tiles > 0x7fffffff || a.lb > MAXLB) return TBIK_ERR_UNSUPPORTED;
-  if (a.ldx >= (1 << 22) || a.ldw >= (1 << 22)) return TBIK_ERR_UNSUPPORTED;  // 32-bit in-tile byte offsets
-  if (leaf_k == 256) return f16 ? wide_launch<4, true>(a, (unsigned)tiles, split, stream) : wide_launch<4, false>(a, (unsigned)tiles, split, stream);
-  if (leaf_k == 128) return f16 ? wide_launch<2, true>(a, (unsigned)tiles, split, stream) : wide_launch<2, false>(a, (unsigned)tiles, split, stream);
+  int64_t tiles;
+  if (const int rc = wide_check(a, &tiles)) return rc;
+  const dim3 grid((unsigned)tiles, (unsigned)split);
+  if (leaf_k == 256) return f16 ? wide_launch<4, true, false>(a, grid, stream) : wide_launch<4, false, false>(a, grid, stream);
+  if (leaf_k == 128) return f16 ? wide_launch<2, true, false>(a, grid, stream) : wide_launch<2, false, false>(a, grid, stream);
+  return TBIK_ERR_UNSUPPORTED;
+}
+
+int gemm_tree_wide_pair_launch(const WidePair& a, int leaf_k, bool f16, hipStream_t stream) {
+  int64_t t1, t2;
+  if (const int rc = wide_check(a.first, &t1)) return rc;
+  if (const int rc = wide_check(a.second, &t2)) return rc;
+  const int64_t wgs = t1 * a.split_first + t2 * a.split_second;
+  if (a.split_first <= 0 || a.split_second <= 0 || wgs > 0x7fffffff) return TBIK_ERR_UNSUPPORTED;
+  const dim3 grid((unsigned)wgs);
+  if (leaf_k == 256) return f16 ? wide_launch<4, true, true>(a, grid, stream) : wide_launch<4, false, true>(a, grid, stream);
+  if (leaf_k == 128) return f16 ? wide_launch<2, true, true>(a, grid, stream) : wide_launch<2, false, true>(a, grid, stream);
   return TBIK_ERR_UNSUPPORTED;
 }
 

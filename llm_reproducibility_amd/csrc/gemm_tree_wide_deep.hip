@@ -38,7 +38,8 @@ constexpr int MAXLB = 16;
 enum Kind { K_NONE = 0, K_ADD = 1, K_P0 = 2, K_P1 = 3, K_P2 = 4 };
 }  // namespace deep
 
-__global__ __launch_bounds__(deep::NT) void gemm_tree_deep_kernel(const WideArgs p) {
+template <bool PAIR>
+__global__ __launch_bounds__(deep::NT) void gemm_tree_deep_kernel(const typename WideKernelArgs<PAIR>::type pp) {
   using namespace deep;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
@@ -48,13 +49,26 @@ __global__ __launch_bounds__(deep::NT) void gemm_tree_deep_kernel(const WideArgs
   const int wm = wave >> 2;  // 0..1
   const int wn = wave & 3;   // 0..3
 
+  // one problem per launch, or two (WidePair): the block index decides which one this work-group belongs to
+  WideArgs p;
+  int wg = blockIdx.x, nwg = gridDim.x, shard = blockIdx.y, nshards = gridDim.y;
+  if constexpr (PAIR) {
+    const int tiles_first = ((pp.first.M + BM - 1) / BM) * ((pp.first.N + BN - 1) / BN);
+    const int wg_second = tiles_first * pp.split_first;
+    const bool second = (int)blockIdx.x >= wg_second;  // wave-uniform
+    p = second ? pp.second : pp.first;
+    nshards = second ? pp.split_second : pp.split_first;
+    nwg = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
+    wg = second ? blockIdx.x - wg_second : blockIdx.x;
+    shard = wg / nwg;
+    wg -= shard * nwg;
+  } else {
+    p = pp;
+  }
   const int tiles_m = (p.M + BM - 1) / BM;
   const int tiles_n = (p.N + BN - 1) / BN;
-  int lid = blockIdx.x;
-  {
-    const int nwg = gridDim.x;
-    if ((nwg & 7) == 0) lid = (lid & 7) * (nwg >> 3) + (lid >> 3);  // consecutive ids share an XCD
-  }
+  int lid = wg;
+  if ((nwg & 7) == 0) lid = (lid & 7) * (nwg >> 3) + (lid >> 3);  // consecutive ids share an XCD
   constexpr int GROUP = 8;
   const int per_group = GROUP * tiles_n;
   const int group_id = lid / per_group;
@@ -64,9 +78,8 @@ __global__ __launch_bounds__(deep::NT) void gemm_tree_deep_kernel(const WideArgs
   const int pid_n = (lid % per_group) / gsz;
   const int m0 = pid_m * BM;
   const int n0 = pid_n * BN;
-  const int shard = blockIdx.y;
   const int tile_id = (shard * tiles_m + pid_m) * tiles_n + pid_n;
-  const int ntiles = tiles_m * tiles_n * gridDim.y;
+  const int ntiles = tiles_m * tiles_n * nshards;
 
   // ---- direct global->LDS loads.  Wave w's i-th load of a slice fills LDS rows [8*(8i+w), +8): lane l
   // lands at row 8*(8i+w) + l/8, physical 16-byte chunk l%8, so it fetches logical chunk (l%8)^(l/8).
@@ -344,17 +357,40 @@ __global__ __launch_bounds__(deep::NT) void gemm_tree_deep_kernel(const WideArgs
   }
 }
 
+static int deep_check(const WideArgs& a, int64_t* tiles) {
+  using namespace deep;
+  *tiles = (int64_t)((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
+  if (*tiles <= 0 || *tiles > 0x7fffffff || a.lb > MAXLB) return TBIK_ERR_UNSUPPORTED;
+  if (a.ldx >= (1 << 22) || a.ldw >= (1 << 22)) return TBIK_ERR_UNSUPPORTED;  // 32-bit in-tile byte offsets
+  return TBIK_OK;
+}
+
 int gemm_tree_deep_launch(const WideArgs& a, int split, hipStream_t stream) {
   using namespace deep;
   constexpr size_t smem = (size_t)NSLOT * STAGE_BYTES + 16384;  // 144 KiB ring + 16 KiB staging
-  const int64_t tiles = (int64_t)((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
-  if (tiles <= 0 || tiles > 0x7fffffff || a.lb > MAXLB) return TBIK_ERR_UNSUPPORTED;
-  if (a.ldx >= (1 << 22) || a.ldw >= (1 << 22)) return TBIK_ERR_UNSUPPORTED;  // 32-bit in-tile byte offsets
-  auto kern = gemm_tree_deep_kernel;
+  int64_t tiles;
+  if (const int rc = deep_check(a, &tiles)) return rc;
+  auto kern = gemm_tree_deep_kernel<false>;
   static std::atomic<uint64_t> done{0};
   hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), (int)smem, done);
   if (e != hipSuccess) return hip_code(e);
   hipLaunchKernelGGL(kern, dim3((unsigned)tiles, (unsigned)split), dim3(NT), smem, stream, a);
+  return hip_code(hipGetLastError());
+}
+
+int gemm_tree_deep_pair_launch(const WidePair& a, hipStream_t stream) {
+  using namespace deep;
+  constexpr size_t smem = (size_t)NSLOT * STAGE_BYTES + 16384;
+  int64_t t1, t2;
+  if (const int rc = deep_check(a.first, &t1)) return rc;
+  if (const int rc = deep_check(a.second, &t2)) return rc;
+  const int64_t wgs = t1 * a.split_first + t2 * a.split_second;
+  if (a.split_first <= 0 || a.split_second <= 0 || wgs > 0x7fffffff) return TBIK_ERR_UNSUPPORTED;
+  auto kern = gemm_tree_deep_kernel<true>;
+  static std::atomic<uint64_t> done{0};
+  hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), (int)smem, done);
+  if (e != hipSuccess) return hip_code(e);
+  hipLaunchKernelGGL(kern, dim3((unsigned)wgs), dim3(NT), smem, stream, a);
   return hip_code(hipGetLastError());
 }
 
