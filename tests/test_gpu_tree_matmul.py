@@ -103,6 +103,34 @@ def test_large_tile_kernels_match_oracle_bitwise(dev, M, N, K, leaf):
     assert_bitwise(h, O.matmul_tree(A.to(torch.float16), Wnk.to(torch.float16).t(), bias.to(torch.float16), leaf=leaf), "fp16")
 
 
+# grids that do not fill whole rounds of work-groups: the dispatcher cuts the columns into two regions, each with a K split
+# of its own, and launches both at once (o_proj 32B at 512 and 1024 rows: 4 and 16 shards / 2 and 8; a leaf-128 tree;
+# a region that is not cut at all next to one cut in two)
+@pytest.mark.parametrize("M,N,K,leaf", [(512, 5120, 8192, 256), (1024, 5120, 8192, 256), (2048, 5120, 6400, 128), (2048, 5120, 2048, 256), (1024, 5120, 16384, 256)])
+def test_column_regions_with_their_own_k_split_match_oracle_bitwise(dev, M, N, K, leaf):
+    print("case", M, N, K, leaf, flush=True)
+    A = O.integer_bf16((M, K), -9, 9, 70 + M % 89)
+    Wnk = O.integer_bf16((N, K), -7, 7, 80 + N % 97)
+    bias = O.integer_bf16((N,), -300, 300, 7)
+    Ad, Wd, bd = A.to(dev), Wnk.to(dev), bias.to(dev)
+    got = matmul_tp_persistent(Ad, Wd.t(), bd, leaf_k=leaf)
+    assert_bitwise(got, O.matmul_tree(A, Wnk.t(), bias, leaf=leaf), f"{M}x{N}x{K}")
+    # any block of columns computed alone (another plan, other regions) has the same bits
+    for lo, hi in ((0, 256), (256, 1280), (4096, N), (1000, 3000)):
+        part = matmul_tp_persistent(Ad, Wd[lo:hi].t(), bd[lo:hi], leaf_k=leaf)
+        assert torch.equal(part, got[:, lo:hi]), (lo, hi)
+    # Gaussian operands: rows alone and simulated TP agree bitwise with the batch
+    g = O.gaussian_bf16((M, K), 1.0, 71).to(dev)
+    gw = O.gaussian_bf16((N, K), 0.02, 72).to(dev)
+    full = matmul_tp_persistent(g, gw.t(), leaf_k=leaf)
+    assert torch.equal(matmul_tp_persistent(g[:1], gw.t(), leaf_k=leaf), full[:1])
+    assert torch.equal(matmul_tp_persistent(g[M - 70:], gw.t(), leaf_k=leaf), full[M - 70:])
+    assert torch.equal(sim_tp(g, gw.t(), 2, leaf), full)
+    if M == 512:  # the same grid in fp16 (the first of the two kernels, instantiated for fp16)
+        h = matmul_tp_persistent(Ad.to(torch.float16), Wd.to(torch.float16).t(), bd.to(torch.float16), leaf_k=leaf)
+        assert_bitwise(h, O.matmul_tree(A.to(torch.float16), Wnk.to(torch.float16).t(), bias.to(torch.float16), leaf=leaf), "fp16")
+
+
 def test_large_tile_kernels_seeded_sweep_of_random_shapes(dev):
     """Random grids of 128x256 tiles (64 or more rows, ragged edges, trees of every depth and group size the leaf count
     allows, leaves of 128 and 256, bf16 and fp16, with and without bias): bit-exact against the oracle on integer inputs."""
