@@ -68,7 +68,7 @@ __global__ __launch_bounds__(sq::NT) void gemm_single_acc_256_kernel(const QuadA
   int lid = blockIdx.x;
   {
     const int nwg = gridDim.x;
-    if ((nwg & 7) == 0) lid = (lid & 7) * (nwg >> 3) + (lid >> 3);  // consecutive ids share an XCD
+    lid = xcd_contiguous_tile(lid, nwg);
   }
   constexpr int GROUP = 4;
   const int per_group = GROUP * tiles_n;

@@ -77,7 +77,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_kernel(const GemmA
   int lid = blockIdx.x;
   {
     const int nwg = gridDim.x;
-    if ((nwg & 7) == 0) lid = (lid & 7) * (nwg >> 3) + (lid >> 3);
+    lid = xcd_contiguous_tile(lid, nwg);
   }
   constexpr int GROUP = 8;
   const int per_group = GROUP * tiles_n;

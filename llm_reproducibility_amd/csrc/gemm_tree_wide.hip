@@ -83,7 +83,7 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const typename
   const int tiles_m = (p.M + BM - 1) / BM;
   const int tiles_n = (p.N + BN - 1) / BN;
   int lid = wg;
-  if ((nwg & 7) == 0) lid = (lid & 7) * (nwg >> 3) + (lid >> 3);  // consecutive ids share an XCD
+  lid = xcd_contiguous_tile(lid, nwg);
   constexpr int GROUP = 8;
   const int per_group = GROUP * tiles_n;
   const int group_id = lid / per_group;
