@@ -67,7 +67,8 @@ __global__ __launch_bounds__(NWAVES * 64) void gemm_single_acc_stream_rows_kerne
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int n0 = (blockIdx.x * NW + wave) * 16;
+  // every XCD streams a contiguous range of the weight rows (lm_head at 8 rows: 228 -> 211 us)
+  const int n0 = (xcd_contiguous_tile(blockIdx.x, gridDim.x) * NW + wave) * 16;
   const int r = lane & 15, g = lane >> 4;
   const uint16_t* wp = p.W + (int64_t)min(n0 + r, p.N - 1) * p.ldw + 8 * g;
   const int nsteps = p.K / 32;
@@ -139,7 +140,8 @@ __global__ __launch_bounds__(NWAVES * 64) void gemm_single_acc_stream_kernel(con
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int n0 = (blockIdx.x * NW + wave) * 16;
+  // every XCD streams a contiguous range of the weight rows (lm_head at 8 rows: 228 -> 211 us)
+  const int n0 = (xcd_contiguous_tile(blockIdx.x, gridDim.x) * NW + wave) * 16;
   const int r = lane & 15, g = lane >> 4;
 
   const uint16_t* wp = p.W + (int64_t)min(n0 + r, p.N - 1) * p.ldw + 8 * g;

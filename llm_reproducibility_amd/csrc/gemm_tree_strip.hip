@@ -29,7 +29,7 @@ __global__ __launch_bounds__(64 * S) __attribute__((amdgpu_waves_per_eu(4, 8))) 
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int n0 = blockIdx.x * 16;
+  const int n0 = xcd_contiguous_tile(blockIdx.x, gridDim.x) * 16;  // every XCD streams a contiguous range of weight rows
   const int r = lane & 15, g = lane >> 4;
   const int groups = (1 << p.lb) / S;   // groups of FLB leaves in this wave's subtree (a power of two)
   const int nch = groups * p.flb * CPL;  // chunks of this wave

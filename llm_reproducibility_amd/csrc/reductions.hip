@@ -357,8 +357,10 @@ __global__ __launch_bounds__(512) void lsm_resident_kernel(const LsmArgs a) {
   typedef typename LsmElem<IN>::type in_t;
   typedef typename LsmElem<OUT>::type out_t;
   const int tid = threadIdx.x, half = tid >> 8, t = tid & 255, lane = tid & 63, wave = (tid >> 6) & 3;
-  const in_t* xr = static_cast<const in_t*>(a.x) + (int64_t)blockIdx.x * a.ldx;
-  out_t* orow = static_cast<out_t*>(a.out) + (int64_t)blockIdx.x * a.ldo;
+  // every XCD walks a contiguous range of rows (4096 rows of 151936 floats: 1026 -> 979 us)
+  const int64_t row = xcd_contiguous_tile(blockIdx.x, gridDim.x);
+  const in_t* xr = static_cast<const in_t*>(a.x) + row * a.ldx;
+  out_t* orow = static_cast<out_t*>(a.out) + row * a.ldo;
   const int cols = (int)a.cols, segs = a.segs;
   const int nfull = cols >> 12;                                       // full segments
   const int nreg = (nfull & ~1) < 2 * RK ? (nfull & ~1) : 2 * RK;     // ... of which in registers (whole slots)
