@@ -29,10 +29,10 @@
 namespace tbik {
 
 namespace sq {
-constexpr int BM = 256, BN = 256, BK = 64, NT = 256, NWAVE = 4, TM = 8, TN = 8;
+constexpr int BM = 256, BK = 64, NT = 256, NWAVE = 4, TM = 8;
 constexpr int BLOCK_ROWS = 128, BLOCK_BYTES = BLOCK_ROWS * BK * 2;  // 16 KiB
 constexpr int NBLOCK = 10;                                         // ring positions: 160 KiB
-constexpr int BDMA = BLOCK_ROWS / 8 / NWAVE;                       // direct loads per wave per block: 4 (8 rows each)
+constexpr int BDMA = BLOCK_ROWS / 8 / NWAVE;                       // direct loads per wave per block of X: 4 (8 rows each)
 __device__ __forceinline__ int wrap(int pos) { return pos >= NBLOCK ? pos - NBLOCK : pos; }
 }  // namespace sq
 
@@ -56,8 +56,15 @@ __device__ __forceinline__ void mfma_results_ready() {
   __builtin_amdgcn_sched_barrier(0);
 }
 
+// TN = 8: 256x256 tile.  TN = 6: 256x192 tile (wave tiles of 128x96) for grids that the square tile does not spread
+// evenly: the W blocks then hold 96 rows at the same ring positions.
+template <int TN>
 __global__ __launch_bounds__(sq::NT) void gemm_single_acc_256_kernel(const QuadArgs p) {
   using namespace sq;
+  constexpr int BN = 2 * TN * 16;
+  constexpr int WROWS = TN * 16;             // rows of a W block
+  constexpr int WDMA = WROWS / 8 / NWAVE;    // direct loads per wave per block of W: 4 / 3
+  static_assert(WROWS % (8 * NWAVE) == 0 && (TN == 6 || TN == 8), "tile width");
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -82,26 +89,31 @@ __global__ __launch_bounds__(sq::NT) void gemm_single_acc_256_kernel(const QuadA
   const uint8_t* xbase = reinterpret_cast<const uint8_t*>(p.X + (int64_t)m0 * p.ldx);
   const uint8_t* wbase = reinterpret_cast<const uint8_t*>(p.W + (int64_t)n0 * p.ldw);
   // byte offsets of this lane's direct loads inside the tile's operands: [half][load]; rows past the edge are clamped
-  uint32_t voffx[2 * BDMA], voffw[2 * BDMA];
+  uint32_t voffx[2 * BDMA], voffw[2 * WDMA];
   {
     const int r = lane >> 3, c = (lane & 7) ^ r;
 #pragma unroll
     for (int i = 0; i < 2 * BDMA; i++) {
       const int row = (i / BDMA) * BLOCK_ROWS + ((i % BDMA) * NWAVE + wave) * 8 + r;
       voffx[i] = (uint32_t)(((min(m0 + row, p.M - 1) - m0) * p.ldx + c * 8) * 2);
+    }
+#pragma unroll
+    for (int i = 0; i < 2 * WDMA; i++) {
+      const int row = (i / WDMA) * WROWS + ((i % WDMA) * NWAVE + wave) * 8 + r;
       voffw[i] = (uint32_t)(((min(n0 + row, p.N - 1) - n0) * p.ldw + c * 8) * 2);
     }
   }
   const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
   const int nslices = p.K / BK;
-  // load i (0..7: half i / 4, rows of load i % 4) of the X or W blocks of slice s into ring position pos of that half;
+  // load i (half i / BDMA, rows of load i % BDMA; WDMA for W) of the X or W blocks of slice s into ring position pos of
+  // that half;
   // slices past the end of K load the last one again (never read): the count of loads in flight stays the same
   auto dma_x = [&](int s, int pos, int i) __attribute__((always_inline)) {
     dma16(lds0 + pos * BLOCK_BYTES + ((i % BDMA) * NWAVE + wave) * 1024, voffx[i],
           xbase + (int64_t)min(s, nslices - 1) * (BK * 2));
   };
   auto dma_w = [&](int s, int pos, int i) __attribute__((always_inline)) {
-    dma16(lds0 + pos * BLOCK_BYTES + ((i % BDMA) * NWAVE + wave) * 1024, voffw[i],
+    dma16(lds0 + pos * BLOCK_BYTES + ((i % WDMA) * NWAVE + wave) * 1024, voffw[i],
           wbase + (int64_t)min(s, nslices - 1) * (BK * 2));
   };
   const int frow = lane & 15, fchk = lane >> 4;
@@ -121,7 +133,7 @@ __global__ __launch_bounds__(sq::NT) void gemm_single_acc_256_kernel(const QuadA
 #pragma unroll
     for (int i = 0; i < 2 * BDMA; i++) dma_x(s, 4 * s + i / BDMA, i);
 #pragma unroll
-    for (int i = 0; i < 2 * BDMA; i++) dma_w(s, 4 * s + 2 + i / BDMA, i);
+    for (int i = 0; i < 2 * WDMA; i++) dma_w(s, 4 * s + 2 + i / WDMA, i);
   }
 #pragma unroll
   for (int i = 0; i < 2 * BDMA; i++) dma_x(2, 8 + i / BDMA, i);
@@ -132,10 +144,10 @@ __global__ __launch_bounds__(sq::NT) void gemm_single_acc_256_kernel(const QuadA
       // zero here, long before the first MFMA, and opaque from here on: a zero that the compiler knows to be zero is
       // written again right in front of the first MFMA, closer than an MFMA may follow a write of its accumulator
       acc[a][b] = f32x4{0.f, 0.f, 0.f, 0.f};
-      if (b < TN - 1) asm volatile("" : "+a"(acc[a][b]));
+      if (TN < 8 || b < TN - 1) asm volatile("" : "+a"(acc[a][b]));
       else asm volatile("" : "+v"(acc[a][b]));
     }
-  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(6 * BDMA) : "memory");
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(4 * BDMA + 2 * WDMA) : "memory");  // all but slice 0
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
 #pragma unroll
@@ -152,21 +164,24 @@ __global__ __launch_bounds__(sq::NT) void gemm_single_acc_256_kernel(const QuadA
       for (int q = 0; q < TM; q++) {
 #pragma unroll
         for (int b = 0; b < TN; b++) {
-          if (b < TN - 1) mfma_in_agprs(acc[q][b], fw[kk][b], fx[kk][q]);
+          if (TN < 8 || b < TN - 1) mfma_in_agprs(acc[q][b], fw[kk][b], fx[kk][q]);
           else mfma_in_vgprs(acc[q][b], fw[kk][b], fx[kk][q]);
           if (b == 0 || b == 2) {
             // fragments of the next k step: the second of this slice, or the first of the next slice (behind the
             // last slice that reads blocks whose loads have landed and are never used)
-            if (kk == 0) read_frag(1, xpos, wpos, 1, 2 * q + (b >> 1));
-            else read_frag(0, xpos1, wpos1, 0, 2 * q + (b >> 1));
+            const int f = 2 * q + (b >> 1);
+            if (f < TM + TN) {
+              if (kk == 0) read_frag(1, xpos, wpos, 1, f);
+              else read_frag(0, xpos1, wpos1, 0, f);
+            }
           }
-          if (b == 4) {
+          if (b == (TN > 4 ? 4 : 3)) {
             // first k step: X blocks of slice s+2 into the positions of the W blocks of slice s-1 (the prologue has
             // issued those of slice 2); second k step: W blocks of slice s+2 into the positions of the X blocks of s
             if (kk == 0) {
               if (s > 0) dma_x(s + 2, wrap(px + 8 + q / BDMA), q);
-            } else {
-              dma_w(s + 2, wrap(px + q / BDMA), q);
+            } else if (q < 2 * WDMA) {
+              dma_w(s + 2, wrap(px + q / WDMA), q);
             }
           }
           __builtin_amdgcn_sched_barrier(0);
@@ -215,17 +230,27 @@ __global__ __launch_bounds__(sq::NT) void gemm_single_acc_256_kernel(const QuadA
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
-int gemm_single_acc_256_launch(const QuadArgs& a, hipStream_t stream) {
+template <int TN>
+static int sq_launch(const QuadArgs& a, hipStream_t stream) {
   using namespace sq;
+  constexpr int BN = 2 * TN * 16;
   constexpr size_t smem = (size_t)NBLOCK * BLOCK_BYTES;  // 160 KiB: all of a CU's LDS
   const int64_t tiles = (int64_t)((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
   if (tiles <= 0 || tiles > 0x7fffffff || a.K < BK || (a.K % BK) != 0) return TBIK_ERR_UNSUPPORTED;
   if (a.ldx >= (1 << 22) || a.ldw >= (1 << 22)) return TBIK_ERR_UNSUPPORTED;  // 32-bit in-tile byte offsets
   static std::atomic<uint64_t> done{0};
-  hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(gemm_single_acc_256_kernel), (int)smem, done);
+  hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(gemm_single_acc_256_kernel<TN>), (int)smem, done);
   if (e != hipSuccess) return hip_code(e);
-  hipLaunchKernelGGL(gemm_single_acc_256_kernel, dim3((unsigned)tiles), dim3(NT), smem, stream, a);
+  hipLaunchKernelGGL(gemm_single_acc_256_kernel<TN>, dim3((unsigned)tiles), dim3(NT), smem, stream, a);
   return hip_code(hipGetLastError());
+}
+
+int gemm_single_acc_256_launch(const QuadArgs& a, int tile_cols, hipStream_t stream) {
+  switch (tile_cols) {
+    case 256: return sq_launch<8>(a, stream);
+    case 192: return sq_launch<6>(a, stream);
+    default: return TBIK_ERR_UNSUPPORTED;
+  }
 }
 
 }  // namespace tbik

@@ -246,47 +246,64 @@ int gemm_single_acc_balanced_launch(const QuadArgs& a, hipStream_t stream) {
   const double floor_us = (double)a.N * a.K * 2.0 / 3.5e6;
   static const int widths[6] = {8, 6, 4, 3, 2, 1};
   int best = 8;
-  double best_t = 0.0;
+  double best_t = 0.0, best_sustained = 0.0;  // the second without the overlap of later rounds (see below)
   for (int i = 0; i < 6; i++) {
     const int tn = widths[i];
     const int64_t tiles = tm * (((int64_t)a.N + 32 * tn - 1) / (32 * tn));
     const double s0 = 0.185 + 0.0665 * tn;
-    double t;
+    double t, ts;
     if (tn <= 2) {  // up to two work-groups per CU
       if (tiles <= 256) {
-        t = 3.0 + nsl * s0 * (1.0 + 0.16 * (double)tiles / 256.0);
+        t = ts = 3.0 + nsl * s0 * (1.0 + 0.16 * (double)tiles / 256.0);
       } else {
         const double rounds = (double)((tiles + 511) / 512);
         t = (3.0 + nsl * s0 * 1.7) * (1.0 + 0.9 * (rounds - 1.0));
+        ts = (3.0 + nsl * s0 * 1.7) * rounds;
       }
     } else {
-      t = 0.0;
+      t = ts = 0.0;
       int64_t left = tiles;
       for (int r = 0; left > 0; r++, left -= 256) {
         const double fill = (double)(left < 256 ? left : 256) / 256.0;
-        t += (r == 0 ? 1.0 : 0.9) * (3.0 + nsl * s0 * (1.0 + 0.16 * fill));
+        const double round = 3.0 + nsl * s0 * (1.0 + 0.16 * fill);
+        t += (r == 0 ? 1.0 : 0.9) * round;
+        ts += round;
       }
     }
     if (t < floor_us) t = floor_us + 1e-3 * t;  // memory-bound either way: keep the order of the compute estimates
+    if (ts < floor_us) ts = floor_us + 1e-3 * ts;
     if (i == 0 || t < best_t) {
       best_t = t;
       best = tn;
     }
+    if (i == 0 || ts < best_sustained) best_sustained = ts;
   }
-  // Many rounds of tiles: the 256x256 tile halves the L2 traffic and the LDS reads per flop.  A round of it costs
-  // 6 us + 1.44 us per slice against 3 us + 0.83 us per slice of the 128x256 tile, which makes twice the rounds;
-  // from six rounds on the estimate above (fitted on grids of few rounds) is below what the 128x256 tile sustains,
-  // so the comparison uses its sustained rate there.  gate_up [M,4096]x[4096,24576]: M=2048 366 -> 301 us,
-  // M=8192 1402 -> 1175 (vendor library 272 / 1048); down [M,12288]x[12288,4096] at M=4096 319 -> 274 (259).
+  // More than one round of 128x256 tiles: tiles of 256 rows halve the L2 traffic and cut the LDS reads per flop.  A
+  // round of them costs 6 us + 1.44 / 1.15 us per slice for 256 / 192 columns, against 3 us + 0.83 us per slice of the
+  // 128x256 tile (a 256x128 tile was measured too, 0.84 us per slice: never ahead); the width that wastes the fewest
+  // CU-rounds wins.  The estimate above overlaps later
+  // rounds with the one before (fitted on grids of one to two rounds); a grid that runs for several rounds sustains no
+  // such overlap, so the comparison uses the sum of whole rounds, and from six rounds on the measured sustained rate.
+  // gate_up [M,4096]x[4096,24576]: M=2048 366 -> 301 us, M=8192 1402 -> 1175 (vendor library 272 / 1048); qkv
+  // (N=6144) at M=2048 97 -> 85 (256 tiles of 256x192: one round; vendor 84), at M=4096 177 -> 161 (159).
   {
     const int64_t tiles8 = tm * (((int64_t)a.N + 255) / 256);
-    const int64_t tiles256 = (((int64_t)a.M + 255) / 256) * (((int64_t)a.N + 255) / 256);
     const double rounds8 = (double)((tiles8 + 255) / 256);
-    double t256 = (double)((tiles256 + 255) / 256) * (6.0 + nsl * 1.44);
-    if (t256 < floor_us) t256 = floor_us + 1e-3 * t256;
-    const double t128 = rounds8 >= 6.0 ? rounds8 * (3.0 + nsl * 0.83) : best_t;
-    if (tiles8 > 256 && t256 < t128)
-      return gemm_single_acc_256_launch(a, stream);
+    static const int cols[2] = {256, 192};
+    static const double per_slice[2] = {1.44, 1.15};
+    int best_cols = 0;
+    double t_sq = 0.0;
+    for (int i = 0; i < 2; i++) {
+      const int64_t tiles = (((int64_t)a.M + 255) / 256) * (((int64_t)a.N + cols[i] - 1) / cols[i]);
+      double t = (double)((tiles + 255) / 256) * (6.0 + nsl * per_slice[i]);
+      if (t < floor_us) t = floor_us + 1e-3 * t;
+      if (i == 0 || t < t_sq) {
+        t_sq = t;
+        best_cols = cols[i];
+      }
+    }
+    const double t128 = rounds8 >= 6.0 ? rounds8 * (3.0 + nsl * 0.83) : best_sustained;
+    if (tiles8 > 256 && t_sq < t128) return gemm_single_acc_256_launch(a, best_cols, stream);
   }
   switch (best) {
     case 8: return quad_launch<8>(a, stream);
