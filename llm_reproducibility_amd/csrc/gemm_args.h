@@ -51,9 +51,9 @@ struct QuadArgs {
 int gemm_single_acc_quad_launch(const QuadArgs& a, hipStream_t stream);
 int gemm_single_acc_slab_launch(const QuadArgs& a, hipStream_t stream);  // at most 128 rows; TBIK_ERR_UNSUPPORTED: use another kernel
 int gemm_single_acc_balanced_launch(const QuadArgs& a, hipStream_t stream);  // any row count: tile width from a cost model
-// gemm_single_acc_256.hip: the same GEMM on tiles of 256 rows and tile_cols = 256 or 192 columns, for grids of
-// many rounds; K % 64 == 0
-int gemm_single_acc_256_launch(const QuadArgs& a, int tile_cols, hipStream_t stream);
+// gemm_single_acc_256.hip: the same GEMM on tiles of 256 or 192 rows by 256 or 192 columns, for grids of more than one
+// round; K % 64 == 0
+int gemm_single_acc_256_launch(const QuadArgs& a, int tile_rows, int tile_cols, hipStream_t stream);
 
 // gemm_single_acc_stream.hip: single-accumulator 16-bit GEMM for at most 64 rows, weights streamed from global memory
 struct StreamArgs {

@@ -29,10 +29,9 @@
 namespace tbik {
 
 namespace sq {
-constexpr int BM = 256, BK = 64, NT = 256, NWAVE = 4, TM = 8;
-constexpr int BLOCK_ROWS = 128, BLOCK_BYTES = BLOCK_ROWS * BK * 2;  // 16 KiB
+constexpr int BK = 64, NT = 256, NWAVE = 4;
+constexpr int BLOCK_BYTES = 128 * BK * 2;                          // 16 KiB: a ring position holds up to 128 rows
 constexpr int NBLOCK = 10;                                         // ring positions: 160 KiB
-constexpr int BDMA = BLOCK_ROWS / 8 / NWAVE;                       // direct loads per wave per block of X: 4 (8 rows each)
 __device__ __forceinline__ int wrap(int pos) { return pos >= NBLOCK ? pos - NBLOCK : pos; }
 }  // namespace sq
 
@@ -56,15 +55,17 @@ __device__ __forceinline__ void mfma_results_ready() {
   __builtin_amdgcn_sched_barrier(0);
 }
 
-// TN = 8: 256x256 tile.  TN = 6: 256x192 tile (wave tiles of 128x96) for grids that the square tile does not spread
-// evenly: the W blocks then hold 96 rows at the same ring positions.
-template <int TN>
+// TM = TN = 8: 256x256 tile.  TM, TN = 6: 192 rows / columns (wave tiles of 96 rows / columns) for grids that the square
+// tile does not spread evenly: the X / W blocks then hold 96 rows at the same ring positions.
+template <int TM, int TN>
 __global__ __launch_bounds__(sq::NT) void gemm_single_acc_256_kernel(const QuadArgs p) {
   using namespace sq;
-  constexpr int BN = 2 * TN * 16;
-  constexpr int WROWS = TN * 16;             // rows of a W block
-  constexpr int WDMA = WROWS / 8 / NWAVE;    // direct loads per wave per block of W: 4 / 3
-  static_assert(WROWS % (8 * NWAVE) == 0 && (TN == 6 || TN == 8), "tile width");
+  constexpr int BM = 2 * TM * 16, BN = 2 * TN * 16;
+  constexpr int XROWS = TM * 16, WROWS = TN * 16;  // rows of an X / W block
+  constexpr int BDMA = XROWS / 8 / NWAVE;          // direct loads per wave per block of X (8 rows each): 4 / 3
+  constexpr int WDMA = WROWS / 8 / NWAVE;          // ... of W
+  constexpr int RPR = (TM + TN + TM - 1) / TM;     // fragment reads behind a row of MFMAs: 2, or 3 for the 192x256 tile
+  static_assert((TM == 6 || TM == 8) && (TN == 6 || TN == 8), "tile shape");
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -94,7 +95,7 @@ __global__ __launch_bounds__(sq::NT) void gemm_single_acc_256_kernel(const QuadA
     const int r = lane >> 3, c = (lane & 7) ^ r;
 #pragma unroll
     for (int i = 0; i < 2 * BDMA; i++) {
-      const int row = (i / BDMA) * BLOCK_ROWS + ((i % BDMA) * NWAVE + wave) * 8 + r;
+      const int row = (i / BDMA) * XROWS + ((i % BDMA) * NWAVE + wave) * 8 + r;
       voffx[i] = (uint32_t)(((min(m0 + row, p.M - 1) - m0) * p.ldx + c * 8) * 2);
     }
 #pragma unroll
@@ -166,22 +167,25 @@ __global__ __launch_bounds__(sq::NT) void gemm_single_acc_256_kernel(const QuadA
         for (int b = 0; b < TN; b++) {
           if (TN < 8 || b < TN - 1) mfma_in_agprs(acc[q][b], fw[kk][b], fx[kk][q]);
           else mfma_in_vgprs(acc[q][b], fw[kk][b], fx[kk][q]);
-          if (b == 0 || b == 2) {
+          if (b < 2 * RPR - 1 && (RPR == 3 || (b & 1) == 0)) {
             // fragments of the next k step: the second of this slice, or the first of the next slice (behind the
             // last slice that reads blocks whose loads have landed and are never used)
-            const int f = 2 * q + (b >> 1);
+            const int f = RPR * q + (RPR == 3 ? b : b >> 1);
             if (f < TM + TN) {
               if (kk == 0) read_frag(1, xpos, wpos, 1, f);
               else read_frag(0, xpos1, wpos1, 0, f);
             }
           }
-          if (b == (TN > 4 ? 4 : 3)) {
+          if (b == 4 || b == 6) {
             // first k step: X blocks of slice s+2 into the positions of the W blocks of slice s-1 (the prologue has
-            // issued those of slice 2); second k step: W blocks of slice s+2 into the positions of the X blocks of s
+            // issued those of slice 2); second k step: W blocks of slice s+2 into the positions of the X blocks of s.
+            // One load behind the fifth MFMA of every row, and where a k step has more loads than rows (the 192x256
+            // tile) the rest behind the seventh MFMA of the first rows
+            const int d = b == 4 ? q : TM + q;
             if (kk == 0) {
-              if (s > 0) dma_x(s + 2, wrap(px + 8 + q / BDMA), q);
-            } else if (q < 2 * WDMA) {
-              dma_w(s + 2, wrap(px + q / WDMA), q);
+              if (s > 0 && d < 2 * BDMA) dma_x(s + 2, wrap(px + 8 + d / BDMA), d);
+            } else if (d < 2 * WDMA) {
+              dma_w(s + 2, wrap(px + d / WDMA), d);
             }
           }
           __builtin_amdgcn_sched_barrier(0);
@@ -230,27 +234,27 @@ __global__ __launch_bounds__(sq::NT) void gemm_single_acc_256_kernel(const QuadA
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
-template <int TN>
+template <int TM, int TN>
 static int sq_launch(const QuadArgs& a, hipStream_t stream) {
   using namespace sq;
-  constexpr int BN = 2 * TN * 16;
+  constexpr int BM = 2 * TM * 16, BN = 2 * TN * 16;
   constexpr size_t smem = (size_t)NBLOCK * BLOCK_BYTES;  // 160 KiB: all of a CU's LDS
   const int64_t tiles = (int64_t)((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
   if (tiles <= 0 || tiles > 0x7fffffff || a.K < BK || (a.K % BK) != 0) return TBIK_ERR_UNSUPPORTED;
   if (a.ldx >= (1 << 22) || a.ldw >= (1 << 22)) return TBIK_ERR_UNSUPPORTED;  // 32-bit in-tile byte offsets
   static std::atomic<uint64_t> done{0};
-  hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(gemm_single_acc_256_kernel<TN>), (int)smem, done);
+  hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(gemm_single_acc_256_kernel<TM, TN>), (int)smem, done);
   if (e != hipSuccess) return hip_code(e);
-  hipLaunchKernelGGL(gemm_single_acc_256_kernel<TN>, dim3((unsigned)tiles), dim3(NT), smem, stream, a);
+  hipLaunchKernelGGL((gemm_single_acc_256_kernel<TM, TN>), dim3((unsigned)tiles), dim3(NT), smem, stream, a);
   return hip_code(hipGetLastError());
 }
 
-int gemm_single_acc_256_launch(const QuadArgs& a, int tile_cols, hipStream_t stream) {
-  switch (tile_cols) {
-    case 256: return sq_launch<8>(a, stream);
-    case 192: return sq_launch<6>(a, stream);
-    default: return TBIK_ERR_UNSUPPORTED;
-  }
+int gemm_single_acc_256_launch(const QuadArgs& a, int tile_rows, int tile_cols, hipStream_t stream) {
+  if (tile_rows == 256 && tile_cols == 256) return sq_launch<8, 8>(a, stream);
+  if (tile_rows == 256 && tile_cols == 192) return sq_launch<8, 6>(a, stream);
+  if (tile_rows == 192 && tile_cols == 256) return sq_launch<6, 8>(a, stream);
+  if (tile_rows == 192 && tile_cols == 192) return sq_launch<6, 6>(a, stream);
+  return TBIK_ERR_UNSUPPORTED;
 }
 
 }  // namespace tbik

@@ -278,32 +278,37 @@ int gemm_single_acc_balanced_launch(const QuadArgs& a, hipStream_t stream) {
     }
     if (i == 0 || ts < best_sustained) best_sustained = ts;
   }
-  // More than one round of 128x256 tiles: tiles of 256 rows halve the L2 traffic and cut the LDS reads per flop.  A
-  // round of them costs 6 us + 1.44 / 1.15 us per slice for 256 / 192 columns, against 3 us + 0.83 us per slice of the
-  // 128x256 tile (a 256x128 tile was measured too, 0.84 us per slice: never ahead); the width that wastes the fewest
-  // CU-rounds wins.  The estimate above overlaps later
-  // rounds with the one before (fitted on grids of one to two rounds); a grid that runs for several rounds sustains no
-  // such overlap, so the comparison uses the sum of whole rounds, and from six rounds on the measured sustained rate.
-  // gate_up [M,4096]x[4096,24576]: M=2048 366 -> 301 us, M=8192 1402 -> 1175 (vendor library 272 / 1048); qkv
-  // (N=6144) at M=2048 97 -> 85 (256 tiles of 256x192: one round; vendor 84), at M=4096 177 -> 161 (159).
+  // More than one round of 128x256 tiles: the kernel with wave tiles of 128x128 (gemm_single_acc_256.hip) halves the L2
+  // traffic and cuts the LDS reads per flop.  It has tiles of 256 or 192 rows by 256 or 192 columns; a round costs 6 us
+  // + 1.44 / 1.17 / 1.20 / 0.94 us per slice (256x256 / 256x192 / 192x256 / 192x192, a little less on a round that does
+  // not fill the chip), against 3 us + 0.83 us per slice of the 128x256 tile; the shape that wastes the fewest CU-rounds
+  // wins.  The estimate above overlaps later rounds with the one before (fitted on grids of one to two rounds); a grid
+  // that runs for several rounds sustains no such overlap, so the comparison uses the sum of whole rounds, and from six
+  // rounds on the measured sustained rate.  gate_up [M,4096]x[4096,24576]: M=384 84 -> 67 us (256 tiles of 192x192,
+  // vendor library 73), M=2048 366 -> 301, M=8192 1402 -> 1175 (272 / 1048); qkv (N=6144) at M=1536 76 -> 67 (74), at
+  // M=2048 97 -> 85 (256 tiles of 256x192: one round; 84), at M=4096 177 -> 161 (159).
   {
     const int64_t tiles8 = tm * (((int64_t)a.N + 255) / 256);
     const double rounds8 = (double)((tiles8 + 255) / 256);
-    static const int cols[2] = {256, 192};
-    static const double per_slice[2] = {1.44, 1.15};
-    int best_cols = 0;
+    static const int shape[4][2] = {{256, 256}, {256, 192}, {192, 256}, {192, 192}};
+    static const double per_slice[4] = {1.44, 1.17, 1.20, 0.94};
+    int pick = 0;
     double t_sq = 0.0;
-    for (int i = 0; i < 2; i++) {
-      const int64_t tiles = (((int64_t)a.M + 255) / 256) * (((int64_t)a.N + cols[i] - 1) / cols[i]);
-      double t = (double)((tiles + 255) / 256) * (6.0 + nsl * per_slice[i]);
+    for (int i = 0; i < 4; i++) {
+      int64_t left = (((int64_t)a.M + shape[i][0] - 1) / shape[i][0]) * (((int64_t)a.N + shape[i][1] - 1) / shape[i][1]);
+      double t = 0.0;
+      for (; left > 0; left -= 256) {
+        const double fill = (double)(left < 256 ? left : 256) / 256.0;
+        t += 6.0 + nsl * per_slice[i] * (1.0 + 0.16 * fill) / 1.16;
+      }
       if (t < floor_us) t = floor_us + 1e-3 * t;
       if (i == 0 || t < t_sq) {
         t_sq = t;
-        best_cols = cols[i];
+        pick = i;
       }
     }
     const double t128 = rounds8 >= 6.0 ? rounds8 * (3.0 + nsl * 0.83) : best_sustained;
-    if (tiles8 > 256 && t_sq < t128) return gemm_single_acc_256_launch(a, best_cols, stream);
+    if (tiles8 > 256 && t_sq < t128) return gemm_single_acc_256_launch(a, shape[pick][0], shape[pick][1], stream);
   }
   switch (best) {
     case 8: return quad_launch<8>(a, stream);

@@ -226,9 +226,11 @@ def test_single_accumulator_mm_balanced_tiles_match_oracle_bitwise(dev, M, N, K)
 
 # grids of more than one round, where the cost model picks tiles of 256 rows: one round of 256 tiles with ragged edges in
 # M and N, an odd number of 64-wide slices, five rounds with a last column of tiles eight columns wide; then 256x192
-# tiles (qkv-like: one round of 256 tiles; two rounds; ragged in M and N)
+# tiles (qkv-like: one round of 256 tiles; two rounds; ragged in M and N), 192x192 tiles (gate_up at 384 rows: one round
+# of 256 tiles; ragged) and 192x256 tiles (one round of 256 tiles)
 @pytest.mark.parametrize("M,N,K", [(2040, 8190, 1024), (4096, 4090, 2112), (8192, 8200, 1024), (2048, 8192, 768),
-                                   (2048, 6144, 1024), (4096, 6144, 512), (1990, 6100, 1088)])
+                                   (2048, 6144, 1024), (4096, 6144, 512), (1990, 6100, 1088),
+                                   (384, 24576, 1024), (1530, 6100, 1024), (3072, 4096, 2048)])
 def test_single_accumulator_mm_256_tiles_match_oracle_bitwise(dev, M, N, K):
     """256x256 tiles (accumulators pinned by hand in both register files, ten-block LDS ring): integer inputs, so the
     oracle's bits are the only right answer; rows alone (streaming kernel), the first 129 rows (128-row tiles) and the
