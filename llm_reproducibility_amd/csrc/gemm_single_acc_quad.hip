@@ -19,7 +19,7 @@
 namespace tbik {
 
 namespace quad {
-constexpr int BM = 128, BK = 64, NT = 256, NWAVE = 4, TM = 4, NSLOT = 3;
+constexpr int BM = 128, BK = 64, NT = 256, NWAVE = 4, TM = 4;
 constexpr int XDMA = BM / 8 / NWAVE;    // direct loads of X rows per wave per slice: 4 (8 rows of 128 B each)
 template <int TN>
 struct Shape {
@@ -33,9 +33,13 @@ struct Shape {
 // TN = 8: the 128x256 tile of the large shapes.  TN = 1..4 and 6: the same pipeline on 128x32 .. 128x192 tiles for
 // grids that the wide tile would not spread over the chip: the width is chosen per call so that the CUs get the same
 // number of work-groups (gemm_single_acc_balanced_launch).
-template <int TN>
+// NSLOT: slices of the ring.  Three keep a work-group fed when the chip is full of them; a grid of at most one narrow
+// tile per CU (a handful of rows times a moderate N) is a chain of slices, each waiting for loads issued NSLOT - 1
+// slices earlier, so those grids get a ring as deep as the LDS allows (5 or 6 slices).
+template <int TN, int NSLOT>
 __global__ __launch_bounds__(quad::NT) void gemm_single_acc_quad_kernel(const QuadArgs p) {
   using namespace quad;
+  static_assert(NSLOT >= 3, "the schedule needs a slice in use, one landing and one in flight");
   constexpr int BN = Shape<TN>::BN, STAGE_BYTES = Shape<TN>::STAGE_BYTES, NDMA = Shape<TN>::NDMA;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -94,7 +98,7 @@ __global__ __launch_bounds__(quad::NT) void gemm_single_acc_quad_kernel(const Qu
   for (int s = 0; s < NSLOT; s++)
 #pragma unroll
     for (int i = 0; i < NDMA; i++) dma_one(s, s, i);
-  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(2 * NDMA) : "memory");
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"((NSLOT - 1) * NDMA) : "memory");
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
 #pragma unroll
@@ -128,8 +132,8 @@ __global__ __launch_bounds__(quad::NT) void gemm_single_acc_quad_kernel(const Qu
             if (f < TM) read_x(kk ^ 1, rslot, kk ^ 1, f);
             else if (f - TM < TN) read_w(kk ^ 1, rslot, kk ^ 1, f - TM);
           } else {
-            if (kk == 1 && q < H1) dma_one(s + 3, slot, q);
-            if (kk == 0 && q < H2 && s > 0) dma_one(s + 2, pslot, H1 + q);
+            if (kk == 1 && q < H1) dma_one(s + NSLOT, slot, q);
+            if (kk == 0 && q < H2 && s > 0) dma_one(s + NSLOT - 1, pslot, H1 + q);
           }
           __builtin_amdgcn_sched_barrier(0);
         };
@@ -147,7 +151,7 @@ __global__ __launch_bounds__(quad::NT) void gemm_single_acc_quad_kernel(const Qu
       }
       if (kk == 0) {
         // mid-slice: slice s+1 has landed (this wave's share) and every fragment read of slice s is done
-        asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NDMA) : "memory");
+        asm volatile("s_waitcnt vmcnt(%0)" : : "n"((NSLOT - 2) * NDMA) : "memory");
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
@@ -184,18 +188,19 @@ __global__ __launch_bounds__(quad::NT) void gemm_single_acc_quad_kernel(const Qu
   }
 }
 
-template <int TN>
+template <int TN, int NSLOT = 3>
 static int quad_launch(const QuadArgs& a, hipStream_t stream) {
   using namespace quad;
   constexpr int BN = Shape<TN>::BN;
   constexpr size_t smem = (size_t)NSLOT * Shape<TN>::STAGE_BYTES;  // 144 KiB for the 256-wide tile
+  static_assert(smem <= 160 * 1024 && (NSLOT - 1) * Shape<TN>::NDMA < 64, "ring does not fit the LDS or the wait counter");
   const int64_t tiles = (int64_t)((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
   if (tiles <= 0 || tiles > 0x7fffffff || a.K < BK || (a.K % BK) != 0) return TBIK_ERR_UNSUPPORTED;
   if (a.ldx >= (1 << 22) || a.ldw >= (1 << 22)) return TBIK_ERR_UNSUPPORTED;  // 32-bit in-tile byte offsets
   static std::atomic<uint64_t> done{0};
-  hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(gemm_single_acc_quad_kernel<TN>), (int)smem, done);
+  hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(gemm_single_acc_quad_kernel<TN, NSLOT>), (int)smem, done);
   if (e != hipSuccess) return hip_code(e);
-  hipLaunchKernelGGL(gemm_single_acc_quad_kernel<TN>, dim3((unsigned)tiles), dim3(NT), smem, stream, a);
+  hipLaunchKernelGGL((gemm_single_acc_quad_kernel<TN, NSLOT>), dim3((unsigned)tiles), dim3(NT), smem, stream, a);
   return hip_code(hipGetLastError());
 }
 
@@ -222,11 +227,14 @@ int gemm_single_acc_slab_launch(const QuadArgs& a, hipStream_t stream) {
       best = tn;
     }
   }
+  // at most one work-group per CU: the deep ring (see the kernel); qkv [M,4096]x[4096,6144] at M=40 27 -> 18 us, at
+  // M=128 28 -> 24; [M,12288]x[12288,4096] at M=64 72 -> 49 (an eight-slice ring was measured too: no further gain)
+  const bool deep = (((int64_t)a.N + 32 * best - 1) / (32 * (best ? best : 1))) <= 256;
   switch (best) {
-    case 4: return quad_launch<4>(a, stream);
-    case 3: return quad_launch<3>(a, stream);
-    case 2: return quad_launch<2>(a, stream);
-    case 1: return quad_launch<1>(a, stream);
+    case 4: return deep ? quad_launch<4, 5>(a, stream) : quad_launch<4>(a, stream);
+    case 3: return deep ? quad_launch<3, 5>(a, stream) : quad_launch<3>(a, stream);
+    case 2: return deep ? quad_launch<2, 6>(a, stream) : quad_launch<2>(a, stream);
+    case 1: return deep ? quad_launch<1, 6>(a, stream) : quad_launch<1>(a, stream);
     default: return TBIK_ERR_UNSUPPORTED;
   }
 }
@@ -310,13 +318,16 @@ int gemm_single_acc_balanced_launch(const QuadArgs& a, hipStream_t stream) {
     const double t128 = rounds8 >= 6.0 ? rounds8 * (3.0 + nsl * 0.83) : best_sustained;
     if (tiles8 > 256 && t_sq < t128) return gemm_single_acc_256_launch(a, shape[pick][0], shape[pick][1], stream);
   }
+  // at most one narrow tile per CU: the deep ring (see the kernel); qkv at M=160 31 -> 25 us, [M,12288]x[12288,4096]
+  // at M=192 73 -> 51
+  const bool deep = tm * (((int64_t)a.N + 32 * best - 1) / (32 * best)) <= 256;
   switch (best) {
     case 8: return quad_launch<8>(a, stream);
     case 6: return quad_launch<6>(a, stream);
-    case 4: return quad_launch<4>(a, stream);
-    case 3: return quad_launch<3>(a, stream);
-    case 2: return quad_launch<2>(a, stream);
-    default: return quad_launch<1>(a, stream);
+    case 4: return deep ? quad_launch<4, 5>(a, stream) : quad_launch<4>(a, stream);
+    case 3: return deep ? quad_launch<3, 5>(a, stream) : quad_launch<3>(a, stream);
+    case 2: return deep ? quad_launch<2, 6>(a, stream) : quad_launch<2>(a, stream);
+    default: return deep ? quad_launch<1, 6>(a, stream) : quad_launch<1>(a, stream);
   }
 }
 
