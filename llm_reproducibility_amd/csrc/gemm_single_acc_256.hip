@@ -22,6 +22,8 @@
 // (a wave issues in order: a cluster of LDS reads and loads behind a row of MFMAs would leave the MFMA pipe idle
 // while it issues).  The 16-byte chunk c of row r sits at position c ^ (r & 7); a lane of a direct load fetches the
 // global chunk that belongs at its linear LDS position, which realises that swizzle on the source side.
+#include <type_traits>
+
 #include "common.h"
 #include "gemm_args.h"
 #include "lds_direct.h"
@@ -32,7 +34,7 @@ namespace sq {
 constexpr int BK = 64, NT = 256, NWAVE = 4;
 constexpr int BLOCK_BYTES = 128 * BK * 2;                          // 16 KiB: a ring position holds up to 128 rows
 constexpr int NBLOCK = 10;                                         // ring positions: 160 KiB
-__device__ __forceinline__ int wrap(int pos) { return pos >= NBLOCK ? pos - NBLOCK : pos; }
+constexpr __device__ __forceinline__ int wrap(int pos) { return pos >= NBLOCK ? pos - NBLOCK : pos; }
 }  // namespace sq
 
 // The 64 accumulator tiles of a wave are 256 registers, the whole accumulation register file.  Left to the compiler, all
@@ -109,22 +111,24 @@ __global__ __launch_bounds__(sq::NT) void gemm_single_acc_256_kernel(const QuadA
   // load i (half i / BDMA, rows of load i % BDMA; WDMA for W) of the X or W blocks of slice s into ring position pos of
   // that half;
   // slices past the end of K load the last one again (never read): the count of loads in flight stays the same
+  const uint32_t lds_wave = lds0 + wave * 1024;  // this wave's 1 KiB of every group of eight rows
   auto dma_x = [&](int s, int pos, int i) __attribute__((always_inline)) {
-    dma16(lds0 + pos * BLOCK_BYTES + ((i % BDMA) * NWAVE + wave) * 1024, voffx[i],
-          xbase + (int64_t)min(s, nslices - 1) * (BK * 2));
+    dma16_at(lds_wave, pos * BLOCK_BYTES + (i % BDMA) * NWAVE * 1024, voffx[i], xbase + (int64_t)min(s, nslices - 1) * (BK * 2));
   };
   auto dma_w = [&](int s, int pos, int i) __attribute__((always_inline)) {
-    dma16(lds0 + pos * BLOCK_BYTES + ((i % WDMA) * NWAVE + wave) * 1024, voffw[i],
-          wbase + (int64_t)min(s, nslices - 1) * (BK * 2));
+    dma16_at(lds_wave, pos * BLOCK_BYTES + (i % WDMA) * NWAVE * 1024, voffw[i], wbase + (int64_t)min(s, nslices - 1) * (BK * 2));
   };
   const int frow = lane & 15, fchk = lane >> 4;
   const uint32_t frag = (frow * BK + ((fchk ^ (frow & 7)) << 3)) * 2;  // inside a block, row a * 16 + frow, k step 0
 
   f32x4 acc[TM][TN];
   bf16x8 fx[2][TM], fw[2][TN];
-  auto read_frag = [&](int buf, int xpos, int wpos, int kk, int f) __attribute__((always_inline)) {
-    if (f < TM) fx[buf][f] = *reinterpret_cast<const bf16x8*>(smem + xpos * BLOCK_BYTES + (frag ^ (kk * 64)) + f * 16 * BK * 2);
-    else fw[buf][f - TM] = *reinterpret_cast<const bf16x8*>(smem + wpos * BLOCK_BYTES + (frag ^ (kk * 64)) + (f - TM) * 16 * BK * 2);
+  // this wave's fragment addresses inside the first X block / W block of a slice (its half selects the block)
+  const uint32_t xfrag = frag + wm * BLOCK_BYTES, wfrag = frag + wn * BLOCK_BYTES;
+  // fragment f (X rows first) of k step kk of the slice whose first block sits at ring position px (a constant)
+  auto read_frag = [&](int buf, int px, int kk, int f) __attribute__((always_inline)) {
+    if (f < TM) fx[buf][f] = *reinterpret_cast<const bf16x8*>(smem + (xfrag ^ (kk * 64)) + px * BLOCK_BYTES + f * 16 * BK * 2);
+    else fw[buf][f - TM] = *reinterpret_cast<const bf16x8*>(smem + (wfrag ^ (kk * 64)) + wrap(px + 2) * BLOCK_BYTES + (f - TM) * 16 * BK * 2);
   };
 
   // prologue: slices 0 and 1 and the X blocks of slice 2 fill the ten positions; slice 0 visible, fragments of its
@@ -152,13 +156,12 @@ __global__ __launch_bounds__(sq::NT) void gemm_single_acc_256_kernel(const QuadA
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
 #pragma unroll
-  for (int f = 0; f < TM + TN; f++) read_frag(0, wm, 2 + wn, 0, f);
+  for (int f = 0; f < TM + TN; f++) read_frag(0, 0, 0, f);
 
-  int px = 0;  // ring position of the first block of slice s
-  for (int s = 0; s < nslices; s++) {
-    const int px1 = wrap(px + 4);
-    const int xpos = wrap(px + wm), wpos = wrap(px + 2 + wn);      // this wave's blocks of slice s
-    const int xpos1 = wrap(px1 + wm), wpos1 = wrap(px1 + 2 + wn);  // and of slice s+1
+  // One slice; PX, the ring position of its first block, is a constant: the positions repeat every five slices, so the
+  // loop below takes five slices per trip and no instruction is spent on ring arithmetic.
+  auto slice = [&](auto px_c, int s) __attribute__((always_inline)) {
+    constexpr int px = decltype(px_c)::value, px1 = wrap(px + 4);
 #pragma unroll
     for (int kk = 0; kk < 2; kk++) {
 #pragma unroll
@@ -172,8 +175,8 @@ __global__ __launch_bounds__(sq::NT) void gemm_single_acc_256_kernel(const QuadA
             // last slice that reads blocks whose loads have landed and are never used)
             const int f = RPR * q + (RPR == 3 ? b : b >> 1);
             if (f < TM + TN) {
-              if (kk == 0) read_frag(1, xpos, wpos, 1, f);
-              else read_frag(0, xpos1, wpos1, 0, f);
+              if (kk == 0) read_frag(1, px, 1, f);
+              else read_frag(0, px1, 0, f);
             }
           }
           if (b == 4 || b == 6) {
@@ -183,9 +186,9 @@ __global__ __launch_bounds__(sq::NT) void gemm_single_acc_256_kernel(const QuadA
             // tile) the rest behind the seventh MFMA of the first rows
             const int d = b == 4 ? q : TM + q;
             if (kk == 0) {
-              if (s > 0 && d < 2 * BDMA) dma_x(s + 2, wrap(px + 8 + d / BDMA), d);
+              if (s > 0 && d < 2 * BDMA) dma_x(s + 2, wrap(px + 8) + d / BDMA, d);
             } else if (d < 2 * WDMA) {
-              dma_w(s + 2, wrap(px + d / WDMA), d);
+              dma_w(s + 2, px + d / WDMA, d);
             }
           }
           __builtin_amdgcn_sched_barrier(0);
@@ -200,7 +203,17 @@ __global__ __launch_bounds__(sq::NT) void gemm_single_acc_256_kernel(const QuadA
         asm volatile("" ::: "memory");
       }
     }
-    px = px1;
+  };
+  for (int s = 0; s < nslices; s += 5) {
+    slice(std::integral_constant<int, 0>{}, s);
+    if (s + 1 >= nslices) break;
+    slice(std::integral_constant<int, 4>{}, s + 1);
+    if (s + 2 >= nslices) break;
+    slice(std::integral_constant<int, 8>{}, s + 2);
+    if (s + 3 >= nslices) break;
+    slice(std::integral_constant<int, 2>{}, s + 3);
+    if (s + 4 >= nslices) break;
+    slice(std::integral_constant<int, 6>{}, s + 4);
   }
 
   mfma_results_ready();

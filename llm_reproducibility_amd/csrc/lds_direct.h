@@ -20,6 +20,16 @@ __device__ __forceinline__ void dma16(uint32_t lds_addr, uint32_t voff, const vo
                : "memory", "m0");
 }
 
+// The same load to lds_base + offset, the offset a compile-time constant: the sum is formed in m0 itself (one scalar
+// instruction instead of an add and a move; the scalar condition code is clobbered).
+__device__ __forceinline__ void dma16_at(uint32_t lds_base, int offset, uint32_t voff, const void* base) {
+  const void* base_copy;
+  asm volatile("s_add_u32 m0, %1, %4\n\ts_mov_b64 %0, %3\n\tglobal_load_lds_dwordx4 %2, %0"
+               : "=&s"(base_copy)
+               : "s"(lds_base), "v"(voff), "s"(base), "n"(offset)
+               : "memory", "m0", "scc");
+}
+
 // 16-byte-per-lane store to (wave-uniform base) + voff, scalar-base addressing: no per-lane 64-bit pointer.
 __device__ __forceinline__ void store16_sbase(void* base, uint32_t voff, u32x4 v) {
   // the wait states behind the store keep the next instruction from overwriting the data registers while the store
