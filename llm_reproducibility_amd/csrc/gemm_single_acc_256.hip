@@ -217,6 +217,46 @@ __global__ __launch_bounds__(sq::NT) void gemm_single_acc_256_kernel(const QuadA
   }
 
   mfma_results_ready();
+  // Tiles that lie inside N and whose rows allow 16-byte stores go through the LDS (the ring is done with): a lane of
+  // an MFMA tile owns four columns of one row, 8 bytes, and sixteen rows at a time make a store of sixteen 32-byte
+  // pieces; read back row by row, sixteen lanes store one 256-byte row of the wave's tile, whole cache lines.  All
+  // work-groups of a round finish together, so their stores are one burst that the next round's loads queue behind.
+  const bool rows_by_16_bytes = n0 + BN <= p.N && (p.ldc & 7) == 0 && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0;
+  if (rows_by_16_bytes) {
+    constexpr int ROWB = TN * 32 + 16;  // bytes per row of a wave's tile, padded against bank conflicts
+    static_assert(NWAVE * TM * 16 * ROWB <= NBLOCK * BLOCK_BYTES, "staging does not fit");
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the loads past the end of K still write into the ring
+    __builtin_amdgcn_s_barrier();                    // ... and no wave reads it any more
+    uint8_t* stage = smem + wave * (TM * 16 * ROWB);
+#pragma unroll
+    for (int a = 0; a < TM; a++) {
+#pragma unroll
+      for (int b = 0; b < TN; b++) {
+        float bv[4] = {0.f, 0.f, 0.f, 0.f};
+        if (p.bias) {
+          const int n = n0 + (wn * TN + b) * 16 + fchk * 4;
+#pragma unroll
+          for (int e = 0; e < 4; e++) bv[e] = bf16_bits_to_f32(p.bias[n + e]);
+        }
+        const uint32_t lo = pack_bf16x2(acc[a][b][0] + bv[0], acc[a][b][1] + bv[1]);
+        const uint32_t hi = pack_bf16x2(acc[a][b][2] + bv[2], acc[a][b][3] + bv[3]);
+        *reinterpret_cast<uint2*>(stage + (a * 16 + frow) * ROWB + (b * 16 + fchk * 4) * 2) = make_uint2(lo, hi);
+      }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // a wave reads back only what it wrote itself
+    const int rl = lane / (TN * 2), cl = lane % (TN * 2);  // TN * 2 lanes of 16 bytes per row
+    constexpr int RPI = 64 / (TN * 2);                   // rows per instruction: 4, or 5 of which lanes 60..63 idle
+#pragma unroll
+    for (int j = 0; j < (TM * 16 + RPI - 1) / RPI; j++) {
+      const int row = j * RPI + rl;
+      const int m = m0 + wm * TM * 16 + row;
+      if (rl < RPI && row < TM * 16 && m < p.M) {
+        const uint4 v = *reinterpret_cast<const uint4*>(stage + row * ROWB + cl * 16);
+        *reinterpret_cast<uint4*>(p.C + (int64_t)m * p.ldc + n0 + wn * TN * 16 + cl * 8) = v;
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int a = 0; a < TM; a++) {
     const int m = m0 + (wm * TM + a) * 16 + frow;
