@@ -38,6 +38,10 @@ template <> struct WideKernelArgs<true> { using type = WidePair; };
 int gemm_tree_wide_pair_launch(const WidePair& a, int leaf_k, bool f16, hipStream_t stream);
 int gemm_tree_deep_pair_launch(const WidePair& a, hipStream_t stream);
 
+// gemm_tree_quad.hip: tree-ordered bf16 GEMM with leaves of 256 on 128x128 tiles (one wave per SIMD, the tree of a shard
+// in registers: a.lb <= 1, a.ws unused); grid.y = split as for the kernels above
+int gemm_tree_quad_launch(const WideArgs& a, int split, hipStream_t stream);
+
 // gemm_single_acc_quad.hip: single-accumulator bf16 GEMM, one wave per SIMD
 struct QuadArgs {
   const uint16_t* X;   // [M,K], row stride ldx

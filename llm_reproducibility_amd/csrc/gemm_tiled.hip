@@ -534,8 +534,50 @@ static bool plan_regions(int M, int N, int K, int leaf_k, bool f16, RegionPlan* 
   return true;
 }
 
+// 96 .. 128 rows, leaves of 256: one row of 128x256 tiles needs a deep cut of K to occupy the chip, and the pass over
+// that many partial results then weighs as much as a quarter of the GEMM.  Tiles of 128 columns (gemm_tree_quad.hip)
+// occupy it with half the cut.  That kernel is slower per slice than the 128x256-tile kernels, so it is taken only where
+// a shard is short and the grid close to one work-group per CU, the region where a sweep over N = 2048 .. 8192 and
+// K = 2048 .. 16384 on MI355X measured it ahead (by 8 % on average, up to 20 %): shards of 512 .. 1024 of K on 160 .. 256
+// work-groups, or up to 1536 on 224 .. 256.  The shards are aligned subtrees like every other K split, so the bits do
+// not change.
+struct NarrowPlan {
+  int split;
+  int T, flb, lb;  // tree of ONE shard
+  size_t partial_bytes;
+};
+
+static bool narrow_plan(int M, int N, int K, int leaf_k, bool f16, NarrowPlan* np) {
+  int T, flb, level_k;
+  if (f16 || leaf_k != 256 || M < 96 || M > 128 || tbik_tree_params(K, leaf_k, &T, &flb, &level_k) != TBIK_OK) return false;
+  const int lb = level_k - 1;
+  const int64_t tiles = ((int64_t)N + 127) / 128;
+  int best = 0, best_ls = 0;
+  int64_t best_wgs = 0;
+  for (int ls = 0; ls <= lb && ls <= 5; ls++) {
+    const int sp = 1 << ls;
+    const int ks = K / sp;
+    const int64_t wgs = tiles * sp;
+    if (lb - ls > 1 || ks < 512 || ks > 1536 || wgs > 256 || wgs < (ks > 1024 ? 224 : 160)) continue;
+    if (wgs > best_wgs) {
+      best_wgs = wgs;
+      best = sp;
+      best_ls = ls;
+    }
+  }
+  if (!best) return false;
+  np->split = best;
+  np->T = T / best;
+  np->flb = flb;
+  np->lb = lb - best_ls;
+  np->partial_bytes = best > 1 ? (((size_t)best * M * N * sizeof(uint16_t) + 255) & ~(size_t)255) : 0;
+  return true;
+}
+
 size_t gemm_workspace_bytes(int M, int N, int K, int leaf_k, bool f16, bool rowmajor_b) {
   if (!rowmajor_b) {
+    NarrowPlan np;
+    if (narrow_plan(M, N, K, leaf_k, f16, &np)) return np.partial_bytes;
     RegionPlan rp;
     if (plan_regions(M, N, K, leaf_k, f16, &rp)) return rp.bytes;
   }
@@ -628,6 +670,24 @@ static int gemm_dispatch_impl(bool tree, bool f16, const void* A, int64_t lda, c
       StripArgs sa{a.X, a.W, a.C, a.bias, a.ldx, a.ldw, a.ldc, M, N, K, flb, level_k - 1, a.vec_store};
       return gemm_tree_strip_launch(sa, leaf_k, waves, f16, stream);
     }
+  }
+  NarrowPlan np;
+  if (whole_problem && !rowmajor_b && narrow_plan(M, N, K, leaf_k, f16, &np)) {
+    if (np.partial_bytes > 0 && (!ws || ws_bytes < np.partial_bytes || !aligned16(ws))) return TBIK_ERR_WORKSPACE;
+    WideArgs w{a.X, a.W, a.C, a.bias, nullptr, a.ldx, a.ldw, a.ldc, M, N, K / np.split, np.T, np.flb, np.lb, a.vec_store,
+               (int64_t)(K / np.split), 0};
+    if (np.split > 1) {
+      w.C = static_cast<uint16_t*>(ws);
+      w.ldc = N;
+      w.c_shard = (int64_t)M * N;
+      w.vec_store = (N & 3) == 0 ? 1 : 0;
+      w.bias = nullptr;
+    }
+    const int rc = gemm_tree_quad_launch(w, np.split, stream);
+    if (rc != TBIK_OK || np.split == 1) return rc;
+    const void* parts[32];
+    for (int i = 0; i < np.split; i++) parts[i] = static_cast<uint8_t*>(ws) + (size_t)i * M * N * sizeof(uint16_t);
+    return tree_combine_bias_dispatch(parts, np.split, C, (int64_t)M * N, bias, N, f16, stream, ldc);
   }
   RegionPlan rp;
   if (whole_problem && !rowmajor_b && plan_regions(M, N, K, leaf_k, f16, &rp)) {

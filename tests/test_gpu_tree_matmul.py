@@ -131,6 +131,36 @@ def test_column_regions_with_their_own_k_split_match_oracle_bitwise(dev, M, N, K
         assert_bitwise(h, O.matmul_tree(A.to(torch.float16), Wnk.to(torch.float16).t(), bias.to(torch.float16), leaf=leaf), "fp16")
 
 
+# 96..128 rows with short K shards take 128x128 tiles with the shard's tree in registers: shards of one group of 2, 3 or
+# 5 leaves, shards of two groups (one binary level inside the shard), a ragged last tile, a width that is not a multiple
+# of 4 (element-wise stores of the partial results), 160..256 work-groups
+@pytest.mark.parametrize("M,N,K", [(128, 4096, 4096), (100, 3072, 6144), (128, 4000, 12288), (96, 2048, 8192),
+                                   (128, 7162, 5120), (128, 4096, 8192), (113, 5120, 2048)])
+def test_narrow_tiles_for_short_shards_match_oracle_and_the_other_kernels_bitwise(dev, M, N, K):
+    print("case", M, N, K, flush=True)
+    A = O.integer_bf16((M, K), -9, 9, 170 + M % 89)
+    Wnk = O.integer_bf16((N, K), -7, 7, 180 + N % 97)
+    bias = O.integer_bf16((N,), -300, 300, 9)
+    Ad, Wd, bd = A.to(dev), Wnk.to(dev), bias.to(dev)
+    got = matmul_tp_persistent(Ad, Wd.t(), bd, leaf_k=256)
+    assert_bitwise(got, O.matmul_tree(A, Wnk.t(), bias, leaf=256), f"{M}x{N}x{K} with bias")
+    assert_bitwise(matmul_tp_persistent(Ad, Wd.t(), leaf_k=256), O.matmul_tree(A, Wnk.t(), leaf=256), f"{M}x{N}x{K}")
+    # Gaussian operands: fewer rows (the few-rows kernels), more rows (128x256 tiles), a block of columns and the
+    # simulated TP shards all run on other kernels and agree bitwise with this batch (how close those bits are to the
+    # oracle's on Gaussian data is the subject of test_gaussian_inputs_within_one_ulp_of_oracle)
+    g = O.gaussian_bf16((300, K), 1.0, 171).to(dev)
+    gw = O.gaussian_bf16((N, K), 0.02, 172).to(dev)
+    full = matmul_tp_persistent(g[:M], gw.t(), leaf_k=256)
+    assert torch.equal(matmul_tp_persistent(g[:1], gw.t(), leaf_k=256), full[:1])
+    assert torch.equal(matmul_tp_persistent(g[M - 40:M], gw.t(), leaf_k=256), full[M - 40:])
+    assert torch.equal(matmul_tp_persistent(g, gw.t(), leaf_k=256)[:M], full)
+    assert torch.equal(matmul_tp_persistent(g[:M], gw[256:1024].t(), leaf_k=256), full[:, 256:1024])
+    groups = K // 256 // O.tree_params(K, 256)[1]  # a TP degree has to cut K into aligned subtrees
+    for p in (2, 4, 8):
+        if groups % p == 0:
+            assert torch.equal(sim_tp(g[:M], gw.t(), p, 256), full), p
+
+
 def test_large_tile_kernels_seeded_sweep_of_random_shapes(dev):
     """Random grids of 128x256 tiles (64 or more rows, ragged edges, trees of every depth and group size the leaf count
     allows, leaves of 128 and 256, bf16 and fp16, with and without bias): bit-exact against the oracle on integer inputs."""
