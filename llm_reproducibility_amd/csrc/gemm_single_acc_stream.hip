@@ -134,7 +134,9 @@ __global__ __launch_bounds__(NWAVES * 64) void gemm_single_acc_stream_kernel(con
   constexpr int ROWB = rowb(WS);
   constexpr int ROWS = MB * 16;
   constexpr int XBUF = ROWS * ROWB;
-  constexpr int XLD = ROWS * (KW / 8) / NT;  // 16-byte loads per thread per window: 4 * MB
+  constexpr int XCHUNKS = ROWS * (KW / 8);          // 16-byte chunks of a window of X
+  constexpr int XLD = (XCHUNKS + NT - 1) / NT;      // loads per thread per window; where NT does not divide the chunks,
+                                                    // the threads past the end move the last chunk once more
   extern __shared__ __attribute__((aligned(16))) uint8_t xs[];  // two X windows of XBUF bytes
 
   const int tid = threadIdx.x;
@@ -151,7 +153,7 @@ __global__ __launch_bounds__(NWAVES * 64) void gemm_single_acc_stream_kernel(con
   uint32_t xdst[XLD];
 #pragma unroll
   for (int i = 0; i < XLD; i++) {
-    const int q = tid + NT * i;
+    const int q = min(tid + NT * i, XCHUNKS - 1);
     const int row = q / (KW / 8), c = q % (KW / 8);
     xsrc[i] = p.X + (int64_t)min(row, p.M - 1) * p.ldx + c * 8;
     xdst[i] = row * ROWB + c * 16;
@@ -250,15 +252,38 @@ static int stream_launch_nw(const StreamArgs& a, hipStream_t stream) {
 
 template <int MB, int WS, bool F16>
 static int stream_launch(const StreamArgs& a, hipStream_t stream) {
-  // few strips and few rows: two strips per work-group, so that more CUs take part
-  // many strips and three or four blocks of rows: eight strips share each staged window of X, which halves the
-  // activation traffic per strip (gate_up of an 8B model at M=64: 80 us with four strips per work-group, 55 us
-  // with eight; with fewer than about 1500 strips the grid gets too small for this)
-  if constexpr (MB >= 3) {
-    if ((int64_t)a.N >= 1536 * 16) return stream_launch_nw<MB, WS, 8, F16>(a, stream);
+  // Strips per work-group.  More strips share each staged window of X (gate_up of an 8B model at M=64: 80 us with four
+  // strips per work-group, 55 us with eight), but HBM bandwidth is shared about equally among the CUs that ask for it,
+  // so the CU with the most work-groups finishes last.  The estimate is the pass over the weights, stretched by the share
+  // of CU slots that the last round of work-groups leaves idle, plus the restaging of X per strip at a third of the
+  // price of a weight byte (it comes from the L2).  Measured: gate_up at M=32 (1536 strips) 48.4 us as 384 groups of
+  // four (two on every second CU), 41.2 us as 256 groups of six; [32,4096]x[4096,18432] 48.6 -> 35.4; lm_head (9496
+  // strips, ten rounds of groups of four) is within 2 % for three, four and six.
+  const int64_t strips = ((int64_t)a.N + 15) / 16;
+  // grids of many rounds do not run in rounds: the last one matters little there, the restaging of X more
+  if (strips > 4 * 1024) return MB >= 3 ? stream_launch_nw<MB, WS, 8, F16>(a, stream) : stream_launch_nw<MB, WS, 4, F16>(a, stream);
+  static const int cand[5] = {8, 6, 4, 3, 2};
+  int best = 4;
+  double best_cost = 0.0;
+  for (int i = 0; i < 5; i++) {
+    const int nw = cand[i];
+    if (nw == 8 && (MB < 3 || strips < 1536)) continue;  // eight strips per group: many rows and a large grid only
+    if (nw == 2 && MB > 2) continue;                     // two: one or two blocks of rows only
+    const int64_t groups = (strips + nw - 1) / nw;
+    const double fill = (double)groups / (double)(((groups + 255) / 256) * 256);
+    const double cost = (1.0 + 0.35 * (double)a.M / (16.0 * nw)) / fill;
+    if (best_cost == 0.0 || cost < best_cost) {
+      best_cost = cost;
+      best = nw;
+    }
   }
-  if (MB <= 2 && a.N <= 16 * 1024) return stream_launch_nw<MB, WS, (MB <= 2 ? 2 : 4), F16>(a, stream);
-  return stream_launch_nw<MB, WS, 4, F16>(a, stream);
+  switch (best) {
+    case 8: return stream_launch_nw<MB, WS, 8, F16>(a, stream);
+    case 6: return stream_launch_nw<MB, WS, 6, F16>(a, stream);
+    case 3: return stream_launch_nw<MB, WS, 3, F16>(a, stream);
+    case 2: return stream_launch_nw<MB, WS, (MB <= 2 ? 2 : 4), F16>(a, stream);
+    default: return stream_launch_nw<MB, WS, 4, F16>(a, stream);
+  }
 }
 
 template <int NWAVES, bool F16>

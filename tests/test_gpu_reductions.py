@@ -286,6 +286,22 @@ def test_single_accumulator_mm_streaming_kernels_on_ragged_shapes(dev):
     assert torch.equal(bio.matmul_persistent(a1.to(dev), w1.to(dev).t()).cpu(), O.matmul_single_acc(a1, w1.t()))
 
 
+# the windowed streaming kernel forms work-groups of 2, 3, 4, 6 or 8 strips so that every CU gets the same number; with 3
+# and 6 the staging loads of a window do not divide among the threads (the last ones repeat the last chunk)
+@pytest.mark.parametrize("M,N,K", [(32, 24576, 1024), (20, 12288, 1024), (12, 24576, 4096), (40, 2048, 1024), (17, 18432, 544),
+                                   (9, 10240, 4096), (31, 16380, 1056)])
+def test_single_accumulator_mm_streaming_kernel_with_balanced_strip_counts(dev, M, N, K):
+    print("case", M, N, K, flush=True)
+    a = O.integer_bf16((M, K), -9, 9, 300 + M)
+    w = O.integer_bf16((N, K), -7, 7, 310 + N % 101)
+    bias = O.integer_bf16((N,), -50, 50, 320)
+    want = O.matmul_single_acc(a, w.t(), bias)
+    got = bio.matmul_persistent(a.to(dev), w.to(dev).t(), bias.to(dev))
+    assert torch.equal(got.cpu(), want)
+    # a row alone (the whole-X kernel) has the bits it has in the batch
+    assert torch.equal(bio.matmul_persistent(a[M - 1:].to(dev), w.to(dev).t(), bias.to(dev)).cpu(), want[M - 1:])
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 6144, 4096), (5, 1000, 1120), (40, 24576, 512), (64, 1544, 2048), (100, 520, 1024), (300, 4096, 4096)])
 def test_single_accumulator_mm_c_abi_strided_and_misaligned_output(dev, M, N, K):
     """bi_gemm_bf16 itself (no wrapper): C is a column block of a wider matrix, then the same block shifted by one
