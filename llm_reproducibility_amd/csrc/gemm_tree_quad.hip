@@ -1,4 +1,4 @@
-// Tree-ordered bf16 GEMM for gfx950, path of 64 .. 128 rows with short K shards: 128x128 tiles, 4 wavefronts (one per
+// Tree-ordered bf16 GEMM for gfx950, path of 64 .. 256 rows with short K shards: 128x128 tiles, 4 wavefronts (one per
 // SIMD) of 64x64 each, K streamed through a 4-slot LDS ring in 64-element slices -- the pipeline of
 // gemm_single_acc_quad.hip with the merge tree of gemm_tree_wide.hip, and the whole tree of a shard in registers.
 // Replaces matmul_kernel_tp_persistent, src/tbik/tree_based_matmul.py:50-187, where one row of 128x256 tiles needs a
@@ -17,7 +17,7 @@
 //
 // Where it pays (measured on MI355X against the 128x256-tile kernels with their own best split, weights cold): only
 // where a work-group's shard is short, 512 .. 1536 of K -- [128,4096]x[4096,4096] 20.3 -> 17.7 us, [128,6144]x[6144,4096]
-// 25.1 -> 20.7, [128,12288]x[12288,4096] 33.8 -> 32.1, [96,6144]x[6144,3072] 22.4 -> 18.8, [64,8192]x[8192,4096] 22.9 -> 21.0.  On longer shards a slice
+// 25.1 -> 20.7, [128,12288]x[12288,4096] 33.8 -> 32.1, [96,6144]x[6144,3072] 22.4 -> 18.8, [64,8192]x[8192,4096] 22.9 -> 21.0, [256,6144]x[6144,2048] 23.6 -> 19.9.  On longer shards a slice
 // costs 0.59 us against 0.385 us in the single-accumulator kernel with the same tile: the tree's two to three vector
 // instructions per MFMA do not fit behind the MFMAs of ONE wave per SIMD ([512,8192]x[8192,5120] uncut on 128x96 tiles
 // 75 us against 70 us for the 128x256-tile kernels with their K split; [256,K]x[K,N] 10-20 % slower from K = 6144 on),
