@@ -534,14 +534,14 @@ static bool plan_regions(int M, int N, int K, int leaf_k, bool f16, RegionPlan* 
   return true;
 }
 
-// 64 .. 256 rows, leaves of 256: one or two rows of 128x256 tiles need a deep cut of K to occupy the chip, and the pass over
+// 64 .. 512 rows, leaves of 256: one to four rows of 128x256 tiles need a deep cut of K to occupy the chip, and the pass over
 // that many partial results then weighs as much as a quarter of the GEMM.  Tiles of 128 columns (gemm_tree_quad.hip)
 // occupy it with half the cut.  That kernel is slower per slice than the 128x256-tile kernels, so it is taken only where
 // a shard is short and the grid close to one work-group per CU, the region where a sweep over N = 2048 .. 8192 and
 // K = 2048 .. 16384 at 64 .. 128 rows on MI355X measured it ahead (by 8 % on average, up to 20 %; with fewer rows the
 // 64-row tiles of the tiled kernel win): shards of 512 .. 1024 of K on 160 .. 256
-// work-groups, or up to 1536 on 224 .. 256; with two rows of tiles (129 .. 256 rows) only shards of at most 1024 and a
-// cut into at least four (5 % on average there, ahead in every one of 42 shapes, three alternating repetitions each).
+// work-groups, or up to 1536 on 224 .. 256; with two to four rows of tiles (129 .. 512 rows) only shards of at most 1024 and
+// a cut into at least four (6 % on average there, ahead in every one of 59 shapes, three alternating repetitions each).
 // The shards are aligned subtrees like every other K split, so the bits do not change.
 struct NarrowPlan {
   int split;
@@ -551,7 +551,7 @@ struct NarrowPlan {
 
 static bool narrow_plan(int M, int N, int K, int leaf_k, bool f16, NarrowPlan* np) {
   int T, flb, level_k;
-  if (f16 || leaf_k != 256 || M < 64 || M > 256 || tbik_tree_params(K, leaf_k, &T, &flb, &level_k) != TBIK_OK) return false;
+  if (f16 || leaf_k != 256 || M < 64 || M > 512 || tbik_tree_params(K, leaf_k, &T, &flb, &level_k) != TBIK_OK) return false;
   const int lb = level_k - 1;
   const int64_t tiles = (((int64_t)N + 127) / 128) * ((M + 127) / 128);
   int best = 0, best_ls = 0;

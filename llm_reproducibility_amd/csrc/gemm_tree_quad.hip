@@ -1,4 +1,4 @@
-// Tree-ordered bf16 GEMM for gfx950, path of 64 .. 256 rows with short K shards: 128x128 tiles, 4 wavefronts (one per
+// Tree-ordered bf16 GEMM for gfx950, path of 64 .. 512 rows with short K shards: 128x128 tiles, 4 wavefronts (one per
 // SIMD) of 64x64 each, K streamed through a 4-slot LDS ring in 64-element slices -- the pipeline of
 // gemm_single_acc_quad.hip with the merge tree of gemm_tree_wide.hip, and the whole tree of a shard in registers.
 // Replaces matmul_kernel_tp_persistent, src/tbik/tree_based_matmul.py:50-187, where one row of 128x256 tiles needs a

@@ -131,12 +131,12 @@ def test_column_regions_with_their_own_k_split_match_oracle_bitwise(dev, M, N, K
         assert_bitwise(h, O.matmul_tree(A.to(torch.float16), Wnk.to(torch.float16).t(), bias.to(torch.float16), leaf=leaf), "fp16")
 
 
-# 64..256 rows with short K shards take 128x128 tiles with the shard's tree in registers: shards of one group of 2, 3 or
+# 64..512 rows with short K shards take 128x128 tiles with the shard's tree in registers: shards of one group of 2, 3 or
 # 5 leaves, shards of two groups (one binary level inside the shard), a ragged last tile, a width that is not a multiple
 # of 4 (element-wise stores of the partial results), 160..256 work-groups
 @pytest.mark.parametrize("M,N,K", [(128, 4096, 4096), (100, 3072, 6144), (128, 4000, 12288), (96, 2048, 8192),
                                    (128, 7162, 5120), (128, 4096, 8192), (113, 5120, 2048), (64, 4096, 6144), (80, 2048, 12288), (256, 4096, 4096), (192, 2048, 6144),
-                                   (160, 1500, 8192)])
+                                   (160, 1500, 8192), (500, 1024, 6144)])
 def test_narrow_tiles_for_short_shards_match_oracle_and_the_other_kernels_bitwise(dev, M, N, K):
     print("case", M, N, K, flush=True)
     A = O.integer_bf16((M, K), -9, 9, 170 + M % 89)
@@ -149,7 +149,7 @@ def test_narrow_tiles_for_short_shards_match_oracle_and_the_other_kernels_bitwis
     # Gaussian operands: fewer rows (the few-rows kernels), more rows (128x256 tiles), a block of columns and the
     # simulated TP shards all run on other kernels and agree bitwise with this batch (how close those bits are to the
     # oracle's on Gaussian data is the subject of test_gaussian_inputs_within_one_ulp_of_oracle)
-    g = O.gaussian_bf16((300, K), 1.0, 171).to(dev)
+    g = O.gaussian_bf16((M + 172, K), 1.0, 171).to(dev)
     gw = O.gaussian_bf16((N, K), 0.02, 172).to(dev)
     full = matmul_tp_persistent(g[:M], gw.t(), leaf_k=256)
     assert torch.equal(matmul_tp_persistent(g[:1], gw.t(), leaf_k=256), full[:1])
