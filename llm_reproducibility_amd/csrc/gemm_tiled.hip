@@ -509,31 +509,6 @@ static bool make_plan(int M, int N, int K, int leaf_k, bool f16, Plan* pl, bool 
   return true;
 }
 
-// The two column regions of a problem (column_regions): when both run on the same 128x256-tile kernel they go out as
-// ONE launch (the short work-groups of one region fill the CUs that the long ones of the other leave early) and each
-// needs a workspace of its own; otherwise they run one after the other and share it.
-struct RegionPlan {
-  int na;     // columns of the first region; 0: the problem runs in one piece
-  bool pair;  // one launch for both
-  Plan a, b;
-  size_t bytes_a, bytes_b, bytes;
-};
-
-static bool plan_regions(int M, int N, int K, int leaf_k, bool f16, RegionPlan* rp) {
-  rp->na = column_regions(M, N, K, leaf_k, f16);
-  if (!rp->na) return false;
-  if (!make_plan(M, rp->na, K, leaf_k, f16, &rp->a) || !make_plan(M, N - rp->na, K, leaf_k, f16, &rp->b)) {
-    rp->na = 0;
-    return false;
-  }
-  rp->bytes_a = (rp->a.partial_bytes + rp->a.parked_bytes + 255) & ~(size_t)255;
-  rp->bytes_b = (rp->b.partial_bytes + rp->b.parked_bytes + 255) & ~(size_t)255;
-  rp->pair = rp->a.wide && rp->b.wide &&
-             wide_uses_deep_kernel(leaf_k, f16, rp->a.flb, rp->a.lb) == wide_uses_deep_kernel(leaf_k, f16, rp->b.flb, rp->b.lb);
-  rp->bytes = rp->pair ? rp->bytes_a + rp->bytes_b : std::max(rp->bytes_a, rp->bytes_b);
-  return true;
-}
-
 // 64 .. 512 rows, leaves of 256: one to four rows of 128x256 tiles need a deep cut of K to occupy the chip, and the pass over
 // that many partial results then weighs as much as a quarter of the GEMM.  Tiles of 128 columns (gemm_tree_quad.hip)
 // occupy it with half the cut.  That kernel is slower per slice than the 128x256-tile kernels, so it is taken only where
@@ -574,6 +549,39 @@ static bool narrow_plan(int M, int N, int K, int leaf_k, bool f16, NarrowPlan* n
   np->flb = flb;
   np->lb = lb - best_ls;
   np->partial_bytes = best > 1 ? (((size_t)best * M * N * sizeof(uint16_t) + 255) & ~(size_t)255) : 0;
+  return true;
+}
+
+// The two column regions of a problem (column_regions): when both run on the same 128x256-tile kernel they go out as
+// ONE launch (the short work-groups of one region fill the CUs that the long ones of the other leave early) and each
+// needs a workspace of its own; otherwise they run one after the other and share it.
+struct RegionPlan {
+  int na;     // columns of the first region; 0: the problem runs in one piece
+  bool pair;  // one launch for both
+  Plan a, b;
+  bool narrow_a, narrow_b;  // the region runs on 128x128 tiles (narrow_plan) instead of plan a / b
+  size_t bytes_a, bytes_b, bytes;
+};
+
+static bool plan_regions(int M, int N, int K, int leaf_k, bool f16, RegionPlan* rp) {
+  rp->na = column_regions(M, N, K, leaf_k, f16);
+  if (!rp->na) return false;
+  if (!make_plan(M, rp->na, K, leaf_k, f16, &rp->a) || !make_plan(M, N - rp->na, K, leaf_k, f16, &rp->b)) {
+    rp->na = 0;
+    return false;
+  }
+  rp->bytes_a = (rp->a.partial_bytes + rp->a.parked_bytes + 255) & ~(size_t)255;
+  rp->bytes_b = (rp->b.partial_bytes + rp->b.parked_bytes + 255) & ~(size_t)255;
+  // a region that qualifies for the 128x128 tiles as a problem of its own takes them (o_proj 32B at M=512: the 1024
+  // columns cut into sixteen become 32 tiles cut into eight)
+  NarrowPlan np;
+  rp->narrow_a = narrow_plan(M, rp->na, K, leaf_k, f16, &np);
+  if (rp->narrow_a) rp->bytes_a = np.partial_bytes;
+  rp->narrow_b = narrow_plan(M, N - rp->na, K, leaf_k, f16, &np);
+  if (rp->narrow_b) rp->bytes_b = np.partial_bytes;
+  rp->pair = !rp->narrow_a && !rp->narrow_b && rp->a.wide && rp->b.wide &&
+             wide_uses_deep_kernel(leaf_k, f16, rp->a.flb, rp->a.lb) == wide_uses_deep_kernel(leaf_k, f16, rp->b.flb, rp->b.lb);
+  rp->bytes = rp->pair ? rp->bytes_a + rp->bytes_b : std::max(rp->bytes_a, rp->bytes_b);
   return true;
 }
 
@@ -675,7 +683,7 @@ static int gemm_dispatch_impl(bool tree, bool f16, const void* A, int64_t lda, c
     }
   }
   NarrowPlan np;
-  if (whole_problem && !rowmajor_b && narrow_plan(M, N, K, leaf_k, f16, &np)) {
+  if (!rowmajor_b && narrow_plan(M, N, K, leaf_k, f16, &np)) {
     if (np.partial_bytes > 0 && (!ws || ws_bytes < np.partial_bytes || !aligned16(ws))) return TBIK_ERR_WORKSPACE;
     WideArgs w{a.X, a.W, a.C, a.bias, nullptr, a.ldx, a.ldw, a.ldc, M, N, K / np.split, np.T, np.flb, np.lb, a.vec_store,
                (int64_t)(K / np.split), 0};
