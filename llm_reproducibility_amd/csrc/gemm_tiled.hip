@@ -509,14 +509,15 @@ static bool make_plan(int M, int N, int K, int leaf_k, bool f16, Plan* pl, bool 
   return true;
 }
 
-// 64 .. 512 rows, leaves of 256: one to four rows of 128x256 tiles need a deep cut of K to occupy the chip, and the pass over
-// that many partial results then weighs as much as a quarter of the GEMM.  Tiles of 128 columns (gemm_tree_quad.hip)
-// occupy it with half the cut.  That kernel is slower per slice than the 128x256-tile kernels, so it is taken only where
-// a shard is short and the grid close to one work-group per CU, the region where a sweep over N = 2048 .. 8192 and
-// K = 2048 .. 16384 at 64 .. 128 rows on MI355X measured it ahead (by 8 % on average, up to 20 %; with fewer rows the
-// 64-row tiles of the tiled kernel win): shards of 512 .. 1024 of K on 160 .. 256
-// work-groups, or up to 1536 on 224 .. 256; with two to four rows of tiles (129 .. 512 rows) only shards of at most 1024 and
-// a cut into at least four (6 % on average there, ahead in every one of 59 shapes, three alternating repetitions each).
+// 64 .. 512 rows, leaves of 256: one to four rows of 128x256 tiles need a deep cut of K to occupy the chip, and the pass
+// over that many partial results then weighs as much as a quarter of the GEMM.  Tiles of 128 columns
+// (gemm_tree_quad.hip) occupy it with half the cut.  That kernel is slower per slice than the 128x256-tile kernels, so it
+// is taken only where a shard is short and the grid close to one work-group per CU, the region where sweeps over
+// N = 1024 .. 8192 and K = 2048 .. 16384 on MI355X measured it ahead:
+//   * 64 .. 128 rows (one row of tiles): shards of 512 .. 1024 of K on 160 .. 256 work-groups, or up to 1536 on
+//     224 .. 256 -- 8 % on average, up to 20 %; with fewer rows the 64-row tiles of the tiled kernel win;
+//   * 129 .. 512 rows (two to four rows of tiles): only shards of at most 1024 and a cut into at least four -- 6 % on
+//     average, ahead in every one of 59 shapes in three alternating repetitions each.
 // The shards are aligned subtrees like every other K split, so the bits do not change.
 struct NarrowPlan {
   int split;
