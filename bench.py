@@ -95,7 +95,13 @@ def ceiling(settle_ms):
     import ctypes
     import torch
     from llm_reproducibility_amd import _lib
-    L = _lib.lib()
+    from llm_reproducibility_amd.build import MEASURE_LIB_PATH
+    if not os.path.exists(MEASURE_LIB_PATH):
+        raise RuntimeError(f"{MEASURE_LIB_PATH} is missing: build it with `python -m llm_reproducibility_amd.build`")
+    L = ctypes.CDLL(MEASURE_LIB_PATH)                      # the machine probes live outside the product library
+    vp = ctypes.c_void_p
+    L.tbik_probe_mfma_bf16.argtypes = [vp, vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp]
+    L.tbik_probe_read.argtypes = [vp, ctypes.c_int64, vp, ctypes.c_int, vp]
     dev = torch.device("cuda:0")
     cus = torch.cuda.get_device_properties(dev).multi_processor_count
     stream = torch.cuda.current_stream().cuda_stream

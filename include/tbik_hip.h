@@ -324,18 +324,6 @@ int bi_qk_norm_rope_cache_bf16(const void* qkv, int64_t ld,
  */
 int bi_argmax_bf16(const void* x, int64_t ld, void* out, int64_t rows, int cols, tbik_stream_t stream);
 
-/*
- * Ceiling probes used by the benchmark (no counterpart in the reference: they measure the machine, not the path).
- *   tbik_probe_mfma_bf16: `work_groups` work-groups (one per CU: each requests 100 KiB of LDS) of `waves` (4 or 8)
- *     wavefronts run iters x 16 v_mfma_f32_16x16x32_bf16 each on register operands taken once from `operands`
- *     (65,536 bytes of bf16, 16-byte aligned); `out` receives work_groups * waves * 64 floats.  Work done:
- *     work_groups * waves * iters * 16 instructions of 16,384 flop.
- *   tbik_probe_read: one grid-stride pass of 16-byte loads over `bytes` of `src` by `work_groups` work-groups of
- *     256 threads; `out` receives work_groups * 256 32-bit words.
- */
-int tbik_probe_mfma_bf16(const void* operands, void* out, int work_groups, int waves, int iters, tbik_stream_t stream);
-int tbik_probe_read(const void* src, int64_t bytes, void* out, int work_groups, tbik_stream_t stream);
-
 #ifdef __cplusplus
 }
 #endif

@@ -1,4 +1,5 @@
-"""Builds libtbik_hip.so (the gfx950 kernels + their C ABI) in-tree with hipcc.
+"""Builds libtbik_hip.so (the gfx950 kernels + their C ABI) in-tree with hipcc, and beside it measure/libtbik_measure.so
+(the benchmark's machine probes, which are not part of the product library).
 
     python -m llm_reproducibility_amd.build            # compile every source, link
     python -m llm_reproducibility_amd.build --if-stale # only when a source is newer than the library
@@ -18,6 +19,8 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 INCLUDE = os.path.join(os.path.dirname(PKG_DIR), "include")
 LIB_PATH = os.path.join(PKG_DIR, "libtbik_hip.so")
+MEASURE_DIR = os.path.join(PKG_DIR, "measure")
+MEASURE_LIB_PATH = os.path.join(MEASURE_DIR, "libtbik_measure.so")
 OBJ_DIR = os.path.join(PKG_DIR, "build")
 
 # -packed-fp32-ops: keep the compiler from forming packed fp32 VALU ops out of scalar float code.
@@ -45,16 +48,20 @@ def sources():
     return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
 
 
+def measure_sources():
+    return sorted(os.path.join(MEASURE_DIR, f) for f in os.listdir(MEASURE_DIR) if f.endswith(".hip"))
+
+
 def _deps():
-    deps = sources() + [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")]
-    deps.append(os.path.join(INCLUDE, "tbik_hip.h"))
+    deps = sources() + measure_sources() + [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")]
+    deps += [os.path.join(INCLUDE, "tbik_hip.h"), os.path.join(INCLUDE, "tbik_measure.h")]
     return deps
 
 
 def is_stale() -> bool:
-    if not os.path.exists(LIB_PATH):
+    if not os.path.exists(LIB_PATH) or not os.path.exists(MEASURE_LIB_PATH):
         return True
-    t = os.path.getmtime(LIB_PATH)
+    t = min(os.path.getmtime(LIB_PATH), os.path.getmtime(MEASURE_LIB_PATH))
     return any(os.path.getmtime(d) > t for d in _deps())
 
 
@@ -74,19 +81,24 @@ def _compile(src: str) -> str:
     return obj
 
 
-def build(verbose: bool = True) -> str:
-    os.makedirs(OBJ_DIR, exist_ok=True)
-    srcs = sources()
-    with cf.ThreadPoolExecutor(max_workers=min(8, len(srcs))) as ex:
-        objs = list(ex.map(_compile, srcs))
-    tmp = LIB_PATH + ".tmp"
+def _link(objs, path: str) -> None:
+    tmp = path + ".tmp"
     cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", "-o", tmp, *objs]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"link failed:\n{r.stdout}\n{r.stderr}")
-    os.replace(tmp, LIB_PATH)
+    os.replace(tmp, path)
+
+
+def build(verbose: bool = True) -> str:
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    srcs, msrcs = sources(), measure_sources()
+    with cf.ThreadPoolExecutor(max_workers=min(8, len(srcs) + len(msrcs))) as ex:
+        objs = list(ex.map(_compile, srcs + msrcs))
+    _link(objs[:len(srcs)], LIB_PATH)
+    _link(objs[len(srcs):], MEASURE_LIB_PATH)
     if verbose:
-        print(f"built {LIB_PATH} from {len(srcs)} sources")
+        print(f"built {LIB_PATH} from {len(srcs)} sources and {MEASURE_LIB_PATH} from {len(msrcs)}")
     return LIB_PATH
 
 

@@ -27,13 +27,11 @@ int qk_norm_rope_cache_dispatch(const void* qkv, int64_t ld, const void* q_weigh
                                 int max_len, int batch, float eps, hipStream_t stream);
 int silu_mul_dispatch(const void* gate_up, int64_t ld_in, void* out, int64_t ld_out, int64_t rows, int inter, bool f16,
                       hipStream_t stream);
-int probe_mfma_dispatch(const void* operands, void* out, int work_groups, int waves, int iters, hipStream_t stream);
-int probe_read_dispatch(const void* src, int64_t bytes, void* out, int work_groups, hipStream_t stream);
 }  // namespace tbik
 
 extern "C" {
 
-int tbik_abi_version(void) { return 10; }
+int tbik_abi_version(void) { return 11; }
 
 const char* tbik_error_string(int code) {
   switch (code) {
@@ -176,14 +174,6 @@ int bi_qk_norm_rope_cache_bf16(const void* qkv, int64_t ld, const void* q_weight
 
 int bi_argmax_bf16(const void* x, int64_t ld, void* out, int64_t rows, int cols, tbik_stream_t stream) {
   return tbik::argmax_dispatch(x, ld, out, rows, cols, static_cast<hipStream_t>(stream));
-}
-
-int tbik_probe_mfma_bf16(const void* operands, void* out, int work_groups, int waves, int iters, tbik_stream_t stream) {
-  return tbik::probe_mfma_dispatch(operands, out, work_groups, waves, iters, static_cast<hipStream_t>(stream));
-}
-
-int tbik_probe_read(const void* src, int64_t bytes, void* out, int work_groups, tbik_stream_t stream) {
-  return tbik::probe_read_dispatch(src, bytes, out, work_groups, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

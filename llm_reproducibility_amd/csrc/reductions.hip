@@ -263,14 +263,13 @@ __device__ __forceinline__ float seg_thread_max(const float (&v)[4][4]) {
   return m;
 }
 __device__ __forceinline__ float seg_thread_expsum(const float (&v)[4][4], float m) {
-  // exp(x - m) = 2^(x * log2 e - m * log2 e): one fused multiply-add and the hardware exponential per element
-  constexpr float kLog2e = 1.44269504088896340736f;
-  const float ml = m * kLog2e;
+  // exp(x - m) = 2^((x - m) * log2 e): the difference is formed first (exact near the maximum, where the terms that
+  // matter are), so a common offset of the logits does not enter the rounding; then the hardware exponential
   float s = 0.f;
 #pragma unroll
   for (int i = 0; i < 4; i++)
 #pragma unroll
-    for (int j = 0; j < 4; j++) s += __builtin_amdgcn_exp2f(__builtin_fmaf(v[i][j], kLog2e, -ml));  // 2^(-inf) = 0 for the padding
+    for (int j = 0; j < 4; j++) s += fast_exp(v[i][j] - m);  // 2^(-inf) = 0 for the padding
   return s;
 }
 

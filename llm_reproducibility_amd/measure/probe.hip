@@ -2,7 +2,10 @@
 // kernel on given operand data, below the nominal peak because the chip is power limited) and on a plain one-pass
 // read of a buffer (the ceiling of the bandwidth-bound kernels).  They have no counterpart in the reference; they
 // exist so that a roofline fraction can be read against a measured ceiling as well as against the published peak.
-#include "common.h"
+// They measure the machine, not the path: built into libtbik_measure.so, a library of its own that only the
+// benchmark loads (declared in include/tbik_measure.h), and absent from libtbik_hip.so and its header.
+#include "../csrc/common.h"
+#include "../../include/tbik_measure.h"
 
 namespace tbik {
 
@@ -65,3 +68,15 @@ int probe_read_dispatch(const void* src, int64_t bytes, void* out, int work_grou
 }
 
 }  // namespace tbik
+
+extern "C" {
+
+int tbik_probe_mfma_bf16(const void* operands, void* out, int work_groups, int waves, int iters, void* stream) {
+  return tbik::probe_mfma_dispatch(operands, out, work_groups, waves, iters, static_cast<hipStream_t>(stream));
+}
+
+int tbik_probe_read(const void* src, int64_t bytes, void* out, int work_groups, void* stream) {
+  return tbik::probe_read_dispatch(src, bytes, out, work_groups, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

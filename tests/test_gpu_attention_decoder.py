@@ -88,6 +88,75 @@ def test_attention_matches_fp32_reference_and_is_batch_and_phase_invariant(dev):
         assert torch.equal(oa, ob), (hq, hkv)
 
 
+def _oracle_heads(q, k, v, heads, rep, scale):
+    """O.causal_attention for a subset of query heads (each with its own KV head), as [n, len(heads), D]."""
+    outs = []
+    for h in heads:
+        kv = h // rep
+        outs.append(O.causal_attention(q[:, h:h + 1], k[:, kv:kv + 1], v[:, kv:kv + 1], scale))
+    return torch.cat(outs, dim=1)
+
+
+def test_attention_matches_the_oracle_at_the_decoder_configuration(dev):
+    """32 query heads over 8 KV heads of 128 channels (the grouped kernel with four waves per KV head), contexts of
+    512-768 keys and one of 2304 (72 key tiles: the prefetch ring of the decode kernel wraps 18 times), prefill,
+    chunked prefill and decode, against the float64 oracle; stated tolerance: within 1 bf16 ulp OR within 2^-8 of the
+    output scale.  The one-wave-per-head kernel (a cache length that is not a whole number of tiles) must give the
+    same bits."""
+    torch.manual_seed(4)
+    Hq, Hkv, D, scale = 32, 8, 128, 1.0 / math.sqrt(128)
+    rep = Hq // Hkv
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)  # noqa: E731
+    rnd = lambda *shape: torch.randn(shape, device=dev).to(torch.bfloat16)  # noqa: E731
+
+    def check(got, q, k, v, heads, what):
+        want = _oracle_heads(q.cpu(), k.cpu(), v.cpu(), heads, rep, scale).to(torch.bfloat16)
+        bad = O.outside_tolerance(got[:, heads].cpu(), want)
+        assert not bad.any(), (what, int(bad.sum()), O.bf16_ulp_distance(got[:, heads].cpu(), want).max().item())
+
+    # ---- prefill of a ragged batch at 512 / 300 / 512 tokens: every head of the first sequence, one head of each
+    # position inside a KV group for the others
+    lens = [512, 300, 512]
+    ks, vs, qs = [rnd(n, Hkv, D) for n in lens], [rnd(n, Hkv, D) for n in lens], [rnd(n, Hq, D) for n in lens]
+    starts = [0, 512, 812]
+    kc, vt = _make_cache(ks, vs, 768, dev)
+    print("case prefill 32/8 heads", lens, flush=True)
+    out = ops.bi_attention_bf16(torch.cat(qs), kc, vt, i32(starts), i32(lens), i32(lens), 512, scale)
+    check(out[:512], qs[0], ks[0], vs[0], list(range(Hq)), "prefill seq 0")
+    check(out[512:812], qs[1], ks[1], vs[1], [0, 5, 14, 31], "prefill seq 1")
+    check(out[812:], qs[2], ks[2], vs[2], [3, 9, 22, 28], "prefill seq 2")
+    kc2, vt2 = _make_cache(ks, vs, 772, dev)
+    assert torch.equal(ops.bi_attention_bf16(torch.cat(qs), kc2, vt2, i32(starts), i32(lens), i32(lens), 512, scale), out)
+
+    # ---- decode at contexts 768 / 768 / 700 / 513: the caches above grown by random keys, one query each
+    ctx = [768, 768, 700, 513]
+    kd, vd, qd = [rnd(n, Hkv, D) for n in ctx], [rnd(n, Hkv, D) for n in ctx], [rnd(1, Hq, D) for _ in ctx]
+    kc, vt = _make_cache(kd, vd, 768, dev)
+    print("case decode 32/8 heads", ctx, flush=True)
+    dec = ops.bi_attention_bf16(torch.cat(qd), kc, vt, i32([0, 1, 2, 3]), i32([1] * 4), i32(ctx), 1, scale)
+    for b in range(4):
+        check(dec[b:b + 1], qd[b], kd[b], vd[b], list(range(Hq)), f"decode seq {b}")
+    kc2, vt2 = _make_cache(kd, vd, 780, dev)
+    assert torch.equal(ops.bi_attention_bf16(torch.cat(qd), kc2, vt2, i32([0, 1, 2, 3]), i32([1] * 4), i32(ctx), 1, scale), dec)
+
+    # ---- a long context: 2304 keys; decode (all heads), a chunk of 40 new tokens (all heads), and the whole prefill
+    # on four heads (one per position inside a KV group)
+    L = 2304
+    k1, v1, q1 = rnd(L, Hkv, D), rnd(L, Hkv, D), rnd(L, Hq, D)
+    kc, vt = _make_cache([k1], [v1], L, dev)
+    print("case long context", L, flush=True)
+    full = ops.bi_attention_bf16(q1, kc, vt, i32([0]), i32([L]), i32([L]), L, scale)
+    check(full, q1, k1, v1, [1, 6, 19, 28], "prefill 2304")
+    one = ops.bi_attention_bf16(q1[-1:], kc, vt, i32([0]), i32([1]), i32([L]), 1, scale)
+    check(one, q1[-1:], k1, v1, list(range(Hq)), "decode 2304")
+    assert torch.equal(one[0], full[-1])
+    chunk = ops.bi_attention_bf16(q1[-40:], kc, vt, i32([0]), i32([40]), i32([L]), 40, scale)
+    check(chunk, q1[-40:], k1, v1, list(range(Hq)), "chunk of 40 at 2304")
+    assert torch.equal(chunk, full[-40:])
+    kc2, vt2 = _make_cache([k1], [v1], L + 4, dev)
+    assert torch.equal(ops.bi_attention_bf16(q1[-40:], kc2, vt2, i32([0]), i32([40]), i32([L]), 40, scale), chunk)
+
+
 SMALL = DecoderConfig(vocab_size=3000, hidden_size=1024, num_layers=2, num_q_heads=16, num_kv_heads=4, head_dim=128,
                       intermediate_size=4096)
 

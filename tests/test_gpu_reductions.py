@@ -34,6 +34,23 @@ def test_rmsnorm_parity_and_batch_invariance(dev):
     assert torch.equal(bio.rms_norm(s.to(dev), torch.ones(4096, dtype=torch.bfloat16, device=dev), 1e-6).cpu(), s)
 
 
+def test_rmsnorm_rounding_points_on_an_exact_case(dev):
+    """The case of tests/test_oracle_reductions.py whose normalisation factor is exactly 1/3 (integer squares: the
+    sum is exact in any order), so the kernel has to give the bits of exact rational arithmetic with the documented
+    rounding points -- the normalised value rounded to bf16 BEFORE the bf16 multiply by the weight -- and not those of a
+    single rounding after an fp32 multiply."""
+    from test_oracle_reductions import rounding_point_case
+    x, w, two_roundings, one_rounding = rounding_point_case()
+    got = bio.rms_norm(x.to(dev), w.to(dev), 0.0).cpu()
+    assert torch.equal(got, two_roundings)
+    assert (got != one_rounding).sum() > 100
+    half = (x.float() / 2).to(torch.bfloat16)
+    y, new_res = bio.rms_norm(half.to(dev), w.to(dev), 0.0, residual=half.to(dev))
+    assert torch.equal(new_res.cpu(), x) and torch.equal(y.cpu(), two_roundings)
+    rows = x.repeat(300, 1)
+    assert torch.equal(bio.rms_norm(rows.to(dev), w.to(dev), 0.0).cpu(), two_roundings.repeat(300, 1))
+
+
 def test_fp16_rmsnorm_and_silu_mul(dev):
     from llm_reproducibility_amd import ops
     x = O.gaussian_bf16((300, 4096), 1.0, 0).to(torch.float16)
@@ -101,6 +118,43 @@ def test_log_softmax_parity_and_batch_invariance(dev):
     # bf16 input keeps its dtype
     yb = torch.randn((4, 512), generator=g).to(torch.bfloat16)
     assert bio.log_softmax(yb.to(dev)).dtype == torch.bfloat16
+
+
+def test_log_softmax_4096_distinct_rows_against_fp64(dev):
+    """The largest reduction of the benchmark configuration with every row different: 4096 x 151936 fp32 logits
+    drawn on the GPU (2.5 GB), float64 parity on 64 rows spread over the whole batch (first, last, and a stride that
+    is odd so that every XCD's share of the rows is sampled), and those rows alone / in small batches bit for bit."""
+    V, R = 151936, 4096
+    g = torch.Generator(device=dev).manual_seed(11)
+    x = torch.randn((R, V), generator=g, device=dev) * 3.0
+    out = bio.log_softmax(x)
+    pick = sorted(set([0, 1, R - 2, R - 1] + [(61 * i + 17) % R for i in range(60)]))
+    idx = torch.tensor(pick, device=dev)
+    want = torch.log_softmax(x[idx].cpu().double(), dim=-1)
+    got = out[idx].cpu().double()
+    assert (got - want).abs().max() < 2e-5, (got - want).abs().max()
+    assert not torch.equal(out[0], out[1])
+    for r in (0, 777, R - 1):                                        # a row alone (two-launch schedule)
+        assert torch.equal(bio.log_softmax(x[r:r + 1]), out[r:r + 1]), r
+    assert torch.equal(bio.log_softmax(x[2000:2007]), out[2000:2007])
+    assert torch.equal(bio.log_softmax(x[1024:1280]), out[1024:1280])   # 256 rows: the resident schedule again
+    del x, out
+    torch.cuda.empty_cache()
+
+
+def test_log_softmax_of_offset_logits(dev):
+    """log_softmax(x + c) = log_softmax(x): with the difference to the maximum formed before the scaling by log2(e) a
+    common offset costs only the rounding of x + c itself.  Logits around +1000 and -1e4 against float64 of the same
+    fp32 values; the tolerance is that of the unshifted test (2e-5) -- a kernel that folds max * log2(e) into a fused
+    multiply-add is off by 3e-4 at |max| = 1e4."""
+    g = torch.Generator().manual_seed(12)
+    base = torch.randn((200, 151936), generator=g) * 3.0
+    for shift in (1000.0, -1.0e4):
+        x = base + shift                                             # rounded to fp32 here, on both sides alike
+        got = bio.log_softmax(x.to(dev))
+        want = torch.log_softmax(x[:8].double(), dim=-1)
+        assert (got[:8].cpu().double() - want).abs().max() < 2e-5, (shift, (got[:8].cpu().double() - want).abs().max())
+        assert torch.equal(bio.log_softmax(x[:3].to(dev)), got[:3]), shift      # both schedules
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])

@@ -366,6 +366,26 @@ def test_headline_shape_matches_the_oracle_at_full_size(dev):
     assert_bitwise(matmul_tp_persistent(Xi.to(dev), Wi.to(dev).t()), O.matmul_tree(Xi, Wi.t()), "headline, integer inputs")
 
 
+@pytest.mark.parametrize("name,M,K,N,leaf", [
+    ("o_proj 32B", 4096, 8192, 5120, 256),
+    ("down_proj 32B", 4096, 25600, 5120, 128),
+    ("down_proj 32B mid-sized batch", 512, 25600, 5120, 128),
+])
+def test_qwen3_32b_shapes_match_the_oracle_bit_for_bit_at_full_size(dev, name, M, K, N, leaf):
+    """The row-split layers of the 32B configuration at their full sizes on integer-valued inputs (every leaf sum an
+    exact integer in fp32 whatever the order inside the leaf, so only the tree order and the bf16 roundings decide the
+    bits): K = 8192 is a tree of 32 leaves in groups of two, K = 25600 with leaves of 128 a tree of 200 leaves in
+    groups of 25 under three binary levels (src/tbik/tree_based_matmul.py:242-249 with the leaf of the layer)."""
+    assert O.tree_params(K, leaf)[1:] == ((2, 5) if K == 8192 else (25, 4))
+    Xi = O.integer_bf16((M, K), -9, 9, 15)
+    Wi = O.integer_bf16((N, K), -7, 7, 16)
+    print("case", name, M, K, N, leaf, flush=True)
+    got = matmul_tp_persistent(Xi.to(dev), Wi.to(dev).t(), leaf_k=leaf).cpu()
+    want = O.matmul_tree(Xi, Wi.t(), leaf=leaf)
+    assert_bitwise(got, want, name)
+    assert want.float().abs().max() > 2048          # sums far beyond the 8 significant bits: the roundings matter
+
+
 def test_invariance_qwen3_32b_o_proj(dev):
     _invariance(dev, 8192, 5120, (1, 64, 512), "gauss", 4096)
 
@@ -534,3 +554,17 @@ def test_fp32_rational_known_answers_and_invariance(dev):
         assert torch.equal(tree_combine(parts), nb), f"fp32 TP={p}"
     for m in (1, 17, 64):
         assert torch.equal(matmul_tp_persistent(X[:m], W.t(), bias), full[:m]), f"fp32 rows {m}"
+
+
+def test_invariance_check_module_honours_the_flag(dev, monkeypatch):
+    """`python -m llm_reproducibility_amd.check_matmul`: with TP_INVARIANT_MATMUL=1 both differences are exactly zero
+    on the reference's smoke-test shape (simple_matmul.py:6) and on other shard counts; with the flag off the product
+    is the vendor library's and the check still runs."""
+    from llm_reproducibility_amd import check_matmul
+    monkeypatch.setenv("TP_INVARIANT_MATMUL", "1")
+    for shards in (2, 4, 8):
+        assert check_matmul.run(1024, 6144, 2048, shards) == ("matmul_tp_persistent", 0.0, 0.0), shards
+    assert check_matmul.main(["--m", "256", "--k", "4096", "--n", "512", "--shards", "8"]) == 0
+    monkeypatch.setenv("TP_INVARIANT_MATMUL", "0")
+    name, batch_diff, shard_diff = check_matmul.run(1024, 6144, 2048, 4)
+    assert name == "torch.matmul" and batch_diff >= 0.0 and shard_diff >= 0.0

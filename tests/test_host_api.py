@@ -85,6 +85,28 @@ def test_env_flags(monkeypatch):
     assert utils.tp_invariant_matmul_is_enabled()
 
 
+def test_tp_invariant_matmul_flag_selects_the_product(monkeypatch):
+    """TP_INVARIANT_MATMUL picks the product of the invariance check (the switch of the reference's smoke script,
+    simple_matmul.py:8,14): off -> torch.matmul, on -> matmul_tp_persistent."""
+    from llm_reproducibility_amd import check_matmul
+    f, name = check_matmul.select_matmul()
+    assert f is torch.matmul and name == "torch.matmul"
+    monkeypatch.setenv("TP_INVARIANT_MATMUL", "1")
+    f, name = check_matmul.select_matmul()
+    assert f is matmul_tp_persistent and name == "matmul_tp_persistent"
+    # the pairwise tree of the check: ((p0 + p1) + (p2 + p3)) with every add rounded to the parts' type -- on values
+    # where a left-to-right sum rounds differently
+    parts = [torch.tensor([v], dtype=torch.bfloat16) for v in (256.0, 1.0, 1.0, 1.0)]
+    assert check_matmul.pairwise_tree_sum(parts).item() == 258.0      # (256+1 -> 256) + (1+1) = 258
+    assert (((parts[0] + parts[1]) + parts[2]) + parts[3]).item() == 256.0
+    with pytest.raises(ValueError):
+        check_matmul.pairwise_tree_sum(parts[:3])
+    # run on the CPU with the library product: the check itself works without a GPU (and without the kernels)
+    monkeypatch.setenv("TP_INVARIANT_MATMUL", "0")
+    name, batch_diff, shard_diff = check_matmul.run(64, 512, 32, 4, device="cpu", dtype=torch.float32)
+    assert name == "torch.matmul" and batch_diff >= 0.0 and 0.0 <= shard_diff < 1e-3
+
+
 def test_apply_patches_dispatch(monkeypatch, capsys):
     from llm_reproducibility_amd import layers, patch
     from llm_reproducibility_amd.bio import batch_invariant_ops as bio

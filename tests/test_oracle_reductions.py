@@ -89,6 +89,38 @@ def _rne_bf16(x: Fraction) -> float:
     return float(sign * Fraction(n) * Fraction(2) ** e)
 
 
+def rounding_point_case():
+    """A row whose normalisation is exact rational arithmetic: the pattern (1,2,3,4,5,6,7,2,0 x 8) has mean(x^2) = 9,
+    so with eps = 0 the factor is exactly 1/3; repeated 128 times, with column block b weighted by the bf16 value
+    1 + b/128 (every bf16 in [1, 2)).  Returns x [1, 2048], w [2048] and, from exact fractions with an independent
+    round-to-nearest-even, the result of (a) rounding x/3 to bf16 and then multiplying by w in bf16 -- the documented
+    order, vLLM's `x.to(orig_dtype) * weight` -- and (b) multiplying in full precision and rounding once."""
+    pat = [1, 2, 3, 4, 5, 6, 7, 2] + [0] * 8
+    x = torch.tensor([pat * 128], dtype=torch.float32).to(torch.bfloat16)
+    w = torch.tensor([1.0 + b / 128.0 for b in range(128) for _ in range(16)], dtype=torch.float32).to(torch.bfloat16)
+    two, one = [], []
+    for b in range(128):
+        wb = Fraction(128 + b, 128)
+        for v in pat:
+            two.append(_rne_bf16(Fraction(_rne_bf16(Fraction(v, 3))) * wb))
+            one.append(_rne_bf16(Fraction(v, 3) * wb))
+    as_bf16 = lambda vals: torch.tensor([vals], dtype=torch.float64).to(torch.bfloat16)  # noqa: E731  (exact: already bf16 values)
+    return x, w, as_bf16(two), as_bf16(one)
+
+
+def test_rmsnorm_rounds_to_the_input_type_before_the_weight_multiply():
+    x, w, two_roundings, one_rounding = rounding_point_case()
+    differ = (two_roundings != one_rounding).sum().item()
+    assert differ > 100, differ                       # the case separates the two orders on many elements
+    got = O.rmsnorm(x, w, 0.0)
+    assert torch.equal(got, two_roundings)
+    assert not torch.equal(got, one_rounding)
+    # the same with a residual: x = r = half the pattern, so the fp32 sum is the pattern again, and a NON-unit weight
+    half = (x.float() / 2).to(torch.bfloat16)
+    y, new_res = O.rmsnorm(half, w, 0.0, residual=half)
+    assert torch.equal(new_res, x) and torch.equal(y, two_roundings)
+
+
 def test_single_accumulator_matmul_against_exact_rational_arithmetic():
     # integer operands: every product and every partial sum is an integer below 2^24, so an fp32 accumulator is exact
     # in ANY order and the result is one rounding of the exact sum (+ bias); sums reach the thousands, so an
