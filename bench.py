@@ -1,12 +1,17 @@
 """Benchmark of the TBIK hot path on ONE MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--table]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--table] [--ceiling]
 
 A step is one tree-ordered matmul (`matmul_tp_persistent`) over the headline batch: X[2048,12288]
 (SiLU-gated synthetic activations, bf16) times the down_proj weight W[4096,12288] (N(0,0.02), bf16,
 stored [N,K] as nn.Linear does), inputs resident in HBM before the timed region.  Prints ONE JSON line.
-`--table` additionally prints (to stderr) the other shapes of the workload family: decode-sized M,
-simulated TP shards + combine, and the batch-invariant reductions.
+
+Order of a run: the step is timed twice -- right after the host-side set-up (`value_after_idle`: W warm-up steps, K
+timed steps, nothing else) and after `--settle-ms` of the same step run back to back (`value`: the settled rate);
+then the context figures (the vendor library and this library's plain mm on the same operands, and `context.table`:
+the other shapes of the workload family, each with its algorithmic flops or bytes and the fraction of the stated
+peak); the CPU baseline and the full-size parity check against it come last, so that they do not sit between the
+set-up and the timed region.  `--table` prints the long form of the table to stderr as well.
 """
 import argparse
 import json
@@ -43,8 +48,8 @@ def hip_time_ms(fn, steps, warmup, settle_ms=0.0):
 
     settle_ms > 0: the same call is first repeated for about that long.  After an idle period the chip's power
     management takes some 25 ms of continuous load to settle: the first ten headline launches run at 225 us, the next
-    ten at 270-280 us, and only after about a hundred the rate is steady (210-215 us).  A benchmark of a handful of
-    steps taken right after the host-side set-up would measure that transient, not the kernel."""
+    ten at 270-280 us, and only after about a hundred the rate is steady.  A handful of steps taken right after the
+    host-side set-up measures that transient, not the kernel."""
     import torch
     if settle_ms > 0:
         t_end = time.perf_counter() + settle_ms * 1e-3
@@ -66,26 +71,50 @@ def hip_time_ms(fn, steps, warmup, settle_ms=0.0):
     return s.elapsed_time(e) / steps, wall_ms / steps
 
 
-def cpu_baseline(budget_s=12.0, max_runs=30):
-    """The CPU oracle (PyTorch restatement of the reference's tree order) on the whole headline workload, all host
-    threads: one warm-up, then repeated until about `budget_s` seconds of CPU work are spent; the median is reported."""
+def _median_time(fn, budget_s, max_runs, min_runs=3):
+    ts, spent = [], 0.0
+    while (spent < budget_s or len(ts) < min_runs) and len(ts) < max_runs:
+        t0 = time.perf_counter()
+        fn()
+        ts.append(time.perf_counter() - t0)
+        spent += ts[-1]
+    return statistics.median(ts), len(ts), spent
+
+
+def cpu_baseline(budget_s=9.0, max_runs=30):
+    """The CPU oracle (PyTorch restatement of the reference's tree order, the reference has no CPU path of its own) on
+    the whole headline workload, all host threads: one warm-up, then repeated for about `budget_s` seconds, median.
+    Beside it, bounded to a few seconds in all: the oracle on configuration 1 (A[256,4096] x W[4096,4096]) as a whole
+    and cut into 2 / 4 / 8 shards with the shard tree, and the CPU library's plain bf16 `torch.matmul` on both shapes
+    (order not fixed, no tree) for context.  Returns (record, oracle product of the headline workload)."""
     import torch
     from oracle import tbik_oracle as O
     X = O.silu_gated_bf16((M_, K_), 0)
     W = O.gaussian_bf16((N_, K_), 0.02, 1)
     Wt = W.t()
     O.matmul_tree(X[:256], Wt)
-    ts, spent = [], 0.0
-    while spent < budget_s and len(ts) < max_runs:
-        t0 = time.perf_counter()
-        O.matmul_tree(X, Wt)
-        ts.append(time.perf_counter() - t0)
-        spent += ts[-1]
-    t = statistics.median(ts)
-    return {"value": round(2.0 * M_ * N_ * K_ / t / 1e12, 4), "unit": "TFLOP/s", "cores": torch.get_num_threads(),
-            "kind": "port",
-            "sample": f"oracle matmul_tree on the full X[{M_},{K_}] and W[{N_},{K_}] of the headline workload, "
-                      f"{len(ts)} runs in {spent:.1f} s, median {t:.2f} s each"}, O.matmul_tree(X, Wt)
+    t, n, spent = _median_time(lambda: O.matmul_tree(X, Wt), budget_s, max_runs)
+    rec = {"value": round(2.0 * M_ * N_ * K_ / t / 1e12, 4), "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+           "kind": "port",
+           "sample": f"oracle matmul_tree on the full X[{M_},{K_}] and W[{N_},{K_}] of the headline workload, "
+                     f"{n} runs in {spent:.1f} s, median {t:.2f} s each"}
+    want = O.matmul_tree(X, Wt)
+    A1 = O.gaussian_bf16((256, 4096), 1.0, 0)
+    W1 = O.gaussian_bf16((4096, 4096), 0.02, 1).t()
+    fl1 = 2.0 * 256 * 4096 * 4096
+    c1 = {}
+    for p in (1, 2, 4, 8):
+        tp, _, _ = _median_time(lambda p=p: O.simulated_tp_matmul(A1, W1, p), 0.5, 10)
+        c1[f"tp{p}_ms"] = round(tp * 1e3, 2)
+    rec["config1_oracle_A256x4096_W4096x4096"] = dict(c1, GFLOPs_tp1=round(fl1 / (c1["tp1_ms"] * 1e-3) / 1e9, 1),
+                                                      note="oracle per shard + shard tree, median")
+    tm1, _, _ = _median_time(lambda: torch.matmul(A1, W1), 0.5, 10)
+    tmh, _, _ = _median_time(lambda: torch.matmul(X, Wt), 2.0, 5, min_runs=2)
+    rec["plain_cpu_torch_matmul_bf16"] = {"config1_ms": round(tm1 * 1e3, 2), "config1_GFLOPs": round(fl1 / tm1 / 1e9, 1),
+                                          "headline_s": round(tmh, 3),
+                                          "headline_TFLOPs": round(2.0 * M_ * N_ * K_ / tmh / 1e12, 4),
+                                          "note": "CPU library matmul, bf16, order not fixed, no tree"}
+    return rec, want
 
 
 def ceiling(settle_ms):
@@ -107,7 +136,7 @@ def ceiling(settle_ms):
     stream = torch.cuda.current_stream().cuda_stream
     out = torch.empty(cus * 512, device=dev, dtype=torch.float32)
     res = {"work_groups": cus}
-    iters = 800        # 800 x 16 MFMAs x 2 waves per SIMD = the MFMA count of one headline launch per SIMD on 256 CUs
+    iters = 800
     g = torch.Generator().manual_seed(0)
     ops_rand = torch.randn(32768, generator=g)
     ops_rand[:16384] *= 0.02                      # a operands like the weights, b operands like the activations
@@ -132,13 +161,21 @@ def ceiling(settle_ms):
     return res
 
 
-def table(steps, warmup, hot=False, settle_ms=20.0):
+def table(steps, warmup, hot=False, settle_ms=20.0, full=False):
     """Per-shape figures, each after `settle_ms` of the same call run back to back (the settled rate, as for the
-    headline).  Unless `hot`, every case cycles through enough distinct input sets (more than 768 MB in
-    all) that nothing it reads is still in the 256 MB memory-side cache from the previous call: the GB/s are HBM
-    figures, as in a model whose every layer has its own weights."""
+    headline).  Unless `hot`, every case cycles through enough distinct input sets (more than 768 MB in all) that
+    nothing it reads is still in the 256 MB memory-side cache from the previous call: the GB/s are HBM figures, as in
+    a model whose every layer has its own weights.
+
+    Returns a list of rows {case, us, flop, bytes, TFLOPs, GBps, bound, frac}: `flop` and `bytes` are the algorithmic
+    work of one call -- 2*M*N*K and 2*(M*K + K*N + M*N) for a matmul, the formulas of the reference's launch metadata
+    (src/tbik/tree_based_matmul.py:23-24, src/bio/batch_invariant_ops.py:13-29); (p+1)*M*N*2 for the shard combine;
+    rows*hidden*4 + hidden*2 for RMSNorm; 8 B per logit for the fp32 log_softmax; 4 B per element for the mean; K, V, q
+    and the output once for attention -- `bound` names the roofline that applies to the case ("mfma": 2.5 PFLOP/s
+    dense bf16, "hbm": 8 TB/s) and `frac` is the achieved share of it.  `full` adds the long list (vendor-library rows for
+    context, the mm shapes of the decoder, prefill attention)."""
     import torch
-    from oracle import tbik_oracle as O
+    from llm_reproducibility_amd import ops
     from llm_reproducibility_amd.bio import batch_invariant_ops as bio
     from llm_reproducibility_amd.tbik import choose_leaf_k, matmul_tp_persistent, tree_combine
     dev = torch.device("cuda:0")
@@ -155,83 +192,81 @@ def table(steps, warmup, hot=False, settle_ms=20.0):
             return fn(*args)
         return call
 
-    def gemm_row(name, M, K, N, leaf):
-        def make():
-            return (torch.randn((M, K), device=dev).to(torch.bfloat16), (torch.randn((N, K), device=dev) * 0.02).to(torch.bfloat16))
-        fl, by = 2.0 * M * N * K, 2.0 * (M * K + K * N + M * N)
-        ms, _ = hip_time_ms(cycling(make, by, lambda X, W: matmul_tp_persistent(X, W.t(), leaf_k=leaf)), steps, warmup, settle_ms)
-        rows.append((name, ms * 1e3, fl / ms / 1e9, by / ms / 1e6))
+    def add(name, make, fn, flop, nbytes, bound, nsteps=None, short=None):
+        """`short`: the key of the row in the JSON line; rows without one appear in the long form only."""
+        if short is None and not full:
+            return
+        ms, _ = hip_time_ms(cycling(make, nbytes, fn), nsteps or steps, warmup, settle_ms)
+        tf, gbs = flop / ms / 1e9, nbytes / ms / 1e6
+        frac = tf / PEAK_BF16_TFLOPS if bound == "mfma" else gbs / PEAK_HBM_GBS
+        rows.append({"case": name, "short": short, "us": round(ms * 1e3, 1), "flop": flop, "bytes": nbytes,
+                     "TFLOPs": round(tf, 1), "GBps": round(gbs, 1), "bound": bound, "frac": round(frac, 4)})
 
-    for M in (1, 16, 128, 2048):
-        gemm_row(f"down_proj 8B  M={M} K=12288 N=4096", M, 12288, 4096, 256)
+    def operands(M, K, N):
+        return lambda: (torch.randn((M, K), device=dev).to(torch.bfloat16), (torch.randn((N, K), device=dev) * 0.02).to(torch.bfloat16))
+
+    def gemm_row(name, M, K, N, leaf, fn=None, short=None):
+        fl, by = 2.0 * M * N * K, 2.0 * (M * K + K * N + M * N)
+        f = fn or (lambda X, W: matmul_tp_persistent(X, W.t(), leaf_k=leaf))
+        # decode-sized batches stream the weights once (memory bound); from a few hundred rows on the matrix cores bound
+        add(name, operands(M, K, N), f, fl, by, "hbm" if fl / by < 312 else "mfma", short=short)
+
     def library_row(M, K, N):
         # context only: the vendor library GEMM behind torch.matmul (no tree, reduction order not fixed) on like operands
-        def make():
-            return (torch.randn((M, K), device=dev).to(torch.bfloat16), (torch.randn((N, K), device=dev) * 0.02).to(torch.bfloat16))
-        fl, by = 2.0 * M * N * K, 2.0 * (M * K + K * N + M * N)
-        ms, _ = hip_time_ms(cycling(make, by, lambda X, W: torch.matmul(X, W.t())), steps, warmup, settle_ms)
-        rows.append((f"  [torch.matmul, not invariant] M={M} K={K} N={N}", ms * 1e3, fl / ms / 1e9, by / ms / 1e6))
+        gemm_row(f"  [torch.matmul, not invariant] M={M} K={K} N={N}", M, K, N, 0, lambda X, W: torch.matmul(X, W.t()))
 
+    for M in (1, 16, 128, 2048):
+        gemm_row(f"tree matmul down_proj 8B M={M} K=12288 N=4096", M, 12288, 4096, 256, short=None if M == 2048 else f"tree dn8B M={M}")
     for M in (1, 128, 2048):
         library_row(M, 12288, 4096)
     for p in (2, 4, 8):
-        gemm_row(f"  shard TP={p}  M=2048 K={12288 // p} N=4096", 2048, 12288 // p, 4096, 256)
+        gemm_row(f"tree matmul shard TP={p} M=2048 K={12288 // p} N=4096", 2048, 12288 // p, 4096, 256)
     for M in (1, 64, 512, 4096):
-        gemm_row(f"o_proj 32B    M={M} K=8192 N=5120", M, 8192, 5120, 256)
+        gemm_row(f"tree matmul o_proj 32B M={M} K=8192 N=5120", M, 8192, 5120, 256, short=f"tree o32B M={M}")
     for M in (1, 64, 512, 4096):
-        gemm_row(f"down_proj 32B M={M} K=25600 N=5120 leaf128", M, 25600, 5120, choose_leaf_k(25600))
+        gemm_row(f"tree matmul down_proj 32B M={M} K=25600 N=5120 leaf128", M, 25600, 5120, choose_leaf_k(25600),
+                 short=f"tree dn32B/128 M={M}")
     library_row(4096, 8192, 5120)
     library_row(4096, 25600, 5120)
     library_row(2048, 4096, 24576)
     library_row(8192, 4096, 24576)
-    for name, M, K, N in (("qkv 8B", 2048, 4096, 6144), ("gate_up 8B", 2048, 4096, 24576), ("gate_up 8B", 8192, 4096, 24576),
-                          ("lm_head 8B", 128, 4096, 151936),
-                          ("qkv 8B", 1, 4096, 6144), ("qkv 8B", 32, 4096, 6144), ("qkv 8B", 128, 4096, 6144),
-                          ("gate_up 8B", 1, 4096, 24576), ("gate_up 8B", 32, 4096, 24576), ("gate_up 8B", 128, 4096, 24576),
-                          ("lm_head 8B", 1, 4096, 151936), ("lm_head 8B", 32, 4096, 151936)):
-        def make(M=M, K=K, N=N):
-            return (torch.randn((M, K), device=dev).to(torch.bfloat16), (torch.randn((N, K), device=dev) * 0.02).to(torch.bfloat16))
-        by = 2.0 * (M * K + K * N + M * N)
-        ms, _ = hip_time_ms(cycling(make, by, lambda X, W: bio.matmul_persistent(X, W.t())), steps, warmup, settle_ms)
-        rows.append((f"batch-invariant mm {name} M={M} K={K} N={N}", ms * 1e3, 2.0 * M * N * K / ms / 1e9, by / ms / 1e6))
+    in_json = {("qkv", 1), ("qkv", 2048), ("gate_up", 1), ("gate_up", 2048), ("lm_head", 1), ("lm_head", 128)}
+    for name, M, K, N in (("qkv", 1, 4096, 6144), ("qkv", 32, 4096, 6144), ("qkv", 128, 4096, 6144), ("qkv", 2048, 4096, 6144),
+                          ("gate_up", 1, 4096, 24576), ("gate_up", 32, 4096, 24576), ("gate_up", 128, 4096, 24576),
+                          ("gate_up", 2048, 4096, 24576), ("gate_up", 8192, 4096, 24576),
+                          ("lm_head", 1, 4096, 151936), ("lm_head", 32, 4096, 151936), ("lm_head", 128, 4096, 151936)):
+        gemm_row(f"batch-invariant mm {name} 8B M={M} K={K} N={N}", M, K, N, 0, lambda X, W: bio.matmul_persistent(X, W.t()),
+                 short=f"mm {name} M={M}" if (name, M) in in_json else None)
     for p in (2, 4, 8):
         by = (p + 1) * 2048 * 4096 * 2
-        make = lambda p=p: ([torch.randn((2048, 4096), device=dev).to(torch.bfloat16) for _ in range(p)],)  # noqa: E731
-        ms, _ = hip_time_ms(cycling(make, by, tree_combine), steps, warmup, settle_ms)
-        rows.append((f"tree_combine p={p} [2048,4096]", ms * 1e3, 0.0, by / ms / 1e6))
+        add(f"tree_combine p={p} [2048,4096]", lambda p=p: ([torch.randn((2048, 4096), device=dev).to(torch.bfloat16) for _ in range(p)],),
+            tree_combine, 0.0, by, "hbm", short=f"comb p={p}")
     w = torch.ones(4096, device=dev, dtype=torch.bfloat16)
     for r in (1, 7, 256, 4096):
-        by = r * 4096 * 4 + 8192
-        make = lambda r=r: (torch.randn((r, 4096), device=dev).to(torch.bfloat16),)  # noqa: E731
-        ms, _ = hip_time_ms(cycling(make, by, lambda x: bio.rms_norm(x, w, 1e-6)), steps, warmup, settle_ms)
-        rows.append((f"rmsnorm rows={r} hidden=4096", ms * 1e3, 0.0, by / ms / 1e6))
+        add(f"rmsnorm rows={r} hidden=4096", lambda r=r: (torch.randn((r, 4096), device=dev).to(torch.bfloat16),),
+            lambda x: bio.rms_norm(x, w, 1e-6), 0.0, r * 4096 * 4 + 8192, "hbm", short=f"rms r={r}")
     for r in (1, 7, 256, 4096):
-        by = r * 151936 * 8
-        make = lambda r=r: (torch.randn((r, 151936), device=dev),)  # noqa: E731
-        ms, _ = hip_time_ms(cycling(make, by, bio.log_softmax), max(steps // 4, 3), warmup, settle_ms)
-        rows.append((f"log_softmax rows={r} vocab=151936 (8 B/elem)", ms * 1e3, 0.0, by / ms / 1e6))
+        add(f"log_softmax fp32 rows={r} vocab=151936 (8 B/elem)", lambda r=r: (torch.randn((r, 151936), device=dev),),
+            bio.log_softmax, 0.0, r * 151936 * 8, "hbm", max(steps // 4, 3), short=f"lsm r={r}")
     for r in (256, 4096):
-        by = r * 151936 * 4
-        make = lambda r=r: (torch.randn((r, 151936), device=dev).to(torch.bfloat16),)  # noqa: E731
-        ms, _ = hip_time_ms(cycling(make, by, bio.log_softmax), max(steps // 4, 3), warmup, settle_ms)
-        rows.append((f"log_softmax bf16 in/out rows={r} vocab=151936 (4 B/elem)", ms * 1e3, 0.0, by / ms / 1e6))
+        add(f"log_softmax bf16 in/out rows={r} vocab=151936 (4 B/elem)",
+            lambda r=r: (torch.randn((r, 151936), device=dev).to(torch.bfloat16),), bio.log_softmax, 0.0, r * 151936 * 4, "hbm",
+            max(steps // 4, 3))
     for r in (1, 7, 256, 4096):
-        by = r * 4096 * 4
-        make = lambda r=r: (torch.randn((r, 4096), device=dev),)  # noqa: E731
-        ms, _ = hip_time_ms(cycling(make, 2 * by, lambda x: bio.mean_dim(x, -1)), steps, warmup, settle_ms)
-        rows.append((f"mean rows={r} n=4096", ms * 1e3, 0.0, by / ms / 1e6))
-    from llm_reproducibility_amd import ops
+        add(f"mean rows={r} n=4096", lambda r=r: (torch.randn((r, 4096), device=dev),), lambda x: bio.mean_dim(x, -1), 0.0,
+            r * 4096 * 4, "hbm", short=f"mean r={r}")
     for r in (1, 256, 4096):
-        by = r * 12288 * 6
-        make = lambda r=r: (torch.randn((r, 2 * 12288), device=dev).to(torch.bfloat16),)  # noqa: E731
-        ms, _ = hip_time_ms(cycling(make, by, ops.bi_silu_mul), steps, warmup, settle_ms)
-        rows.append((f"silu_mul rows={r} inter=12288 (6 B/elem)", ms * 1e3, 0.0, by / ms / 1e6))
+        add(f"silu_mul rows={r} inter=12288 (6 B/elem)", lambda r=r: (torch.randn((r, 2 * 12288), device=dev).to(torch.bfloat16),),
+            ops.bi_silu_mul, 0.0, r * 12288 * 6, "hbm", short="silu_mul r=4096" if r == 4096 else None)
     # fixed-order attention (Qwen3-8B heads: 32 query, 8 key/value, head_dim 128)
     Hq, Hkv, D = 32, 8, 128
+
     def i32(v):
         return torch.tensor(v, dtype=torch.int32, device=dev)
-    for name, B, qlen, ctx in (("prefill 8 x 512", 8, 512, 512), ("prefill 1 x 4096", 1, 4096, 4096),
-                               ("decode 128 seqs ctx 768", 128, 1, 768), ("decode 8 seqs ctx 4096", 8, 1, 4096)):
+    for name, short, B, qlen, ctx in (("decode 128 seqs ctx 768", "attn dec 128x768", 128, 1, 768),
+                                      ("decode 8 seqs ctx 4096", "attn dec 8x4096", 8, 1, 4096),
+                                      ("prefill 8 x 512", "attn pre 8x512", 8, 512, 512),
+                                      ("prefill 1 x 4096", "attn pre 1x4096", 1, 4096, 4096)):
         L = ((ctx + 31) // 32) * 32
         qs, ql, cl = i32([b * qlen for b in range(B)]), i32([qlen] * B), i32([ctx] * B)
         pairs = B * Hq * (qlen * (2 * ctx - qlen + 1) // 2)          # causal (query, key) pairs
@@ -241,15 +276,18 @@ def table(steps, warmup, hot=False, settle_ms=20.0):
             return (torch.randn((B * qlen, Hq, D), device=dev).to(torch.bfloat16),
                     torch.randn((B, Hkv, L, D), device=dev).to(torch.bfloat16),
                     torch.randn((B, Hkv, D, L), device=dev).to(torch.bfloat16))
-        ms, _ = hip_time_ms(cycling(make, byts, lambda q, kc, vt: ops.bi_attention_bf16(q, kc, vt, qs, ql, cl, qlen, D ** -0.5)),
-                            max(steps // 2, 3), warmup, settle_ms)
-        rows.append((f"attention {name}", ms * 1e3, 4.0 * pairs * D / ms / 1e9, byts / ms / 1e6))
+        add(f"attention {name}", make, lambda q, kc, vt: ops.bi_attention_bf16(q, kc, vt, qs, ql, cl, qlen, D ** -0.5),
+            4.0 * pairs * D, byts, "hbm" if qlen == 1 else "mfma", max(steps // 2, 3), short=short)
+    return rows
+
+
+def print_table(rows, hot):
     print("inputs " + ("reused by every call (hot in the memory-side cache)" if hot else
                        "cycled through more than 768 MB of distinct buffers (cold in the 256 MB memory-side cache)"), file=sys.stderr)
-    print(f"{'case':52s} {'us':>10s} {'TFLOP/s':>9s} {'%MFMA':>6s} {'GB/s':>9s} {'%HBM':>6s}", file=sys.stderr)
-    for name, us, tf, gbs in rows:
-        print(f"{name:52s} {us:10.1f} {tf:9.1f} {100 * tf / PEAK_BF16_TFLOPS:6.1f} {gbs:9.1f} {100 * gbs / PEAK_HBM_GBS:6.1f}",
-              file=sys.stderr)
+    print(f"{'case':66s} {'us':>10s} {'TFLOP/s':>9s} {'%MFMA':>6s} {'GB/s':>9s} {'%HBM':>6s} {'bound':>6s}", file=sys.stderr)
+    for r in rows:
+        print(f"{r['case']:66s} {r['us']:10.1f} {r['TFLOPs']:9.1f} {100 * r['TFLOPs'] / PEAK_BF16_TFLOPS:6.1f} "
+              f"{r['GBps']:9.1f} {100 * r['GBps'] / PEAK_HBM_GBS:6.1f} {r['bound']:>6s}", file=sys.stderr)
 
 
 def main():
@@ -257,12 +295,13 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--table", action="store_true", help="also print the per-shape table to stderr")
-    ap.add_argument("--table-hot", action="store_true", help="with --table: reuse one input set per case (cache-hot figures)")
+    ap.add_argument("--table", action="store_true", help="long form of the per-shape table, also printed to stderr")
+    ap.add_argument("--table-hot", action="store_true", help="reuse one input set per table case (cache-hot figures)")
+    ap.add_argument("--no-context-table", action="store_true", help="leave the per-shape table out of the JSON line")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--settle-ms", type=float, default=60.0,
-                    help="continuous load (the step itself) in front of the warm-up steps, so that the timed steps see "
-                         "the chip's settled state and not the transient that follows the host-side set-up; 0 disables")
+                    help="continuous load (the step itself) in front of the warm-up steps of `value`, so that the timed "
+                         "steps see the chip's settled state; `value_after_idle` is always measured without it")
     ap.add_argument("--ceiling", action="store_true",
                     help="also measure the MFMA-only and the one-pass-read ceilings of this chip (reported in `context`)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -274,35 +313,25 @@ def main():
 
     import torch
     from llm_reproducibility_amd import _lib
-    from llm_reproducibility_amd.tbik import matmul_tp_persistent
+    from llm_reproducibility_amd.tbik import matmul_tp_persistent, tree_combine
     from oracle import tbik_oracle as O
 
     _lib.lib()
     dev = torch.device("cuda:0")
-    # host-side work first (the GPU idles meanwhile): the CPU baseline, whose product is also the parity reference
-    cpu, want = (None, None) if args.no_cpu_baseline else cpu_baseline()
     X = O.silu_gated_bf16((M_, K_), 0).to(dev)
     W = O.gaussian_bf16((N_, K_), 0.02, 1).to(dev)      # [N,K], K contiguous
     Wt = W.t()
     step = lambda: matmul_tp_persistent(X, Wt)          # noqa: E731
     C = step()
-    # parity inside the bench (not timed): what is being timed equals the simulated TP=4 run bit for bit and agrees
-    # with the CPU oracle on the same inputs within the stated tolerance (1 bf16 ulp, or 2^-8 of the output scale)
-    from llm_reproducibility_amd.tbik import tree_combine
-    parts = [matmul_tp_persistent(X[:, r * 3072:(r + 1) * 3072], W[:, r * 3072:(r + 1) * 3072].t()) for r in range(4)]
-    assert torch.equal(tree_combine(parts), C), "TP=4 result differs from TP=1"
-    del parts
-    parity = None
-    if want is not None:
-        bad = O.outside_tolerance(C, want)
-        ulp = O.bf16_ulp_distance(C.cpu(), want)
-        assert not bad.any(), f"{int(bad.sum())} elements outside the tolerance against the CPU oracle"
-        scale = float(want.float().abs().max())
-        parity = {"vs_cpu_oracle_full_size": "every element within 1 bf16 ulp or 2^-8 of the output scale",
-                  "bit_equal_fraction": round(float((ulp == 0).float().mean()), 5),
-                  "within_1_ulp_fraction": round(float((ulp <= 1).float().mean()), 6),
-                  "max_abs_diff_over_scale": float((C.cpu().float() - want.float()).abs().max()) / scale,
-                  "tp4_bitwise_equal": True}
+    torch.cuda.synchronize()
+
+    # ---- timed: W warm-up steps and K steps right after the set-up, then the same behind the load phase
+    idle_ms, _ = hip_time_ms(step, args.steps, args.warmup)
+    ms, wall_ms = hip_time_ms(step, args.steps, args.warmup, args.settle_ms)
+    flops = 2.0 * M_ * N_ * K_
+    algo_bytes = 2.0 * (M_ * K_ + K_ * N_ + M_ * N_)
+    tflops = flops / (ms * 1e-3) / 1e12
+    tflops_idle = flops / (idle_ms * 1e-3) / 1e12
 
     if args.calibrate_copy:
         Y = torch.empty_like(X)
@@ -311,12 +340,6 @@ def main():
         torch.cuda.synchronize()
         del Y
 
-    # the figure right after the idle period (the transient), for the record; then the settled rate, which is `value`
-    cold_ms, _ = hip_time_ms(step, args.steps, args.warmup)
-    ms, wall_ms = hip_time_ms(step, args.steps, args.warmup, args.settle_ms)
-    flops = 2.0 * M_ * N_ * K_
-    algo_bytes = 2.0 * (M_ * K_ + K_ * N_ + M_ * N_)
-    tflops = flops / (ms * 1e-3) / 1e12
     out = {
         "metric": "TBIK matmul TFLOP/s & % bf16 MFMA peak, M=2048 K=12288 N=4096",
         "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -324,37 +347,62 @@ def main():
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "Qwen3-8B down_proj tree matmul X[2048,12288] x W[12288,4096] (configs[1], M=2048), leaf 256, TP=1",
                    "M": M_, "K": K_, "N": N_, "leaf_k": 256},
+        "value_after_idle": round(tflops_idle, 2),
+        "protocol": f"value: {args.settle_ms:g} ms of the step back to back, then W warm-up + K timed steps (settled rate); "
+                    "value_after_idle: W warm-up + K timed steps right after the set-up, no load phase",
         "pct_bf16_mfma_peak": round(100 * tflops / PEAK_BF16_TFLOPS, 2),
         "algorithmic_GBps": round(algo_bytes / (ms * 1e-3) / 1e9, 1),
         "roofline": {"bound": "mfma", "achieved": round(tflops, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(tflops / PEAK_BF16_TFLOPS, 4), "traffic": traffic_from_profile(),
-                     "traffic_source": "profiles/gemm_tree_deep_headline_counters.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
-                                       "scaled by a copy of known size; a figure of that profile, not of this run)",
-                     "kernel_avg_us": round(ms * 1e3, 2)},
+                     "traffic_source": "profiles/gemm_tree_deep_headline_counters.txt (a figure of that profile, not of this run)",
+                     "kernel_avg_us": round(ms * 1e3, 2), "frac_after_idle": round(tflops_idle / PEAK_BF16_TFLOPS, 4)},
     }
-    if cpu is not None:
-        out["cpu_baseline"] = cpu
-    context = {"settle_ms": args.settle_ms,
-               "settle_note": "the timed steps follow settle_ms of the same step run back to back (then the warm-up steps): "
-                              "after idling the chip needs about 25 ms of load to reach its steady rate",
-               "first_steps_after_idle_TFLOPs": round(flops / (cold_ms * 1e-3) / 1e12, 2)}
-    if parity is not None:
-        context["parity"] = parity
+    context = {}
     # the vendor library's plain GEMM on the same operands, measured the same way (reduction order not fixed, no tree;
     # not a code path of this library)
     lib_ms, _ = hip_time_ms(lambda: torch.matmul(X, Wt), args.steps, args.warmup, args.settle_ms)
     context["vendor_gemm_same_operands_TFLOPs"] = round(flops / (lib_ms * 1e-3) / 1e12, 2)
     context["note"] = "torch.matmul (vendor library), reduction order not fixed, no tree"
     # this library's own matmul without the tree (one fp32 accumulator over all of K, the batch-invariant mm) on the
-    # same operands: the same tile, ring and MFMA chain, so the difference to `value` is what the tree order costs
+    # same operands: the same ring and MFMA chain, so the difference to `value` is what the tree order costs
     from llm_reproducibility_amd.bio import batch_invariant_ops as bio
     mm_ms, _ = hip_time_ms(lambda: bio.matmul_persistent(X, Wt), args.steps, args.warmup, args.settle_ms)
     context["single_accumulator_mm_same_operands_TFLOPs"] = round(flops / (mm_ms * 1e-3) / 1e12, 2)
     if args.ceiling:
         context["ceiling"] = ceiling(args.settle_ms)
+    if args.table or not args.no_context_table:
+        t0 = time.perf_counter()
+        rows = table(12, 3, hot=args.table_hot, settle_ms=min(args.settle_ms, 10.0), full=args.table)
+        if args.table:
+            print_table(rows, args.table_hot)
+        # terse in the JSON line: case -> [us per call, algorithmic work of a call (flop when the bound is "m", bytes when
+        # it is "h"), achieved share of the bound's peak, bound]
+        context["table"] = {r["short"]: [r["us"], int(float(f"{(r['flop'] if r['bound'] == 'mfma' else r['bytes']):.4g}")),
+                                         round(r["frac"], 3), r["bound"][0]] for r in rows if r["short"]}
+        context["table_cols"] = ("[us per call (Python operator, HIP events, 12 calls after 10 ms of load, inputs "
+                                 + ("reused" if args.table_hot else "cycled: cold") + "), algorithmic flop (m) or bytes (h), share of "
+                                 f"{PEAK_BF16_TFLOPS:g} TFLOP/s (m) or {PEAK_HBM_GBS:g} GB/s (h), bound]; {time.perf_counter() - t0:.0f} s")
+
+    # ---- not timed: what was timed equals the simulated TP=4 run bit for bit and agrees with the CPU oracle on the same
+    # inputs within the stated tolerance (1 bf16 ulp, or 2^-8 of the output scale); the oracle run is also the CPU baseline
+    parts = [matmul_tp_persistent(X[:, r * 3072:(r + 1) * 3072], W[:, r * 3072:(r + 1) * 3072].t()) for r in range(4)]
+    assert torch.equal(tree_combine(parts), C), "TP=4 result differs from TP=1"
+    assert torch.equal(step(), C), "the step is not reproducible from call to call"
+    del parts
+    parity = {"tp4_bitwise_equal": True}
+    if not args.no_cpu_baseline:
+        cpu, want = cpu_baseline()
+        out["cpu_baseline"] = cpu
+        bad = O.outside_tolerance(C, want)
+        ulp = O.bf16_ulp_distance(C.cpu(), want)
+        assert not bad.any(), f"{int(bad.sum())} elements outside the tolerance against the CPU oracle"
+        scale = float(want.float().abs().max())
+        parity.update({"vs_cpu_oracle_full_size": "every element within 1 bf16 ulp or 2^-8 of the output scale",
+                       "bit_equal_fraction": round(float((ulp == 0).float().mean()), 5),
+                       "within_1_ulp_fraction": round(float((ulp <= 1).float().mean()), 6),
+                       "max_abs_diff_over_scale": float((C.cpu().float() - want.float()).abs().max()) / scale})
+    context["parity"] = parity
     out["context"] = context
-    if args.table:
-        table(max(args.steps // 2, 5), max(args.warmup // 2, 2), hot=args.table_hot, settle_ms=min(args.settle_ms, 20.0))
     print(json.dumps(out))
 
 
