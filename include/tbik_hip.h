@@ -324,6 +324,45 @@ int bi_qk_norm_rope_cache_bf16(const void* qkv, int64_t ld,
  */
 int bi_argmax_bf16(const void* x, int64_t ld, void* out, int64_t rows, int cols, tbik_stream_t stream);
 
+/*
+ * One-launch compositions for decode-sized batches (a handful of rows): the producer of a matmul's activations runs
+ * inside the matmul while it stages them, which saves a launch and a round trip of the activations through memory.
+ * Both evaluate exactly the expressions of the two-launch forms (the same device functions, the same MFMA chains and
+ * tree), so the results are bit-identical to those and a caller may take either form per call.  Both return
+ * TBIK_ERR_UNSUPPORTED (3) when the one-launch kernel does not apply to the shape -- more rows than the work-group can
+ * stage, a row-major B, a strip grid that would not balance the chip: the caller then runs the two launches.
+ *
+ * bi_rmsnorm_gemm_bf16:  C[M,N] = bi_gemm_bf16( bi_rmsnorm_bf16(x [+ residual], norm_weight, eps), B )   (+ bias)
+ *   x [M,K] (row stride ldx), residual [M,K] or NULL, norm_weight [K] or NULL; when residual is given, residual_out
+ *   [M,K] receives bf16(x + residual) and must not be x or residual themselves (every work-group reads both while
+ *   the first one writes it); B = [N,K] K-contiguous (ldb_k == 1).  Applies for K <= 8192 with M * K <= 32768 and
+ *   M * (2K + 16) <= 40 KiB (M <= 4 at a hidden size of 4096).
+ *   Replaces: RMSNorm.forward_native routed through the batch-invariant mean (src/patch/patch_batch_invariant.py:9-16)
+ *             followed by the column-parallel projection through aten::mm (src/bio/batch_invariant_ops.py:442-447).
+ *
+ * tbik_gemm_silu_mul_bf16:  C[M,N] = tbik_gemm_bf16( act, B, leaf_k )   (+ bias),  act = silu(gate) * up as bi_silu_mul_bf16
+ *   gate, up [M,K] with the same row stride ld (the two halves of the merged gate/up projection: up = gate + inter;
+ *   a rank's K shard of both halves in a tensor-parallel run), K = the reduction extent of the row-split projection;
+ *   B = [N,K] K-contiguous.  Applies where the one-launch few-rows tree kernel does (M <= 4).
+ *   Replaces: SiluAndMul followed by the patched RowParallelLinear forward of down_proj,
+ *             src/patch/patch_tp_invariant.py:10-48 (the local matmul of :31).
+ */
+int bi_rmsnorm_gemm_bf16(const void* x, int64_t ldx,
+                         const void* residual_or_null, int64_t ldr,
+                         const void* norm_weight_or_null, float eps,
+                         void* residual_out_or_null, int64_t ldro,
+                         const void* B, int64_t ldb_k, int64_t ldb_n,
+                         void* C, int64_t ldc,
+                         int M, int N, int K,
+                         const void* bias_or_null,
+                         tbik_stream_t stream);
+int tbik_gemm_silu_mul_bf16(const void* gate, const void* up, int64_t ld,
+                            const void* B, int64_t ldb_k, int64_t ldb_n,
+                            void* C, int64_t ldc,
+                            int M, int N, int K, int leaf_k,
+                            const void* bias_or_null,
+                            tbik_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

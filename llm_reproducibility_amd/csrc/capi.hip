@@ -27,11 +27,16 @@ int qk_norm_rope_cache_dispatch(const void* qkv, int64_t ld, const void* q_weigh
                                 int max_len, int batch, float eps, hipStream_t stream);
 int silu_mul_dispatch(const void* gate_up, int64_t ld_in, void* out, int64_t ld_out, int64_t rows, int inter, bool f16,
                       hipStream_t stream);
+int rmsnorm_gemm_dispatch(const void* x, int64_t ldx, const void* res, int64_t ldr, const void* norm_w, float eps,
+                          void* res_out, int64_t ldro, const void* B, int64_t ldb_k, int64_t ldb_n, void* C, int64_t ldc,
+                          int M, int N, int K, const void* bias, hipStream_t stream);
+int gemm_tree_gated_dispatch(const void* gate, const void* up, int64_t ld, const void* B, int64_t ldb_k, int64_t ldb_n, void* C,
+                             int64_t ldc, int M, int N, int K, int leaf_k, const void* bias, hipStream_t stream);
 }  // namespace tbik
 
 extern "C" {
 
-int tbik_abi_version(void) { return 11; }
+int tbik_abi_version(void) { return 12; }
 
 const char* tbik_error_string(int code) {
   switch (code) {
@@ -100,6 +105,19 @@ int bi_gemm_bf16(const void* A, int64_t lda, const void* B, int64_t ldb_k, int64
                  int N, int K, const void* bias_or_null, tbik_stream_t stream) {
   return tbik::gemm_dispatch(false, false, A, lda, B, ldb_k, ldb_n, C, ldc, M, N, K, 0, bias_or_null, nullptr, 0,
                              static_cast<hipStream_t>(stream));
+}
+
+int bi_rmsnorm_gemm_bf16(const void* x, int64_t ldx, const void* residual_or_null, int64_t ldr, const void* norm_weight_or_null,
+                         float eps, void* residual_out_or_null, int64_t ldro, const void* B, int64_t ldb_k, int64_t ldb_n,
+                         void* C, int64_t ldc, int M, int N, int K, const void* bias_or_null, tbik_stream_t stream) {
+  return tbik::rmsnorm_gemm_dispatch(x, ldx, residual_or_null, ldr, norm_weight_or_null, eps, residual_out_or_null, ldro, B,
+                                     ldb_k, ldb_n, C, ldc, M, N, K, bias_or_null, static_cast<hipStream_t>(stream));
+}
+
+int tbik_gemm_silu_mul_bf16(const void* gate, const void* up, int64_t ld, const void* B, int64_t ldb_k, int64_t ldb_n, void* C,
+                            int64_t ldc, int M, int N, int K, int leaf_k, const void* bias_or_null, tbik_stream_t stream) {
+  return tbik::gemm_tree_gated_dispatch(gate, up, ld, B, ldb_k, ldb_n, C, ldc, M, N, K, leaf_k, bias_or_null,
+                                        static_cast<hipStream_t>(stream));
 }
 
 int bi_rmsnorm_bf16(const void* x, int64_t ldx, const void* residual_or_null, int64_t ldr, const void* weight_or_null,

@@ -6,18 +6,10 @@
 // then the product rounded to bf16 -- two roundings, as an unfused `F.silu(gate) * up` on bf16 tensors
 // gives.  Elementwise, so batch invariant by construction.  HBM bound: 6 bytes per output element.
 #include "common.h"
+#include "silu_mul.h"
 
 namespace tbik {
 
-template <bool F16>
-__device__ __forceinline__ uint32_t silu_mul_pair(uint32_t g, uint32_t u) {
-  using Num = Num16<F16>;
-  const float g0 = Num::lo(g), g1 = Num::hi(g);
-  const float s0 = g0 / (1.0f + expf(-g0));
-  const float s1 = g1 / (1.0f + expf(-g1));
-  const uint32_t s = Num::pack(s0, s1);
-  return Num::pack(Num::lo(s) * Num::lo(u), Num::hi(s) * Num::hi(u));
-}
 
 // One thread per 8 outputs (16-byte loads and stores); 2-D grid-stride over (row, pack).
 template <bool F16>

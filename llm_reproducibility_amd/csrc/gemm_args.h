@@ -70,6 +70,16 @@ struct StreamArgs {
   int vec_store;
 };
 int gemm_single_acc_stream_launch(const StreamArgs& a, bool f16, hipStream_t stream);
+// the same product with X = RMSNorm(a.X [+ res]) * w formed while the activations are staged (bf16, a few rows);
+// res_out receives the rounded sum a.X + res when res is given; TBIK_ERR_UNSUPPORTED: run the two launches
+struct StreamNormArgs {
+  const uint16_t* res = nullptr;
+  const uint16_t* w = nullptr;
+  uint16_t* res_out = nullptr;
+  int64_t ldr = 0, ldro = 0;
+  float eps = 0.f;
+};
+int gemm_single_acc_stream_norm_launch(const StreamArgs& a, const StreamNormArgs& nrm, hipStream_t stream);
 
 // gemm_tree_strip.hip: tree-ordered 16-bit GEMM for at most 16 rows, K cut over the waves of a work-group
 struct StripArgs {
@@ -81,9 +91,14 @@ struct StripArgs {
   int M, N, K;
   int flb, lb;         // K = flb * leaf_k * 2^lb
   int vec_store;
+  const uint16_t* X2 = nullptr;  // gated form only: X = gate rows, X2 = up rows (same row stride)
 };
 int gemm_tree_strip_waves(int M, int N, int K, int lb);  // waves per strip, or 0: use another kernel
 int gemm_tree_strip_launch(const StripArgs& a, int leaf_k, int waves, bool f16, hipStream_t stream);
+// the same kernel with the activations silu(a.X) * a.X2 (gate and up rows, [M,K] each, row stride a.ldx) formed while
+// the first weights are in flight (bf16, at most 4 rows); waves = 0: run the two launches
+int gemm_tree_strip_gated_waves(int M, int N, int K, int lb);
+int gemm_tree_strip_gated_launch(const StripArgs& a, int leaf_k, int waves, hipStream_t stream);
 
 // tree_combine.hip
 // ldo != 0: `out` is a [numel / N, N] matrix with row stride ldo (the partials stay contiguous)

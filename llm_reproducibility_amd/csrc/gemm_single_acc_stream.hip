@@ -14,6 +14,7 @@
 // quad kernels, hence the same bits.
 #include "common.h"
 #include "gemm_args.h"
+#include "rmsnorm_row.h"
 
 namespace tbik {
 
@@ -55,10 +56,17 @@ __device__ __forceinline__ void stream_store(const StreamArgs& p, const f32x4* a
 
 // A few rows (M * K small enough for LDS): all of X is staged once, one barrier, and then every wave runs on its
 // own -- nothing couples a wave's stream of weight loads to its neighbours'.
+//
+// NORM > 0: the activations are RMSNorm(x [+ residual]) * weight, computed by the work-group while it stages them -- one
+// wavefront per row with the row function of the stand-alone RMSNorm kernel (NORM = its chunks per lane: 8 for rows
+// of up to 4096 elements, 16 up to 8192), so the staged values are the bits that kernel would have written to memory,
+// and the product is the one of the two-launch composition.  Every work-group normalises all M rows for itself (a few
+// KB from the L2); the first one also stores the new residual.  The norm's loads follow the first weight loads into
+// the memory queue, so its latency is covered by the start of the weight stream.
 constexpr int ROWS_U = 16;        // steps per register chunk (two chunks in flight)
 constexpr int ROWS_MAX_ELEMS = 32768;  // M * K at most: two rounds of staging loads in a work-group of 4 waves
-template <int NWAVES, bool F16>   // strips per work-group: 1 when N is small, so that every CU gets some
-__global__ __launch_bounds__(NWAVES * 64) void gemm_single_acc_stream_rows_kernel(const StreamArgs p) {
+template <int NWAVES, bool F16, int NORM = 0>   // strips per work-group: 1 when N is small, so that every CU gets some
+__global__ __launch_bounds__(NWAVES * 64) void gemm_single_acc_stream_rows_kernel(const StreamArgs p, const StreamNormArgs nrm) {
   using Num = Num16<F16>;
   constexpr int NW = NWAVES, NT = NWAVES * 64;
   constexpr int U = ROWS_U;
@@ -80,9 +88,31 @@ __global__ __launch_bounds__(NWAVES * 64) void gemm_single_acc_stream_rows_kerne
 #pragma unroll
     for (int u = 0; u < U; u++) w[u] = *reinterpret_cast<const bf16x8*>(wp + (int64_t)(c * U + u) * 32);
   };
-  if (nchunks > 0) load(wa, 0);  // the weights start flowing before X is staged
-
-  {
+  if constexpr (NORM > 0) {
+    // A wave's loads return in the order they were issued: the row this wave normalises is asked for FIRST, then the
+    // first chunk of weights, so that the norm (loads, a reduction over the wave, LDS) runs while the weight stream
+    // fills.  No load sits under a branch (a wave without a row of its own loads the last row and drops it; the
+    // launcher guarantees a whole chunk of weights), or the compiler would wait for the weights before the norm.
+    RmsnormRow<NORM, F16, true> row;
+    const bool mine = wave < p.M;
+    const int myrow = min(wave, p.M - 1);
+    row.load(p.X + (int64_t)myrow * p.ldx, nrm.res ? nrm.res + (int64_t)myrow * nrm.ldr : nullptr, nrm.w, p.K, lane);
+    __builtin_amdgcn_sched_barrier(0);   // the scheduler would put the weight loads first
+    load(wa, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    if (mine) {
+      uint8_t* dst = xs + wave * rowb;
+      row.finish((nrm.res_out && blockIdx.x == 0) ? nrm.res_out + (int64_t)wave * nrm.ldro : nullptr, p.K, nrm.eps, lane,
+                 [&](int c, const uint4& o) { *reinterpret_cast<uint4*>(dst + c * 16) = o; });
+    }
+    for (int m = wave + NW; m < p.M; m += NW) {   // more rows than waves: the others queue behind the weights
+      uint8_t* dst = xs + m * rowb;
+      rmsnorm_row<NORM, F16>(p.X + (int64_t)m * p.ldx, nrm.res ? nrm.res + (int64_t)m * nrm.ldr : nullptr, nrm.w,
+                             (nrm.res_out && blockIdx.x == 0) ? nrm.res_out + (int64_t)m * nrm.ldro : nullptr, p.K, nrm.eps,
+                             lane, [&](int c, const uint4& o) { *reinterpret_cast<uint4*>(dst + c * 16) = o; });
+    }
+  } else {
+    if (nchunks > 0) load(wa, 0);  // the weights start flowing before X is staged
     const int kc = p.K / 8, total = p.M * kc;
     for (int base = 0; base < total; base += NT * 8) {  // one or two rounds of 8 loads in flight per thread
       u32x4 xr[8];
@@ -286,35 +316,61 @@ static int stream_launch(const StreamArgs& a, hipStream_t stream) {
   }
 }
 
-template <int NWAVES, bool F16>
-static int stream_rows_launch(const StreamArgs& a, hipStream_t stream) {
+template <int NWAVES, bool F16, int NORM = 0>
+static int stream_rows_launch(const StreamArgs& a, hipStream_t stream, const StreamNormArgs& nrm = StreamNormArgs{}) {
   const int64_t groups = ((int64_t)a.N + 16 * NWAVES - 1) / (16 * NWAVES);
   if (groups > 0x7fffffff) return TBIK_ERR_INVALID;
   const int smem = a.M * (a.K * 2 + 16);
-  hipLaunchKernelGGL((gemm_single_acc_stream_rows_kernel<NWAVES, F16>), dim3((unsigned)groups), dim3(NWAVES * 64), smem, stream, a);
+  hipLaunchKernelGGL((gemm_single_acc_stream_rows_kernel<NWAVES, F16, NORM>), dim3((unsigned)groups), dim3(NWAVES * 64), smem,
+                     stream, a, nrm);
   return hip_code(hipGetLastError());
+}
+
+// Strips per work-group of the whole-X kernel.  HBM bandwidth is shared about equally among the CUs that ask for it, so
+// the CU with the most work-groups finishes last and the grid should put the same number on every CU: the score is the
+// share of CU slots that the last round of work-groups leaves used (measured: gate_up of an 8B model, 1536 strips, 41 us
+// as 384 groups of four, 37 us as 512 groups of three).  One strip per work-group restages X for every strip and is only
+// considered while X is small; two strips per work-group measured worse than either neighbour throughout.
+static int stream_rows_waves(const StreamArgs& a) {
+  const int64_t strips = ((int64_t)a.N + 15) / 16;
+  auto score = [&](int nw, double weight) {
+    const int64_t groups = (strips + nw - 1) / nw;
+    return weight * (double)groups / (double)(((groups + 255) / 256) * 256);
+  };
+  const double s3 = score(3, 1.0), s4 = score(4, 0.98);
+  const double s1 = a.M * a.K <= ROWS_MAX_ELEMS / 4 ? score(1, 0.95) : 0.0;
+  if (s1 > s3 && s1 > s4) return 1;
+  return s3 >= s4 ? 3 : 4;
+}
+
+// all of X fits the staging registers of one pass and 40 KiB of LDS (several work-groups per CU)
+static bool stream_rows_applies(const StreamArgs& a) {
+  return a.M <= 16 && (int64_t)a.M * a.K <= ROWS_MAX_ELEMS && (int64_t)a.M * (a.K * 2 + 16) <= 40 * 1024;
+}
+
+// mm of RMSNorm(x [+ residual]) * weight in one launch: only where the whole-X kernel applies (a few rows) and the
+// row length is one the stand-alone norm kernel takes; TBIK_ERR_UNSUPPORTED otherwise (the caller runs the two launches).
+int gemm_single_acc_stream_norm_launch(const StreamArgs& a, const StreamNormArgs& nrm, hipStream_t stream) {
+  // K >= 512: the kernel issues its first chunk of weight loads (16 steps of 32) unconditionally
+  if (a.M <= 0 || (a.K & 31) != 0 || a.K < 512 || a.K > 8192 || !stream_rows_applies(a)) return TBIK_ERR_UNSUPPORTED;
+  const int nw = stream_rows_waves(a);
+  if (a.K <= 4096) {
+    if (nw == 1) return stream_rows_launch<1, false, 8>(a, stream, nrm);
+    if (nw == 3) return stream_rows_launch<3, false, 8>(a, stream, nrm);
+    return stream_rows_launch<4, false, 8>(a, stream, nrm);
+  }
+  if (nw == 1) return stream_rows_launch<1, false, 16>(a, stream, nrm);
+  if (nw == 3) return stream_rows_launch<3, false, 16>(a, stream, nrm);
+  return stream_rows_launch<4, false, 16>(a, stream, nrm);
 }
 
 // Requires 0 < M <= 64 and K a multiple of 32 (checked by the dispatcher).
 int gemm_single_acc_stream_launch(const StreamArgs& a, bool f16, hipStream_t stream) {
   if (a.M <= 0 || a.M > 64 || (a.K & 31) != 0) return TBIK_ERR_UNSUPPORTED;
-  // one block of rows, and all of X fits the staging registers of one pass and 40 KiB of LDS (several work-groups
-  // per CU)
-  if (a.M <= 16 && (int64_t)a.M * a.K <= ROWS_MAX_ELEMS && (int64_t)a.M * (a.K * 2 + 16) <= 40 * 1024) {
-    // Strips per work-group.  HBM bandwidth is shared about equally among the CUs that ask for it, so the CU with
-    // the most work-groups finishes last and the grid should put the same number on every CU: the score is the share of CU slots that the
-    // last round of work-groups leaves used (measured: gate_up of an 8B model, 1536 strips, 41 us as 384 groups of
-    // four, 37 us as 512 groups of three).  One strip per work-group restages X for every strip and is only
-    // considered while X is small; two strips per work-group measured worse than either neighbour throughout.
-    const int64_t strips = ((int64_t)a.N + 15) / 16;
-    auto score = [&](int nw, double weight) {
-      const int64_t groups = (strips + nw - 1) / nw;
-      return weight * (double)groups / (double)(((groups + 255) / 256) * 256);
-    };
-    const double s3 = score(3, 1.0), s4 = score(4, 0.98);
-    const double s1 = a.M * a.K <= ROWS_MAX_ELEMS / 4 ? score(1, 0.95) : 0.0;
-    if (s1 > s3 && s1 > s4) return f16 ? stream_rows_launch<1, true>(a, stream) : stream_rows_launch<1, false>(a, stream);
-    if (s3 >= s4) return f16 ? stream_rows_launch<3, true>(a, stream) : stream_rows_launch<3, false>(a, stream);
+  if (stream_rows_applies(a)) {
+    const int nw = stream_rows_waves(a);
+    if (nw == 1) return f16 ? stream_rows_launch<1, true>(a, stream) : stream_rows_launch<1, false>(a, stream);
+    if (nw == 3) return f16 ? stream_rows_launch<3, true>(a, stream) : stream_rows_launch<3, false>(a, stream);
     return f16 ? stream_rows_launch<4, true>(a, stream) : stream_rows_launch<4, false>(a, stream);
   }
   const int mb = (a.M + 15) / 16;

@@ -792,4 +792,57 @@ static int gemm_dispatch_impl(bool tree, bool f16, const void* A, int64_t lda, c
   return tree_combine_bias_dispatch(parts, pl.split, C, (int64_t)M * N, bias, N, f16, stream, ldc);
 }
 
+// ------------------------------------------------------------------------------------------------
+// One-launch compositions for decode-sized batches: the producer of a GEMM's activations runs inside the GEMM while
+// it stages them.  Both evaluate exactly the expressions of the two-launch forms (shared device functions), so a
+// caller may take either; both return TBIK_ERR_UNSUPPORTED when the one-launch kernel does not apply to the shape,
+// and the caller then runs the two launches.
+// ------------------------------------------------------------------------------------------------
+int rmsnorm_gemm_dispatch(const void* x, int64_t ldx, const void* res, int64_t ldr, const void* norm_w, float eps,
+                          void* res_out, int64_t ldro, const void* B, int64_t ldb_k, int64_t ldb_n, void* C, int64_t ldc,
+                          int M, int N, int K, const void* bias, hipStream_t stream) {
+  if (M < 0 || N < 0 || K <= 0) return TBIK_ERR_INVALID;
+  if (!x || !B || !C || (res && !res_out)) return TBIK_ERR_INVALID;
+  if (ldb_k != 1) return TBIK_ERR_UNSUPPORTED;  // the weight as nn.Linear stores it
+  if (M == 0 || N == 0) return TBIK_ERR_UNSUPPORTED;
+  if (ldx < K || ldb_n < K || ldc < N || (res && (ldr < K || ldro < K))) return TBIK_ERR_INVALID;
+  auto bad = [](const void* p, int64_t ld) { return (reinterpret_cast<uintptr_t>(p) & 15) != 0 || (ld & 7) != 0; };
+  if (bad(x, ldx) || bad(B, ldb_n) || (K & 7) || (res && (bad(res, ldr) || bad(res_out, ldro))) || (norm_w && bad(norm_w, 8)))
+    return TBIK_ERR_ALIGNMENT;
+  if (reinterpret_cast<uintptr_t>(C) & 1) return TBIK_ERR_ALIGNMENT;
+  // every work-group reads x and the residual while the first one stores the new residual
+  if (res_out && (res_out == x || res_out == res)) return TBIK_ERR_INVALID;
+  const int vec_store = ((reinterpret_cast<uintptr_t>(C) & 7) == 0 && (ldc & 3) == 0) ? 1 : 0;
+  StreamArgs sa{static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(B), static_cast<uint16_t*>(C),
+                static_cast<const uint16_t*>(bias), ldx, ldb_n, ldc, M, N, K, vec_store};
+  StreamNormArgs na;
+  na.res = static_cast<const uint16_t*>(res);
+  na.w = static_cast<const uint16_t*>(norm_w);
+  na.res_out = static_cast<uint16_t*>(res_out);
+  na.ldr = ldr;
+  na.ldro = ldro;
+  na.eps = eps;
+  return gemm_single_acc_stream_norm_launch(sa, na, stream);
+}
+
+int gemm_tree_gated_dispatch(const void* gate, const void* up, int64_t ld, const void* B, int64_t ldb_k, int64_t ldb_n, void* C,
+                             int64_t ldc, int M, int N, int K, int leaf_k, const void* bias, hipStream_t stream) {
+  if (M < 0 || N < 0 || K <= 0) return TBIK_ERR_INVALID;
+  if (!gate || !up || !B || !C) return TBIK_ERR_INVALID;
+  if (leaf_k != 256 && leaf_k != 128) return TBIK_ERR_UNSUPPORTED;
+  if (ldb_k != 1 || M == 0 || N == 0) return TBIK_ERR_UNSUPPORTED;
+  if (ld < K || ldb_n < K || ldc < N) return TBIK_ERR_INVALID;
+  if (!aligned16(gate) || !aligned16(up) || !aligned16(B) || (ld & 7) || (ldb_n & 7) || (K & 7)) return TBIK_ERR_ALIGNMENT;
+  if (reinterpret_cast<uintptr_t>(C) & 1) return TBIK_ERR_ALIGNMENT;
+  int T, flb, level_k;
+  if (tbik_tree_params(K, leaf_k, &T, &flb, &level_k) != TBIK_OK) return TBIK_ERR_INVALID;
+  const int waves = gemm_tree_strip_gated_waves(M, N, K, level_k - 1);
+  if (!waves) return TBIK_ERR_UNSUPPORTED;
+  const int vec_store = ((reinterpret_cast<uintptr_t>(C) & 7) == 0 && (ldc & 3) == 0) ? 1 : 0;
+  StripArgs sa{static_cast<const uint16_t*>(gate), static_cast<const uint16_t*>(B), static_cast<uint16_t*>(C),
+               static_cast<const uint16_t*>(bias), ld, ldb_n, ldc, M, N, K, flb, level_k - 1, vec_store,
+               static_cast<const uint16_t*>(up)};
+  return gemm_tree_strip_gated_launch(sa, leaf_k, waves, stream);
+}
+
 }  // namespace tbik

@@ -12,6 +12,7 @@
 // Replaces matmul_kernel_tp_persistent, src/tbik/tree_based_matmul.py:50-187, for a few rows (the kernel itself takes up to 16).
 #include "common.h"
 #include "gemm_args.h"
+#include "silu_mul.h"
 
 namespace tbik {
 
@@ -20,12 +21,17 @@ constexpr int U = 4;         // 32-wide k steps per register chunk (128 k)
 constexpr int MAXLEV = 3;    // binary levels a wave keeps for its own groups (at most 8 groups per wave)
 }  // namespace strip
 
-// CPL: chunks per leaf (2 = leaf 256, 1 = leaf 128); S: waves per work-group = subtrees K is cut into
-template <int CPL, int S, bool F16>
+// CPL: chunks per leaf (2 = leaf 256, 1 = leaf 128); S: waves per work-group = subtrees K is cut into.
+// GATED: p.X and p.X2 are the gate and the up half of the merged projection and the activations are silu(gate) * up, formed by the
+// work-group once while the first weight chunks are in flight (the function of the stand-alone kernel, so the bits it
+// would have written to memory) and kept in LDS, M rows of 2K + 16 bytes, from where every wave takes its fragments;
+// the tree and the MFMA chains do not change, so the product is the one of the two-launch composition.
+template <int CPL, int S, bool F16, bool GATED = false>
 __global__ __launch_bounds__(64 * S) __attribute__((amdgpu_waves_per_eu(4, 8))) void gemm_tree_strip_kernel(const StripArgs p) {
   using namespace strip;
   using Num = Num16<F16>;
   __shared__ uint2 part[S][64];
+  extern __shared__ __attribute__((aligned(16))) uint8_t act[];   // GATED only
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -45,9 +51,11 @@ __global__ __launch_bounds__(64 * S) __attribute__((amdgpu_waves_per_eu(4, 8))) 
 #pragma unroll
     for (int u = 0; u < U; u++) {
       w[u] = *reinterpret_cast<const bf16x8*>(wp + (int64_t)(cc * U + u) * 32);
-      x[u] = *reinterpret_cast<const bf16x8*>(xp + (int64_t)(cc * U + u) * 32);
+      if constexpr (!GATED) x[u] = *reinterpret_cast<const bf16x8*>(xp + (int64_t)(cc * U + u) * 32);
     }
   };
+  const int act_rowb = p.K * 2 + 16;
+  const uint8_t* act_frag = act + min(r, p.M - 1) * act_rowb + (k0 + 8 * g) * 2;
 
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   uint32_t t[2] = {0u, 0u};        // current node, packed (n, n+1), (n+2, n+3)
@@ -93,16 +101,72 @@ __global__ __launch_bounds__(64 * S) __attribute__((amdgpu_waves_per_eu(4, 8))) 
   };
   // chunks past the end (the loop runs in threes) multiply the re-read last chunk into an accumulator nobody reads
   auto chunk = [&](const bf16x8* w, const bf16x8* x, int c) __attribute__((always_inline)) {
+    if constexpr (GATED) {
+      bf16x8 xa[U];
+      const int cc = min(c, nch - 1);
 #pragma unroll
-    for (int u = 0; u < U; u++) acc = Num::mfma(w[u], x[u], acc);
+      for (int u = 0; u < U; u++) xa[u] = *reinterpret_cast<const bf16x8*>(act_frag + (cc * U + u) * 64);
+#pragma unroll
+      for (int u = 0; u < U; u++) acc = Num::mfma(w[u], xa[u], acc);
+    } else {
+#pragma unroll
+      for (int u = 0; u < U; u++) acc = Num::mfma(w[u], x[u], acc);
+    }
     leaf_done(c < nch && (CPL == 1 || (c & 1)));
   };
 
   // the scheduling barriers keep the loads where they are written: left alone, the scheduler sinks them towards
   // their use to shorten live ranges, and the stream is no longer two chunks ahead
-  load(w0, x0, 0);
-  __builtin_amdgcn_sched_barrier(0);
-  load(w1, x1, 1);
+  if constexpr (GATED) {
+    // A wave's loads return in the order they were issued: the first round of gate / up chunks is asked for BEFORE the
+    // first weight chunks, so that the activations are formed while the weight stream fills.  The loads are issued
+    // unconditionally (clamped to the last chunk), or the compiler would wait for the weights as well before the first
+    // use.  Six chunks per thread and round: one round covers a row of 12288 with four waves.
+    constexpr int R = 6, NT = 64 * S;
+    const int kc = p.K / 8, total = p.M * kc;
+    uint4 gq[R], uq[R];
+    auto issue = [&](int base) __attribute__((always_inline)) {
+#pragma unroll
+      for (int i = 0; i < R; i++) {
+        const int q = min(base + (int)threadIdx.x + NT * i, total - 1);
+        const int row = q / kc, c = q - row * kc;
+        const int64_t off = (int64_t)row * p.ldx + c * 8;
+        gq[i] = *reinterpret_cast<const uint4*>(p.X + off);
+        uq[i] = *reinterpret_cast<const uint4*>(p.X2 + off);
+      }
+    };
+    auto consume = [&](int base) __attribute__((always_inline)) {
+#pragma unroll
+      for (int i = 0; i < R; i++) {
+        const int q = base + (int)threadIdx.x + NT * i;
+        if (q < total) {
+          const int row = q / kc, c = q - row * kc;
+          uint4 o;
+          o.x = silu_mul_pair<F16>(gq[i].x, uq[i].x);
+          o.y = silu_mul_pair<F16>(gq[i].y, uq[i].y);
+          o.z = silu_mul_pair<F16>(gq[i].z, uq[i].z);
+          o.w = silu_mul_pair<F16>(gq[i].w, uq[i].w);
+          *reinterpret_cast<uint4*>(act + row * act_rowb + c * 16) = o;
+        }
+      }
+    };
+    issue(0);
+    __builtin_amdgcn_sched_barrier(0);
+    load(w0, x0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    load(w1, x1, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    consume(0);
+    for (int base = R * NT; base < total; base += R * NT) {
+      issue(base);
+      consume(base);
+    }
+    __syncthreads();
+  } else {
+    load(w0, x0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    load(w1, x1, 1);
+  }
   for (int c = 0; c < nch; c += 3) {
     __builtin_amdgcn_sched_barrier(0);
     load(w2, x2, c + 2);
@@ -187,6 +251,41 @@ static int launch_strip(const StripArgs& a, int s, hipStream_t stream) {
     default: return TBIK_ERR_INVALID;
   }
   return hip_code(hipGetLastError());
+}
+
+template <int CPL, int S>
+static int launch_strip_gated_s(const StripArgs& a, hipStream_t stream) {
+  const unsigned strips = (unsigned)((a.N + 15) / 16);
+  const int smem = a.M * (a.K * 2 + 16);
+  auto kern = gemm_tree_strip_kernel<CPL, S, false, true>;
+  if (smem > 32 * 1024) {
+    static std::atomic<uint64_t> done{0};
+    hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, done);
+    if (e != hipSuccess) return hip_code(e);
+  }
+  hipLaunchKernelGGL(kern, dim3(strips), dim3(64 * S), smem, stream, a);
+  return hip_code(hipGetLastError());
+}
+
+// Tree matmul of silu(gate) * up for a.X = gate, a.X2 = up ([M,K] each, row stride a.ldx), bf16: where the one-launch
+// kernel applies and the activations (M rows of 2K + 16 bytes) fit the LDS; 0 otherwise.
+int gemm_tree_strip_gated_waves(int M, int N, int K, int lb) {
+  if (M > 4 || (int64_t)M * (K * 2 + 16) > 128 * 1024) return 0;
+  return gemm_tree_strip_waves(M, N, K, lb);
+}
+
+int gemm_tree_strip_gated_launch(const StripArgs& a, int leaf_k, int waves, hipStream_t stream) {
+  if (a.M <= 0 || a.M > 4 || a.N <= 0 || !a.X2 || (leaf_k != 256 && leaf_k != 128)) return TBIK_ERR_INVALID;
+  if (a.flb <= 0 || a.lb < 0 || (int64_t)a.flb * leaf_k * (1 << a.lb) != a.K) return TBIK_ERR_INVALID;
+  if (waves < 2 || waves > 8 || (waves & (waves - 1)) || waves > (1 << a.lb)) return TBIK_ERR_INVALID;
+  if (leaf_k == 256) {
+    if (waves == 2) return launch_strip_gated_s<2, 2>(a, stream);
+    if (waves == 4) return launch_strip_gated_s<2, 4>(a, stream);
+    return launch_strip_gated_s<2, 8>(a, stream);
+  }
+  if (waves == 2) return launch_strip_gated_s<1, 2>(a, stream);
+  if (waves == 4) return launch_strip_gated_s<1, 4>(a, stream);
+  return launch_strip_gated_s<1, 8>(a, stream);
 }
 
 int gemm_tree_strip_launch(const StripArgs& a, int leaf_k, int waves, bool f16, hipStream_t stream) {

@@ -4,6 +4,7 @@
 // and the order in which partial sums meet, is a function of the ROW LENGTH only.  The number of rows
 // only changes how many identical work-groups are launched.  No atomics, no split decided at run time.
 #include "common.h"
+#include "rmsnorm_row.h"
 
 namespace tbik {
 
@@ -29,84 +30,13 @@ struct RmsArgs {
 
 template <int CPL, bool F16>  // chunks (8 elements) per lane kept in registers; bf16 or fp16 elements
 __global__ __launch_bounds__(256) void rmsnorm_kernel(const RmsArgs a) {
-  using Num = Num16<F16>;
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= a.rows) return;
-  const int nchunks = a.hidden >> 3;
-  const uint4* xr = reinterpret_cast<const uint4*>(a.x + row * a.ldx);
-  const uint4* rr = a.res ? reinterpret_cast<const uint4*>(a.res + row * a.ldr) : nullptr;
-
-  // the weights do not depend on the row: fetched together with it, not after the reduction (with a single row
-  // the kernel is nothing but memory round trips in a chain)
-  const uint4* wr = reinterpret_cast<const uint4*>(a.w);
-  uint4 wq[CPL];
-  if (wr) {
-#pragma unroll
-    for (int i = 0; i < CPL; i++) {
-      const int c = lane + 64 * i;
-      if (c < nchunks) wq[i] = wr[c];
-    }
-  }
-
-  // all loads of the row go out before the first store: the residual output may alias the inputs as far as the
-  // compiler knows, and loads issued behind a store would wait for one memory round trip per chunk
-  uint4 xq[CPL], rq[CPL];
-#pragma unroll
-  for (int i = 0; i < CPL; i++) {
-    const int c = lane + 64 * i;
-    if (c < nchunks) {
-      xq[i] = xr[c];
-      if (rr) rq[i] = rr[c];
-    }
-  }
-  float v[CPL][8];
-  float ss = 0.f;
-#pragma unroll
-  for (int i = 0; i < CPL; i++) {
-    const int c = lane + 64 * i;
-    if (c < nchunks) {
-      const uint32_t u[4] = {xq[i].x, xq[i].y, xq[i].z, xq[i].w};
-#pragma unroll
-      for (int e = 0; e < 4; e++) {
-        v[i][2 * e] = Num::lo(u[e]);
-        v[i][2 * e + 1] = Num::hi(u[e]);
-      }
-      if (rr) {
-        const uint32_t ru[4] = {rq[i].x, rq[i].y, rq[i].z, rq[i].w};
-        uint32_t so[4];
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-          v[i][2 * e] += Num::lo(ru[e]);
-          v[i][2 * e + 1] += Num::hi(ru[e]);
-          so[e] = Num::pack(v[i][2 * e], v[i][2 * e + 1]);
-        }
-        if (a.res_out) reinterpret_cast<uint4*>(a.res_out + row * a.ldro)[c] = make_uint4(so[0], so[1], so[2], so[3]);
-      }
-#pragma unroll
-      for (int e = 0; e < 8; e++) ss = fmaf(v[i][e], v[i][e], ss);
-    }
-  }
-  ss = wave_sum(ss);
-  const float var = ss / (float)a.hidden;
-  const float rs = 1.0f / sqrtf(var + a.eps);
   uint4* orow = reinterpret_cast<uint4*>(a.out + row * a.ldo);
-#pragma unroll
-  for (int i = 0; i < CPL; i++) {
-    const int c = lane + 64 * i;
-    if (c < nchunks) {
-      uint32_t o[4];
-#pragma unroll
-      for (int e = 0; e < 4; e++) o[e] = Num::pack(v[i][2 * e] * rs, v[i][2 * e + 1] * rs);
-      if (wr) {
-        const uint32_t wu[4] = {wq[i].x, wq[i].y, wq[i].z, wq[i].w};
-#pragma unroll
-        for (int e = 0; e < 4; e++)
-          o[e] = Num::pack(Num::lo(o[e]) * Num::lo(wu[e]), Num::hi(o[e]) * Num::hi(wu[e]));
-      }
-      orow[c] = make_uint4(o[0], o[1], o[2], o[3]);
-    }
-  }
+  rmsnorm_row<CPL, F16>(a.x + row * a.ldx, a.res ? a.res + row * a.ldr : nullptr, a.w,
+                        a.res_out ? a.res_out + row * a.ldro : nullptr, a.hidden, a.eps, lane,
+                        [&](int c, const uint4& o) { orow[c] = o; });
 }
 
 template <bool F16>

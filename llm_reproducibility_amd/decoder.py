@@ -61,13 +61,16 @@ class _Layer:
 
 class Qwen3Decoder:
     def __init__(self, cfg: DecoderConfig, tp_size: int = 1, seed: int = 0, device="cuda:0", use_graphs: bool = False,
-                 fused_rope: bool = True, init_on_device: bool = False):
+                 fused_rope: bool = True, init_on_device: bool = False, fused_producers: bool = True):
         assert cfg.head_dim == 128, "the attention kernel is built for head_dim 128"
         self.cfg, self.tp_size, self.device = cfg, tp_size, torch.device(device)
         # decode steps replayed from one captured HIP graph (same kernels, same order, same bits as eager; the
         # per-step host work shrinks to one graph launch, which is what bounds small batches)
         self.use_graphs = use_graphs
         self.fused_rope = fused_rope
+        # RMSNorm inside the projection that consumes it and SiLU*up inside down_proj (one launch each for a handful of
+        # rows, the two launches otherwise; bit-identical either way, so the switch only exists for the tests)
+        self.fused_producers = fused_producers
         gen = torch.Generator(device=self.device if init_on_device else "cpu").manual_seed(seed)
         emb = lambda *shape: _normal_bf16(shape, gen, self.device)  # noqa: E731
         self.embed = emb(cfg.vocab_size, cfg.hidden_size)
@@ -101,13 +104,18 @@ class Qwen3Decoder:
         Hq, Hkv, D = cfg.num_q_heads, cfg.num_kv_heads, cfg.head_dim
         x = self.embed[token_ids]                                   # [tokens, H]
         residual: Optional[torch.Tensor] = None
+        fused = self.fused_producers
         for li, layer in enumerate(self.layers):
-            if residual is None:
-                residual = x
-                h = rms_norm(x, layer.input_norm, cfg.rms_eps)
+            if fused:
+                qkv, new_res = ops.rmsnorm_gemm(x, layer.input_norm, cfg.rms_eps, residual, layer.qkv_w.t())
+                residual = x if residual is None else new_res
             else:
-                h, residual = rms_norm(x, layer.input_norm, cfg.rms_eps, residual=residual)
-            qkv = matmul_persistent(h, layer.qkv_w.t())
+                if residual is None:
+                    residual = x
+                    h = rms_norm(x, layer.input_norm, cfg.rms_eps)
+                else:
+                    h, residual = rms_norm(x, layer.input_norm, cfg.rms_eps, residual=residual)
+                qkv = matmul_persistent(h, layer.qkv_w.t())
             k_cache, vt_cache = cache[li]
             if self.fused_rope:
                 # per-head q/k norm, rotary embedding and the cache write in one kernel
@@ -123,12 +131,22 @@ class Qwen3Decoder:
                 vt_cache[seq_of_token, :, :, positions] = v         # stored transposed: [B, Hkv, D, L]
             attn = ops.bi_attention_bf16(q, k_cache, vt_cache, q_start, q_len, ctx_len, max_q_len, self.scale)
             x = layer.o_proj(attn.reshape(-1, Hq * D))
-            h, residual = rms_norm(x, layer.post_norm, cfg.rms_eps, residual=residual)
-            gu = matmul_persistent(h, layer.gate_up_w.t())
-            act = ops.bi_silu_mul(gu)
-            x = layer.down_proj(act)
-        h, _ = rms_norm(x, self.final_norm, cfg.rms_eps, residual=residual)
-        return h
+            if fused:
+                gu, residual = ops.rmsnorm_gemm(x, layer.post_norm, cfg.rms_eps, residual, layer.gate_up_w.t())
+                x = layer.down_proj.forward_gated(gu)
+            else:
+                h, residual = rms_norm(x, layer.post_norm, cfg.rms_eps, residual=residual)
+                gu = matmul_persistent(h, layer.gate_up_w.t())
+                act = ops.bi_silu_mul(gu)
+                x = layer.down_proj(act)
+        return x, residual
+
+    def _logits(self, x: torch.Tensor, residual: torch.Tensor) -> torch.Tensor:
+        """Final norm and lm_head for the given rows (the norm is per row, so rows may be selected first)."""
+        if self.fused_producers:
+            return ops.rmsnorm_gemm(x, self.final_norm, self.cfg.rms_eps, residual, self.lm_head.t())[0]
+        h, _ = rms_norm(x, self.final_norm, self.cfg.rms_eps, residual=residual)
+        return matmul_persistent(h, self.lm_head.t())
 
     @staticmethod
     def _greedy(logits: torch.Tensor) -> torch.Tensor:
@@ -157,9 +175,9 @@ class Qwen3Decoder:
         q_start = torch.tensor(starts, dtype=torch.int32, device=dev)
         q_len = torch.tensor(lens, dtype=torch.int32, device=dev)
         ctx = torch.tensor(lens, dtype=torch.int32, device=dev)
-        h = self._forward(tok, pos, seq, q_start, q_len, ctx, max(lens), cache)
+        x, res = self._forward(tok, pos, seq, q_start, q_len, ctx, max(lens), cache)
         last = torch.tensor([s + n - 1 for s, n in zip(starts, lens)], dtype=torch.long, device=dev)
-        logits = matmul_persistent(h[last].contiguous(), self.lm_head.t())
+        logits = self._logits(x[last].contiguous(), res[last].contiguous())
         out_ids = [self._greedy(logits)]
         all_logits = [logits] if return_logits else None
         # ---- decode: one token per sequence per step
@@ -172,8 +190,7 @@ class Qwen3Decoder:
         ctx_s = (pos_s + 1).to(torch.int32)
 
         def step():
-            h = self._forward(tok_s, pos_s, seq, q_start, q_len, ctx_s, 1, cache)
-            logits = matmul_persistent(h, self.lm_head.t())
+            logits = self._logits(*self._forward(tok_s, pos_s, seq, q_start, q_len, ctx_s, 1, cache))
             nxt = self._greedy(logits)
             tok_s.copy_(nxt)
             pos_s.add_(1)

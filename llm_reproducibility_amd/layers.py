@@ -114,6 +114,24 @@ class SimulatedTPRowLinear(nn.Module):
             out = out + self.bias
         return out.reshape(*lead, out.shape[-1])
 
+    def forward_gated(self, gate_up: torch.Tensor) -> torch.Tensor:
+        """forward(silu(gate) * up) for the merged projection gate_up = [gate | up]: the activation is formed inside the
+        per-shard tree matmul where that is one launch (a few rows), by its own kernel otherwise; same bits."""
+        from . import ops
+        lead = gate_up.shape[:-1]
+        g2 = gate_up.reshape(-1, gate_up.shape[-1])
+        K = g2.shape[1] // 2
+        assert K == self.weight.shape[1]
+        if g2.shape[0] > 4 or g2.dtype != torch.bfloat16:
+            return self.forward(ops.bi_silu_mul(g2)).reshape(*lead, self.weight.shape[0])
+        ks = K // self.tp_size
+        parts = [ops.gemm_tree_silu_mul(g2[:, r * ks:(r + 1) * ks], g2[:, K + r * ks:K + (r + 1) * ks],
+                                        self.weight[:, r * ks:(r + 1) * ks].t(), None, self.leaf_k) for r in range(self.tp_size)]
+        out = parts[0] if self.tp_size == 1 else tree_combine(parts)
+        if self.bias is not None:
+            out = out + self.bias
+        return out.reshape(*lead, out.shape[-1])
+
 
 class RMSNorm(nn.Module):
     """RMSNorm with vLLM's call shape: forward(x, residual=None) -> out | (out, new_residual)."""

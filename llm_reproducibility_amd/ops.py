@@ -426,6 +426,70 @@ def _(gate_up):
 
 
 # --------------------------------------------------------------------------------------------
+# one-launch compositions for decode-sized batches (bit-identical to the two-launch forms they fall back to)
+# --------------------------------------------------------------------------------------------
+def rmsnorm_gemm(x: torch.Tensor, norm_weight: Optional[torch.Tensor], eps: float, residual: Optional[torch.Tensor],
+                 B: torch.Tensor, bias: Optional[torch.Tensor] = None):
+    """(bi_gemm(rms_norm(x [+ residual]) * norm_weight, B) (+ bias), new residual or None).
+
+    One launch (`bi_rmsnorm_gemm_bf16`: the matmul normalises the activations while it stages them) for a few bf16 rows
+    against an nn.Linear weight handed over as `weight.t()`; the two launches otherwise.  Same bits either way."""
+    _require_gpu(x, norm_weight, residual, B, bias)
+    M, K = x.shape
+    N = B.shape[1]
+    fusable = (x.dtype == torch.bfloat16 and B.dtype == torch.bfloat16 and M * K <= 32768 and K <= 8192 and K % 32 == 0
+               and B.stride(0) == 1 and not torch.compiler.is_compiling())
+    if fusable:
+        x2, ldx = _rows16(x)
+        r2, ldr = (None, 0) if residual is None else _rows16(residual)
+        w, ldb_k, ldb_n = _weight_operand(B)
+        nw = None if norm_weight is None else norm_weight.contiguous()
+        b = None if bias is None else bias.contiguous()
+        C = torch.empty((M, N), device=x.device, dtype=x.dtype)
+        rout = None if residual is None else torch.empty((M, K), device=x.device, dtype=x.dtype)
+        rc = _lib.lib().bi_rmsnorm_gemm_bf16(x2.data_ptr(), ldx, None if r2 is None else r2.data_ptr(), ldr,
+                                             None if nw is None else nw.data_ptr(), eps,
+                                             None if rout is None else rout.data_ptr(), K, w.data_ptr(), ldb_k, ldb_n,
+                                             C.data_ptr(), C.stride(0), M, N, K, None if b is None else b.data_ptr(), _stream(x))
+        if rc == _lib.TBIK_OK:
+            return C, rout
+        if rc != _lib.TBIK_ERR_UNSUPPORTED:
+            _lib.check(rc, "bi_rmsnorm_gemm_bf16")
+    if residual is None:
+        h, rout = bi_rmsnorm(x, norm_weight, eps), None
+    else:
+        h, rout = bi_add_rmsnorm(x, residual, norm_weight, eps)
+    return bi_gemm(h, B, bias), rout
+
+
+def gemm_tree_silu_mul(gate: torch.Tensor, up: torch.Tensor, B: torch.Tensor, bias: Optional[torch.Tensor], leaf_k: int) -> torch.Tensor:
+    """gemm_tree(silu(gate) * up, B, bias, leaf_k) for the two halves (or a K shard of both halves) of a merged gate/up
+    projection: column slices of one tensor, same row stride.
+
+    One launch (`tbik_gemm_silu_mul_bf16`) for a few bf16 rows, the activation kernel followed by the tree matmul
+    otherwise.  Same bits either way."""
+    _require_gpu(gate, up, B, bias)
+    M, K = gate.shape
+    N = B.shape[1]
+    fusable = (gate.dtype == torch.bfloat16 and B.dtype == torch.bfloat16 and M <= 4 and up.shape == gate.shape
+               and gate.stride(1) == 1 and up.stride(1) == 1 and gate.stride(0) == up.stride(0) and gate.stride(0) % 8 == 0
+               and _aligned16(gate) and _aligned16(up) and B.stride(0) == 1 and not torch.compiler.is_compiling())
+    if fusable:
+        w, ldb_k, ldb_n = _weight_operand(B)
+        b = None if bias is None else bias.contiguous()
+        C = torch.empty((M, N), device=gate.device, dtype=gate.dtype)
+        rc = _lib.lib().tbik_gemm_silu_mul_bf16(gate.data_ptr(), up.data_ptr(), gate.stride(0) if M > 1 else max(gate.stride(0), K),
+                                                w.data_ptr(), ldb_k, ldb_n, C.data_ptr(), C.stride(0), M, N, K, leaf_k,
+                                                None if b is None else b.data_ptr(), _stream(gate))
+        if rc == _lib.TBIK_OK:
+            return C
+        if rc != _lib.TBIK_ERR_UNSUPPORTED:
+            _lib.check(rc, "tbik_gemm_silu_mul_bf16")
+    act = bi_silu_mul(torch.cat((gate, up), dim=-1))
+    return gemm_tree(act, B, bias, leaf_k)
+
+
+# --------------------------------------------------------------------------------------------
 # q/k norm + rotary embedding + KV-cache write in front of the attention
 # --------------------------------------------------------------------------------------------
 def bi_qk_norm_rope_cache_bf16(qkv: torch.Tensor, q_weight: torch.Tensor, k_weight: torch.Tensor, inv_freq: torch.Tensor,

@@ -447,6 +447,10 @@ def test_silu_mul_parity_and_batch_invariance(dev):
     got = ops.bi_silu_mul(gu.to(dev))
     assert got.shape == want.shape
     assert O.bf16_ulp_distance(got.cpu(), want).max().item() <= 1   # device exp vs host exp: at most one rounding flip
+    # gate = 5.9375 is a hard case: silu = 5.92187444, 1.2 fp32 steps below the bf16 boundary 5.921875 -- a quotient
+    # that is off by more than one fp32 step lands on the other side
+    hard = torch.tensor([[5.9375] * 8 + [-2.375, 0.6171875, 2.4375, -2.34375, 0.1669921875, 7.96875, 1.0, -1.0]], dtype=torch.bfloat16)
+    assert torch.equal(ops.bi_silu_mul(hard.to(dev)).cpu(), O.silu_mul(hard))
     for rows in (1, 7, 256):
         assert torch.equal(ops.bi_silu_mul(gu[:rows].to(dev)), got[:rows])
     # a strided view (row stride larger than the row) and a 3-D input
