@@ -262,7 +262,9 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const typename
 #pragma unroll
         for (int a = 0; a < TM; a++) {
 #pragma unroll
-          for (int b = 0; b < TN; b++) {
+          for (int bb = 0; bb < TN; bb++) {
+            // rows of tiles in alternating directions: every MFMA changes ONE of its operands
+            const int b = (a & 1) ? TN - 1 - bb : bb;
             const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
             acc[a][b] = NUM::mfma(fw[b], fx[a], (i == 0 && kk == 0) ? zero : acc[a][b]);
           }
@@ -273,7 +275,7 @@ __global__ __launch_bounds__(wide::NT) void gemm_tree_wide_kernel(const typename
           const int d = kk * TM + a;  // 0..7: loads 0..5 go out after MFMA rows 0..5
           if (d < NDMA) {
             __builtin_amdgcn_sched_barrier(0);
-            dma16(pdst + d * 8192, voff[d], d < 2 ? pxb : pwb);
+            dma16_at(pdst, d * 8192, voff[d], d < 2 ? pxb : pwb);
             __builtin_amdgcn_sched_barrier(0);
           }
         }

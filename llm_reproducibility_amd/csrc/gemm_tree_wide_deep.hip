@@ -264,7 +264,10 @@ __global__ __launch_bounds__(deep::NT) void gemm_tree_deep_kernel(const typename
 #pragma unroll
         for (int a = 0; a < TM; a++) {
 #pragma unroll
-          for (int b = 0; b < TN; b++) {
+          for (int bb = 0; bb < TN; bb++) {
+            // rows of tiles in alternating directions: every MFMA then changes ONE of its operands, never both at the
+            // turn of a row (an MFMA-only loop on random operands runs 2 % faster at the same power this way)
+            const int b = (a & 1) ? TN - 1 - bb : bb;
             const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
             acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[b], fx[a], (i == 0 && kk == 0) ? zero : acc[a][b], 0, 0, 0);
           }
@@ -273,7 +276,7 @@ __global__ __launch_bounds__(deep::NT) void gemm_tree_deep_kernel(const typename
           const int d = kk * TM + a;
           if (d < NDMA) {
             __builtin_amdgcn_sched_barrier(0);
-            dma16(pdst + d * 8192, voff[d], d < 2 ? pxb : pwb);
+            dma16_at(pdst, d * 8192, voff[d], d < 2 ? pxb : pwb);
             __builtin_amdgcn_sched_barrier(0);
           }
         }

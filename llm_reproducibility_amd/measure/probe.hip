@@ -12,6 +12,7 @@ namespace tbik {
 // One work-group per CU (the launch requests 100 KiB of dynamic LDS, which keeps a second one out), WAVES wavefronts each with a 4x4 block of 16x16
 // accumulators, the shape of the 64x64 wave tile of the tree GEMM.  Operands come from `src` (4096 x 16 bytes) once
 // and stay in registers: no loads, no LDS, no other instruction in the loop.
+template <int ORDER>  // 0: tiles row by row; 1: rows in alternating directions, so that every MFMA changes ONE operand
 __global__ __launch_bounds__(512) void probe_mfma_kernel(const bf16x8* __restrict__ src, float* __restrict__ out, int iters) {
   f32x4 acc[4][4];
   bf16x8 a[4], b[4];
@@ -26,7 +27,10 @@ __global__ __launch_bounds__(512) void probe_mfma_kernel(const bf16x8* __restric
 #pragma unroll
     for (int i = 0; i < 4; i++)
 #pragma unroll
-      for (int j = 0; j < 4; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+      for (int jj = 0; jj < 4; jj++) {
+        const int j = (ORDER == 1 && (i & 1)) ? 3 - jj : jj;
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+      }
   }
   float s = 0.f;
 #pragma unroll
@@ -48,14 +52,22 @@ __global__ __launch_bounds__(256) void probe_read_kernel(const uint4* __restrict
 }
 
 int probe_mfma_dispatch(const void* operands, void* out, int work_groups, int waves, int iters, hipStream_t stream) {
-  if (!operands || !out || work_groups <= 0 || iters <= 0 || (waves != 4 && waves != 8)) return TBIK_ERR_INVALID;
+  if (!operands || !out || work_groups <= 0 || iters == 0 || (waves != 4 && waves != 8)) return TBIK_ERR_INVALID;
   if (reinterpret_cast<uintptr_t>(operands) & 15) return TBIK_ERR_ALIGNMENT;
   constexpr int lds = 100 * 1024;
   static std::atomic<uint64_t> done{0};
-  hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(probe_mfma_kernel), lds, done);
+  static std::atomic<uint64_t> done1{0};
+  const bool snake = iters < 0;   // a negative count selects the alternating tile order
+  if (snake) iters = -iters;
+  hipError_t e = snake ? ensure_dynamic_lds(reinterpret_cast<const void*>(probe_mfma_kernel<1>), lds, done1)
+                       : ensure_dynamic_lds(reinterpret_cast<const void*>(probe_mfma_kernel<0>), lds, done);
   if (e != hipSuccess) return hip_code(e);
-  hipLaunchKernelGGL(probe_mfma_kernel, dim3((unsigned)work_groups), dim3(64 * waves), lds, stream,
-                     static_cast<const bf16x8*>(operands), static_cast<float*>(out), iters);
+  if (snake)
+    hipLaunchKernelGGL(probe_mfma_kernel<1>, dim3((unsigned)work_groups), dim3(64 * waves), lds, stream,
+                       static_cast<const bf16x8*>(operands), static_cast<float*>(out), iters);
+  else
+    hipLaunchKernelGGL(probe_mfma_kernel<0>, dim3((unsigned)work_groups), dim3(64 * waves), lds, stream,
+                       static_cast<const bf16x8*>(operands), static_cast<float*>(out), iters);
   return hip_code(hipGetLastError());
 }
 
