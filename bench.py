@@ -161,7 +161,7 @@ def ceiling(settle_ms):
     return res
 
 
-def table(steps, warmup, hot=False, settle_ms=20.0, full=False):
+def table(steps, warmup, hot=False, settle_ms=20.0, full=False, only=None):
     """Per-shape figures, each after `settle_ms` of the same call run back to back (the settled rate, as for the
     headline).  Unless `hot`, every case cycles through enough distinct input sets (more than 768 MB in all) that
     nothing it reads is still in the 256 MB memory-side cache from the previous call: the GB/s are HBM figures, as in
@@ -194,7 +194,7 @@ def table(steps, warmup, hot=False, settle_ms=20.0, full=False):
 
     def add(name, make, fn, flop, nbytes, bound, nsteps=None, short=None):
         """`short`: the key of the row in the JSON line; rows without one appear in the long form only."""
-        if short is None and not full:
+        if (short is None and not full) or (only and only not in name):
             return
         ms, _ = hip_time_ms(cycling(make, nbytes, fn), nsteps or steps, warmup, settle_ms)
         tf, gbs = flop / ms / 1e9, nbytes / ms / 1e6
@@ -297,6 +297,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--table", action="store_true", help="long form of the per-shape table, also printed to stderr")
     ap.add_argument("--table-hot", action="store_true", help="reuse one input set per table case (cache-hot figures)")
+    ap.add_argument("--only", default=None, help="with --table: only the cases whose name contains this (for profiler runs)")
     ap.add_argument("--no-context-table", action="store_true", help="leave the per-shape table out of the JSON line")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--settle-ms", type=float, default=60.0,
@@ -372,7 +373,7 @@ def main():
         context["ceiling"] = ceiling(args.settle_ms)
     if args.table or not args.no_context_table:
         t0 = time.perf_counter()
-        rows = table(12, 3, hot=args.table_hot, settle_ms=min(args.settle_ms, 10.0), full=args.table)
+        rows = table(12, 3, hot=args.table_hot, settle_ms=min(args.settle_ms, 10.0), full=args.table, only=args.only)
         if args.table:
             print_table(rows, args.table_hot)
         # terse in the JSON line: case -> [us per call, algorithmic work of a call (flop when the bound is "m", bytes when

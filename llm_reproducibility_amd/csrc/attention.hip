@@ -33,6 +33,50 @@ struct AttnArgs {
 
 constexpr int HD = 128;
 
+// One online-softmax update of a query row for a tile of 32 keys, shared by all kernels of this file (one body: the same
+// bits).  Lane (j, g) holds the scores of query j for keys k0 + 16u + 4g + i in s[u][i]; on return p holds the four packed
+// probability pairs of the lane (the B operand of the P*V MFMA) and alpha the factor for the output accumulators of the
+// row (exactly 1.0 when the running maximum did not move).  MASK: apply the causal mask (needed only for tiles that
+// reach beyond some row's horizon; the values are the same either way for the others).
+// 2^x is the hardware exponential: the arguments are <= 0, and a result below 2^-126 is dropped, which neither the
+// denominator (>= 1: the row's maximum contributes 2^0) nor a bf16 probability can show.
+template <bool MASK>
+__device__ __forceinline__ void softmax_tile(const f32x4 (&s)[2], int k0, int g, int qpos, float scale_log2, float& m, float& l,
+                                             float& alpha, bf16x8& p) {
+  // every product and sum below is rounded on its own, except the one fused update of the denominator: left to the
+  // compiler, the scaling of a score could be fused with the subtraction of the maximum in one instantiation and not
+  // in another, and the kernels would no longer agree bit for bit
+#pragma clang fp contract(off)
+  float sv[8];
+#pragma unroll
+  for (int u = 0; u < 2; u++)
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      float v = s[u][i] * scale_log2;
+      if (MASK) v = (k0 + 16 * u + 4 * g + i <= qpos) ? v : -INFINITY;
+      sv[4 * u + i] = v;
+    }
+  float tmax = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
+  tmax = xor_step<16, LaneMax>(tmax);
+  tmax = xor_step<32, LaneMax>(tmax);
+  const float m_new = fmaxf(m, tmax);          // key 0 is visible to every query: m_new is finite from tile 0 on
+  alpha = __builtin_amdgcn_exp2f(m - m_new);   // exactly 1.0 when the tile adds nothing new
+  float psum = 0.f;
+  float pv[8];
+#pragma unroll
+  for (int e = 0; e < 8; e++) {
+    pv[e] = __builtin_amdgcn_exp2f(sv[e] - m_new);
+    psum += pv[e];
+  }
+  psum = xor_step<16, LaneSum>(psum);
+  psum = xor_step<32, LaneSum>(psum);
+  l = __builtin_fmaf(l, alpha, psum);
+  m = m_new;
+  // P as the MFMA "B" operand: k slots 0..3 = keys k0+4g.., slots 4..7 = keys k0+16+4g..
+  p = __builtin_bit_cast(bf16x8, u32x4{pack_bf16x2(pv[0], pv[1]), pack_bf16x2(pv[2], pv[3]), pack_bf16x2(pv[4], pv[5]),
+                                       pack_bf16x2(pv[6], pv[7])});
+}
+
 __global__ __launch_bounds__(64) void attention_kernel(const AttnArgs a) {
   const int b = blockIdx.z;
   const int h = blockIdx.y;
@@ -81,36 +125,9 @@ __global__ __launch_bounds__(64) void attention_kernel(const AttnArgs a) {
       }
       s[u] = acc;
     }
-    float sv[8];
-    float tmax = -INFINITY;
-#pragma unroll
-    for (int u = 0; u < 2; u++)
-#pragma unroll
-      for (int i = 0; i < 4; i++) {
-        const int key = k0 + 16 * u + 4 * g + i;
-        const float v = (key <= qpos) ? s[u][i] * a.scale_log2 : -INFINITY;
-        sv[4 * u + i] = v;
-        tmax = fmaxf(tmax, v);
-      }
-    tmax = xor_step<16, LaneMax>(tmax);
-    tmax = xor_step<32, LaneMax>(tmax);
-    const float m_new = fmaxf(m, tmax);          // key 0 is visible to every query: m_new is finite from tile 0 on
-    const float alpha = exp2f(m - m_new);         // exactly 1.0 when the tile adds nothing new
-    float psum = 0.f;
-    float pv[8];
-#pragma unroll
-    for (int e = 0; e < 8; e++) {
-      pv[e] = exp2f(sv[e] - m_new);
-      psum += pv[e];
-    }
-    psum = xor_step<16, LaneSum>(psum);
-    psum = xor_step<32, LaneSum>(psum);
-    l = l * alpha + psum;
-    m = m_new;
-    // P as the MFMA "B" operand: k slots 0..3 = keys k0+4g.., slots 4..7 = keys k0+16+4g..
-    const uint32_t p0 = pack_bf16x2(pv[0], pv[1]), p1 = pack_bf16x2(pv[2], pv[3]);
-    const uint32_t p2 = pack_bf16x2(pv[4], pv[5]), p3 = pack_bf16x2(pv[6], pv[7]);
-    const bf16x8 pf = __builtin_bit_cast(bf16x8, u32x4{p0, p1, p2, p3});
+    float alpha;
+    bf16x8 pf;
+    softmax_tile<true>(s, k0, g, qpos, a.scale_log2, m, l, alpha, pf);
     // ---- out^T += V^T * P: "A" operand lane (j, g) holds channel 16t + j, the same 8 key slots
     const int kv0 = min(k0 + 4 * g, a.max_len - 4);
     const int kv1 = min(k0 + 16 + 4 * g, a.max_len - 4);
@@ -138,7 +155,8 @@ __global__ __launch_bounds__(64) void attention_kernel(const AttnArgs a) {
 // ------------------------------------------------------------------------------------------------
 // Grouped variant: one work-group per (16 consecutive queries, KV head, sequence); its G wavefronts are the G query
 // heads that share the KV head.  Each 32-key tile of K and of V^T is fetched from global memory ONCE per group with
-// coalesced 16-byte loads, staged in LDS (double buffered, XOR-swizzled against bank conflicts) and read from there
+// coalesced 16-byte loads, staged in LDS (double buffered; K rows XOR-swizzled against bank conflicts, V^T rows stored in
+// fragment order) and read from there
 // by every wave.  A row's arithmetic -- the lanes that own it, the MFMA chain, the order of the softmax updates --
 // is exactly that of attention_kernel above, so both kernels produce the same bits; this one just moves 1/G of
 // the bytes and hides the load latency behind the previous tile.
@@ -202,8 +220,14 @@ __global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs 
       if (512 % NT == 0 || ch < 512) {
         const int kr = ch >> 4, kc = ch & 15;   // key row, 16-byte chunk of its 256 bytes
         *reinterpret_cast<u32x4*>(&lds[buf][kr * 256 + ((kc ^ (2 * (kr & 7))) << 4)]) = kreg[i];
-        const int vr = ch >> 2, vc = ch & 3;    // channel row, 16-byte chunk of its 64 bytes
-        *reinterpret_cast<u32x4*>(&lds[buf][8192 + vr * 64 + ((vc ^ ((vr >> 2) & 3)) << 4)]) = vreg[i];
+        // V^T: channel row vr (64 bytes = 32 keys), 16-byte chunk vc = keys 8vc .. 8vc+7.  The keys of a row are stored
+        // in the order a P*V fragment wants them -- lane group g takes keys 4g..4g+3 and 16+4g..16+4g+3 -- so that a
+        // fragment is ONE 16-byte read at byte 16g of the row: keys 4a..4a+3 live in the 8-byte slot 2 (a & 3) + (a >> 2).
+        // A wave then reads sixteen consecutive rows as one linear KiB (no bank conflicts, no swizzle).
+        const int vr = ch >> 2, vc = ch & 3;
+        const int slot0 = 2 * ((2 * vc) & 3) + (vc >> 1), slot1 = 2 * ((2 * vc + 1) & 3) + (vc >> 1);
+        *reinterpret_cast<uint2*>(&lds[buf][8192 + vr * 64 + slot0 * 8]) = make_uint2(vreg[i][0], vreg[i][1]);
+        *reinterpret_cast<uint2*>(&lds[buf][8192 + vr * 64 + slot1 * 8]) = make_uint2(vreg[i][2], vreg[i][3]);
       }
     }
   };
@@ -213,6 +237,14 @@ __global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs 
   for (int t = 0; t < 8; t++) o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY;
   float l = 0.f;
+
+  // LDS offsets of this lane's fragments inside a tile buffer, formed once: key row 16u + j of the K tile (256 bytes a
+  // row, 16-byte chunk c*4 + g swizzled by the row; u adds 4096), channel row 16t + j of the V^T tile (64 bytes a row,
+  // the lane group's eight keys are the 16 bytes at 16g; t adds 1024)
+  uint32_t kofs[4];
+#pragma unroll
+  for (int c = 0; c < 4; c++) kofs[c] = j * 256 + (((c * 4 + g) ^ (2 * (j & 7))) << 4);
+  const uint32_t vofs = 8192 + j * 64 + g * 16;
 
   const int ntiles = last_pos / 32 + 1;
   // loads past the last tile are clamped to a valid address and never used: issuing them unconditionally keeps the
@@ -229,61 +261,26 @@ __global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs 
     const int cur = tile & 1;
     load_tile(tile + DEPTH, d);  // set d held this tile and went to LDS a tile ago
     const int k0 = tile * 32;
+    const uint8_t* tb = &lds[cur][0];
     f32x4 s[2];
 #pragma unroll
     for (int u = 0; u < 2; u++) {
-      const int kr = 16 * u + j;
-      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+      const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+      f32x4 acc;
 #pragma unroll
       for (int c = 0; c < 4; c++) {
-        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(&lds[cur][kr * 256 + (((c * 4 + g) ^ (2 * (kr & 7))) << 4)]);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[c], acc, 0, 0, 0);
+        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(tb + kofs[c] + u * 4096);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[c], c == 0 ? zero : acc, 0, 0, 0);
       }
       s[u] = acc;
     }
-    float sv[8];
-    float tmax = -INFINITY;
     // only the tiles on the causal diagonal need the mask: when every key of the tile is visible to every query of
     // this wave (a uniform condition) the selects are skipped; the values are the same either way.  Prefill only:
     // in decode the tile loop is one dependent chain and a branch on a freshly computed value lengthens it.
-    if (!DEEP && __builtin_amdgcn_ballot_w64(k0 + 31 > qpos) == 0) {
-#pragma unroll
-      for (int u = 0; u < 2; u++)
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-          const float v = s[u][i] * a.scale_log2;
-          sv[4 * u + i] = v;
-          tmax = fmaxf(tmax, v);
-        }
-    } else {
-#pragma unroll
-      for (int u = 0; u < 2; u++)
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-          const int key = k0 + 16 * u + 4 * g + i;
-          const float v = (key <= qpos) ? s[u][i] * a.scale_log2 : -INFINITY;
-          sv[4 * u + i] = v;
-          tmax = fmaxf(tmax, v);
-        }
-    }
-    tmax = xor_step<16, LaneMax>(tmax);
-    tmax = xor_step<32, LaneMax>(tmax);
-    const float m_new = fmaxf(m, tmax);
-    const float alpha = exp2f(m - m_new);
-    float psum = 0.f;
-    float pv[8];
-#pragma unroll
-    for (int e = 0; e < 8; e++) {
-      pv[e] = exp2f(sv[e] - m_new);
-      psum += pv[e];
-    }
-    psum = xor_step<16, LaneSum>(psum);
-    psum = xor_step<32, LaneSum>(psum);
-    l = l * alpha + psum;
-    m = m_new;
-    const uint32_t p0 = pack_bf16x2(pv[0], pv[1]), p1 = pack_bf16x2(pv[2], pv[3]);
-    const uint32_t p2 = pack_bf16x2(pv[4], pv[5]), p3 = pack_bf16x2(pv[6], pv[7]);
-    const bf16x8 pf = __builtin_bit_cast(bf16x8, u32x4{p0, p1, p2, p3});
+    float alpha;
+    bf16x8 pf;
+    if (!DEEP && __builtin_amdgcn_ballot_w64(k0 + 31 > qpos) == 0) softmax_tile<false>(s, k0, g, qpos, a.scale_log2, m, l, alpha, pf);
+    else softmax_tile<true>(s, k0, g, qpos, a.scale_log2, m, l, alpha, pf);
     // rescale the output accumulators only when some row's maximum moved (uniform over the wave): x * 1.0f is x bit
     // for bit, and after the first tiles of a long row the maximum rarely moves (prefill only, as above)
     if (DEEP || __builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
@@ -292,11 +289,7 @@ __global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs 
     }
 #pragma unroll
     for (int t = 0; t < 8; t++) {
-      const int vr = 16 * t + j;
-      const int sw = 2 * ((vr >> 2) & 3);  // 8-byte slots: keys 4g.. sit in slot g, keys 16+4g.. in slot 4+g
-      const uint2 va = *reinterpret_cast<const uint2*>(&lds[cur][8192 + vr * 64 + ((g ^ sw) << 3)]);
-      const uint2 vb = *reinterpret_cast<const uint2*>(&lds[cur][8192 + vr * 64 + (((4 + g) ^ sw) << 3)]);
-      const bf16x8 vf = __builtin_bit_cast(bf16x8, u32x4{va.x, va.y, vb.x, vb.y});
+      const bf16x8 vf = *reinterpret_cast<const bf16x8*>(tb + vofs + t * 1024);
       o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[t], 0, 0, 0);
     }
     if (tile + 1 < ntiles) store_tile(cur ^ 1, (d + 1) % DEPTH);
