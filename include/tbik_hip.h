@@ -90,7 +90,8 @@ size_t tbik_gemm_workspace_bytes_rowmajor_b(int M, int N, int K, int leaf_k, int
  * harnesses that forbid hipMalloc.  Same arguments (without the workspace), same kernels, same bits; the workspace is
  * a fixed array of TBIK_STATIC_SCRATCH_BYTES inside the library, one copy per GPU, held until the process ends.  A
  * problem whose tbik_gemm_workspace_bytes() exceeds that size returns TBIK_ERR_SCRATCH_LIMIT before anything is
- * launched (decode- and mid-sized batches fit; the 2048-row benchmark shape does not).  The call allocates and frees
+ * launched (decode- and mid-sized batches fit, and so does the 2048-row benchmark shape, whose two parked tree levels
+ * are 32 MiB; the 4096-row shapes of the 32B configuration do not).  The call allocates and frees
  * nothing.  The first call on a device resolves the array's device address (hipGetSymbolAddress): make that call
  * outside a graph capture.  Every call on a GPU uses that GPU's one array, whose contents are scratch (written
  * before they are read, nothing has to start at zero): two calls that overlap in time on one GPU -- different
