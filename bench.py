@@ -71,6 +71,61 @@ def hip_time_ms(fn, steps, warmup, settle_ms=0.0):
     return s.elapsed_time(e) / steps, wall_ms / steps
 
 
+class PowerSampler:
+    """Board power while a loop runs, read from the driver's hwmon file (microwatts, `power1_input` or `power1_average`
+    of the first GPU) every 20 ms on a thread of its own; `mean_w()` drops the first quarter of the samples (ramp-up).
+    None where the file does not exist."""
+
+    def __init__(self):
+        import glob
+        import threading
+        paths = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input") +
+                       glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_average"))
+        self.path = paths[0] if paths else None
+        self.samples, self._stop = [], False
+        self._thread = threading.Thread(target=self._run, daemon=True)
+
+    def _run(self):
+        while not self._stop:
+            try:
+                with open(self.path) as f:
+                    self.samples.append(int(f.read().strip()) * 1e-6)
+            except (OSError, ValueError):
+                pass
+            time.sleep(0.02)
+
+    def __enter__(self):
+        if self.path:
+            self._thread.start()
+        return self
+
+    def __exit__(self, *exc):
+        self._stop = True
+        if self.path:
+            self._thread.join()
+
+    def mean_w(self):
+        s = self.samples[len(self.samples) // 4:]
+        return round(sum(s) / len(s), 1) if s else None
+
+
+def power_of(fn, seconds=1.5):
+    """(mean board power in W, microseconds per call) of `fn` run back to back for about `seconds`."""
+    import torch
+    for _ in range(20):
+        fn()
+    torch.cuda.synchronize()
+    n, t0 = 0, time.perf_counter()
+    with PowerSampler() as ps:
+        while time.perf_counter() - t0 < seconds:
+            for _ in range(50):
+                fn()
+            torch.cuda.synchronize()
+            n += 50
+        dt = time.perf_counter() - t0
+    return ps.mean_w(), round(dt / n * 1e6, 1)
+
+
 def _median_time(fn, budget_s, max_runs, min_runs=3):
     ts, spent = [], 0.0
     while (spent < budget_s or len(ts) < min_runs) and len(ts) < max_runs:
@@ -117,10 +172,13 @@ def cpu_baseline(budget_s=9.0, max_runs=30):
     return rec, want
 
 
-def ceiling(settle_ms):
+def ceiling(settle_ms, others=()):
     """What the chip sustains on bf16 MFMAs alone (register operands, one work-group per CU, 2 waves per SIMD: the wave
     shape of the tree kernel) for constant and for random operands, and on a one-pass read of 1 GiB (cold in the 256 MB
-    memory-side cache).  Steady-state figures (same load phase as the headline)."""
+    memory-side cache).  Steady-state figures (same load phase as the headline).  `power_W`: the board power while each
+    of these loops, and each (name, fn) of `others`, runs back to back for 1.5 s (the cap of this board is what
+    `rocm-smi --showmaxpower` prints, 1400 W on MI355X): a kernel that sits at the cap is bound by energy per launch,
+    not by a pipe."""
     import ctypes
     import torch
     from llm_reproducibility_amd import _lib
@@ -144,7 +202,7 @@ def ceiling(settle_ms):
         buf = src.to(torch.bfloat16).to(dev)
 
         def run():
-            _lib.check(L.tbik_probe_mfma_bf16(buf.data_ptr(), out.data_ptr(), cus, 8, iters, stream), "tbik_probe_mfma_bf16")
+            _lib.check(L.tbik_probe_mfma_bf16(buf.data_ptr(), out.data_ptr(), cus, 8, -iters, stream), "tbik_probe_mfma_bf16")
         ms, _ = hip_time_ms(run, 30, 5, settle_ms)
         flop = float(cus) * 8 * iters * 16 * 16384
         res[f"mfma_only_{name}_operands_TFLOPs"] = round(flop / (ms * 1e-3) / 1e12, 1)
@@ -156,6 +214,17 @@ def ceiling(settle_ms):
         _lib.check(L.tbik_probe_read(big.data_ptr(), nbytes, sink.data_ptr(), cus * 16, stream), "tbik_probe_read")
     ms, _ = hip_time_ms(read, 20, 3, settle_ms)
     res["one_pass_read_1GiB_GBps"] = round(nbytes / (ms * 1e-3) / 1e9, 1)
+    power = {}
+    for name, src in (("mfma_only_constant", torch.full((32768,), 1.0)), ("mfma_only_random", ops_rand)):
+        buf = src.to(torch.bfloat16).to(dev)
+        power[name] = power_of(lambda: L.tbik_probe_mfma_bf16(buf.data_ptr(), out.data_ptr(), cus, 8, -iters, stream))
+    for name, fn in others:
+        power[name] = power_of(fn)
+    time.sleep(2.0)
+    with PowerSampler() as ps:
+        time.sleep(1.0)
+    power["idle"] = (ps.mean_w(), None)
+    res["power_W_and_us_per_call"] = power
     res["note"] = ("MFMA-only loop on register operands and a plain grid-stride read: ceilings of any bf16 matmul kernel "
                    "on such data and of any one-pass kernel, measured in this run")
     return res
@@ -370,7 +439,9 @@ def main():
     mm_ms, _ = hip_time_ms(lambda: bio.matmul_persistent(X, Wt), args.steps, args.warmup, args.settle_ms)
     context["single_accumulator_mm_same_operands_TFLOPs"] = round(flops / (mm_ms * 1e-3) / 1e12, 2)
     if args.ceiling:
-        context["ceiling"] = ceiling(args.settle_ms)
+        context["ceiling"] = ceiling(args.settle_ms, (("tree_matmul_headline", step),
+                                                      ("single_accumulator_mm_same_operands", lambda: bio.matmul_persistent(X, Wt)),
+                                                      ("vendor_gemm_same_operands", lambda: torch.matmul(X, Wt))))
     if args.table or not args.no_context_table:
         t0 = time.perf_counter()
         rows = table(12, 3, hot=args.table_hot, settle_ms=min(args.settle_ms, 10.0), full=args.table, only=args.only)

@@ -1,7 +1,7 @@
 """Turns the CSV files of a rocprofv3 run into the short text tables kept under profiles/.
 
     python -m llm_reproducibility_amd.measure.summarise kernels  DIR [--only tbik::] [--sequence SUBSTRING]
-    python -m llm_reproducibility_amd.measure.summarise counters DIR [--kernel SUBSTRING] [--largest N] [--copy-kib KIB]
+    python -m llm_reproducibility_amd.measure.summarise counters DIR [--kernel SUBSTRING] [--largest N] [--copy-kib KIB] [--by-grid]
     python -m llm_reproducibility_amd.measure.summarise decode   DIR --layers L --steps S
 
 DIR is the directory given to `rocprofv3 -d` (searched recursively for *_kernel_trace.csv / *_counter_collection.csv).
@@ -12,7 +12,8 @@ kernels   per kernel: calls, mean / median / min / max duration in microseconds 
 counters  per kernel and counter: mean over its dispatches, from a `--pmc` run (--largest N: over the N dispatches with
           the largest value only, which leaves out smaller launches of the same kernel).  --copy-kib KIB: the run also
           holds plain device copies of that many KiB (bench.py --calibrate-copy: 49152); FETCH_SIZE and WRITE_SIZE are
-          then scaled by what the copy kernel reads for its known size and printed in MB as well.
+          then scaled by what the copy kernel reads for its known size and printed in MB as well.  --by-grid: one entry per
+          (kernel, grid size) instead of per kernel, which separates the shapes one kernel was launched on.
 decode    a `--kernel-trace` run of `python -m llm_reproducibility_amd.e2e_invariance --layers L ...`: kernel time per
           layer and per step over the last S decode steps, grouped by kind of kernel (the step boundaries are found from
           the q/k-norm + rotary kernel, which runs once per layer and step).
@@ -76,7 +77,8 @@ def counters(args) -> int:
     agg = collections.defaultdict(lambda: collections.defaultdict(list))
     for path in _find(args.dir, "_counter_collection.csv"):
         for r in csv.DictReader(open(path)):
-            agg[r["Kernel_Name"]][r["Counter_Name"]].append(float(r["Counter_Value"]))
+            key = r["Kernel_Name"] + (f"  [grid {r['Grid_Size']} x wg {r['Workgroup_Size']}]" if args.by_grid else "")
+            agg[key][r["Counter_Name"]].append(float(r["Counter_Value"]))
     scale = {}
     if args.copy_kib:
         for k, cs in agg.items():
@@ -88,7 +90,7 @@ def counters(args) -> int:
     for k, cs in sorted(agg.items()):
         if args.kernel and args.kernel not in k:
             continue
-        print(_short(k, 110))
+        print(_short(k, 150))
         for c, vals in sorted(cs.items()):
             vals = sorted(vals)[-args.largest:] if args.largest else vals
             m = statistics.mean(vals)
@@ -147,6 +149,7 @@ def main(argv=None) -> int:
     c.add_argument("--kernel", default=None)
     c.add_argument("--largest", type=int, default=0)
     c.add_argument("--copy-kib", type=float, default=0.0)
+    c.add_argument("--by-grid", action="store_true")
     d = sub.add_parser("decode")
     d.add_argument("dir")
     d.add_argument("--layers", type=int, required=True)
