@@ -164,11 +164,14 @@ __global__ __launch_bounds__(64) void attention_kernel(const AttnArgs a) {
 template <int G, bool DEEP>
 __global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs a) {
   __shared__ __attribute__((aligned(16))) uint8_t lds[2][16384];  // per buffer: K tile [32][128] (8 KiB), V^T tile [128][32] (8 KiB)
-  const int b = blockIdx.z;
-  const int kvh = blockIdx.y;
-  // causal attention: the last query blocks have the most keys, so they are dispatched first (longest work first
-  // keeps the tail of the launch short); which work-group computes a block has no numeric effect
-  const int qb = gridDim.x - 1 - blockIdx.x;
+  const int b = blockIdx.y;
+  // Work-groups are dealt to the eight XCDs round robin, each with an L2 of its own: with the KV head as the fastest
+  // index every XCD serves the query blocks of the same few KV heads, and the key tiles those blocks share (every block
+  // of a head walks the same keys) stay in ITS L2 instead of being fetched by all eight.
+  // Causal attention: the last query blocks have the most keys, so they are dispatched first (longest work first
+  // keeps the tail of the launch short); which work-group computes a block has no numeric effect.
+  const int kvh = blockIdx.x % a.kv_heads;
+  const int qb = gridDim.x / a.kv_heads - 1 - blockIdx.x / a.kv_heads;
   const int qlen = a.q_len[b];
   if (qb * 16 >= qlen) return;  // uniform over the work-group
   const int tid = threadIdx.x;
@@ -198,16 +201,35 @@ __global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs 
   // hides none of them.  Prefill has arithmetic to overlap and prefers the registers (more waves per SIMD).
   constexpr int DEPTH = !DEEP ? 1 : (NCH <= 2 ? 4 : (NCH <= 4 ? 2 : 1));
   u32x4 kregs[DEPTH][NCH], vregs[DEPTH][NCH];
+  // A K tile is 8 KiB of consecutive bytes (32 rows of 256), chunk ch at byte 16 ch; a V^T tile is 128 rows of 64 bytes,
+  // max_len elements apart.  Per-thread byte offsets inside a tile (global and LDS side) are formed once; per tile only
+  // a wave-uniform base moves, so the loads take a scalar base and the loop spends no vector instruction on addresses.
+  uint32_t vsrc[NCH], kdst[NCH], vdst0[NCH], vdst1[NCH];
+#pragma unroll
+  for (int i = 0; i < NCH; i++) {
+    const int ch = min(tid + i * NT, 511);
+    const int kr = ch >> 4, kc = ch & 15;   // key row, 16-byte chunk of its 256 bytes
+    kdst[i] = kr * 256 + ((kc ^ (2 * (kr & 7))) << 4);
+    // V^T: channel row vr (64 bytes = 32 keys), 16-byte chunk vc = keys 8vc .. 8vc+7.  The keys of a row are stored
+    // in the order a P*V fragment wants them -- lane group g takes keys 4g..4g+3 and 16+4g..16+4g+3 -- so that a
+    // fragment is ONE 16-byte read at byte 16g of the row: keys 4a..4a+3 live in the 8-byte slot 2 (a & 3) + (a >> 2).
+    // A wave then reads sixteen consecutive rows as one linear KiB (no bank conflicts, no swizzle).
+    const int vr = ch >> 2, vc = ch & 3;
+    vsrc[i] = (uint32_t)vr * (uint32_t)a.max_len * 2u + vc * 16;
+    vdst0[i] = 8192 + vr * 64 + (2 * ((2 * vc) & 3) + (vc >> 1)) * 8;
+    vdst1[i] = 8192 + vr * 64 + (2 * ((2 * vc + 1) & 3) + (vc >> 1)) * 8;
+  }
   auto load_tile = [&](int tile, int set) __attribute__((always_inline)) {
     u32x4* kreg = kregs[set];
     u32x4* vreg = vregs[set];
     const int k0 = min(tile * 32, a.max_len - 32);  // max_len is a multiple of 32: never past the cache
+    const uint8_t* kt = kbase + (int64_t)k0 * (HD * 2);
+    const uint8_t* vt = vbase + (int64_t)k0 * 2;
 #pragma unroll
     for (int i = 0; i < NCH; i++) {
-      const int ch = tid + i * NT;
-      if (512 % NT == 0 || ch < 512) {
-        kreg[i] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)(k0 + (ch >> 4)) * (HD * 2) + (ch & 15) * 16);
-        vreg[i] = *reinterpret_cast<const u32x4*>(vbase + ((int64_t)(ch >> 2) * a.max_len + k0) * 2 + (ch & 3) * 16);
+      if (512 % NT == 0 || tid + i * NT < 512) {
+        kreg[i] = *reinterpret_cast<const u32x4*>(kt + (uint32_t)((tid + i * NT) * 16));
+        vreg[i] = *reinterpret_cast<const u32x4*>(vt + vsrc[i]);
       }
     }
   };
@@ -216,18 +238,10 @@ __global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs 
     const u32x4* vreg = vregs[set];
 #pragma unroll
     for (int i = 0; i < NCH; i++) {
-      const int ch = tid + i * NT;
-      if (512 % NT == 0 || ch < 512) {
-        const int kr = ch >> 4, kc = ch & 15;   // key row, 16-byte chunk of its 256 bytes
-        *reinterpret_cast<u32x4*>(&lds[buf][kr * 256 + ((kc ^ (2 * (kr & 7))) << 4)]) = kreg[i];
-        // V^T: channel row vr (64 bytes = 32 keys), 16-byte chunk vc = keys 8vc .. 8vc+7.  The keys of a row are stored
-        // in the order a P*V fragment wants them -- lane group g takes keys 4g..4g+3 and 16+4g..16+4g+3 -- so that a
-        // fragment is ONE 16-byte read at byte 16g of the row: keys 4a..4a+3 live in the 8-byte slot 2 (a & 3) + (a >> 2).
-        // A wave then reads sixteen consecutive rows as one linear KiB (no bank conflicts, no swizzle).
-        const int vr = ch >> 2, vc = ch & 3;
-        const int slot0 = 2 * ((2 * vc) & 3) + (vc >> 1), slot1 = 2 * ((2 * vc + 1) & 3) + (vc >> 1);
-        *reinterpret_cast<uint2*>(&lds[buf][8192 + vr * 64 + slot0 * 8]) = make_uint2(vreg[i][0], vreg[i][1]);
-        *reinterpret_cast<uint2*>(&lds[buf][8192 + vr * 64 + slot1 * 8]) = make_uint2(vreg[i][2], vreg[i][3]);
+      if (512 % NT == 0 || tid + i * NT < 512) {
+        *reinterpret_cast<u32x4*>(&lds[buf][kdst[i]]) = kreg[i];
+        *reinterpret_cast<uint2*>(&lds[buf][vdst0[i]]) = make_uint2(vreg[i][0], vreg[i][1]);
+        *reinterpret_cast<uint2*>(&lds[buf][vdst1[i]]) = make_uint2(vreg[i][2], vreg[i][3]);
       }
     }
   };
@@ -253,13 +267,16 @@ __global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs 
   for (int d = 0; d < DEPTH; d++) load_tile(d, d);
   store_tile(0, 0);
   __syncthreads();
-  for (int t0 = 0; t0 < ntiles; t0 += DEPTH) {
+  // the loop body covers UNROLL (an even number of) tiles, so that the LDS buffer of each is a compile-time constant and
+  // every LDS address is a per-thread offset plus an immediate
+  constexpr int UNROLL = DEPTH < 2 ? 2 : DEPTH;
+  for (int t0 = 0; t0 < ntiles; t0 += UNROLL) {
 #pragma unroll
-   for (int d = 0; d < DEPTH; d++) {
+   for (int d = 0; d < UNROLL; d++) {
     const int tile = t0 + d;
     if (tile >= ntiles) break;
-    const int cur = tile & 1;
-    load_tile(tile + DEPTH, d);  // set d held this tile and went to LDS a tile ago
+    const int cur = d & 1;
+    load_tile(tile + DEPTH, d % DEPTH);  // that set held this tile and went to LDS a tile ago
     const int k0 = tile * 32;
     const uint8_t* tb = &lds[cur][0];
     f32x4 s[2];
@@ -323,7 +340,8 @@ int attention_dispatch(const void* q, const void* k_cache, const void* vt_cache,
   const int G = q_heads / kv_heads;
   const bool grouped = (max_len & 31) == 0 && (G == 1 || G == 2 || G == 4 || G == 8) && kv_heads <= 65535;
   if (grouped) {
-    const dim3 grid((unsigned)((max_q_len + 15) / 16), (unsigned)kv_heads, (unsigned)batch);
+    if ((int64_t)((max_q_len + 15) / 16) * kv_heads > 0x7fffffff) return TBIK_ERR_INVALID;
+    const dim3 grid((unsigned)((max_q_len + 15) / 16) * (unsigned)kv_heads, (unsigned)batch, 1u);
     const bool deep = max_q_len <= 16;  // decode: one block of queries per sequence
     if (G == 1) hipLaunchKernelGGL((attention_group_kernel<1, false>), grid, dim3(64), 0, stream, a);
     else if (G == 2 && deep) hipLaunchKernelGGL((attention_group_kernel<2, true>), grid, dim3(128), 0, stream, a);
