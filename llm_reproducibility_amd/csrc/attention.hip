@@ -43,31 +43,34 @@ constexpr int HD = 128;
 template <bool MASK>
 __device__ __forceinline__ void softmax_tile(const f32x4 (&s)[2], int k0, int g, int qpos, float scale_log2, float& m, float& l,
                                              float& alpha, bf16x8& p) {
-  // every product and sum below is rounded on its own, except the one fused update of the denominator: left to the
-  // compiler, the scaling of a score could be fused with the subtraction of the maximum in one instantiation and not
-  // in another, and the kernels would no longer agree bit for bit
+  // every product and sum below is rounded on its own, except where a fused multiply-add is written out: left to the
+  // compiler, a multiplication could be fused with the next addition in one instantiation and not in another, and the
+  // kernels would no longer agree bit for bit
 #pragma clang fp contract(off)
   float sv[8];
 #pragma unroll
   for (int u = 0; u < 2; u++)
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-      float v = s[u][i] * scale_log2;
+      float v = s[u][i];
       if (MASK) v = (k0 + 16 * u + 4 * g + i <= qpos) ? v : -INFINITY;
       sv[4 * u + i] = v;
     }
-  float tmax = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
-  tmax = xor_step<16, LaneMax>(tmax);
-  tmax = xor_step<32, LaneMax>(tmax);
-  const float m_new = fmaxf(m, tmax);          // key 0 is visible to every query: m_new is finite from tile 0 on
-  alpha = __builtin_amdgcn_exp2f(m - m_new);   // exactly 1.0 when the tile adds nothing new
-  float psum = 0.f;
+  // the maximum is taken over the raw scores and scaled once (the scale is positive and rounding is monotonic, so this
+  // is the maximum of the scaled scores); 2^(score * scale - maximum) is then one fused multiply-add and one exponential
+  // (NaN-propagating maxima: a NaN score makes the row NaN, as it would through the sum)
+  float tmax = LaneMaxNaN::f(LaneMaxNaN::f(LaneMaxNaN::f(sv[0], sv[1]), LaneMaxNaN::f(sv[2], sv[3])),
+                             LaneMaxNaN::f(LaneMaxNaN::f(sv[4], sv[5]), LaneMaxNaN::f(sv[6], sv[7])));
+  tmax = xor_step<16, LaneMaxNaN>(tmax);
+  tmax = xor_step<32, LaneMaxNaN>(tmax);
+  const float m_new = LaneMaxNaN::f(m, tmax * scale_log2);  // key 0 is visible to every query: m_new is finite from tile 0 on
+  alpha = __builtin_amdgcn_exp2f(m - m_new);        // exactly 1.0 when the tile adds nothing new
   float pv[8];
 #pragma unroll
-  for (int e = 0; e < 8; e++) {
-    pv[e] = __builtin_amdgcn_exp2f(sv[e] - m_new);
-    psum += pv[e];
-  }
+  for (int e = 0; e < 8; e++) pv[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[e], scale_log2, -m_new));
+  float psum = pv[0];
+#pragma unroll
+  for (int e = 1; e < 8; e++) psum += pv[e];
   psum = xor_step<16, LaneSum>(psum);
   psum = xor_step<32, LaneSum>(psum);
   l = __builtin_fmaf(l, alpha, psum);
@@ -213,23 +216,31 @@ __global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs 
     // V^T: channel row vr (64 bytes = 32 keys), 16-byte chunk vc = keys 8vc .. 8vc+7.  The keys of a row are stored
     // in the order a P*V fragment wants them -- lane group g takes keys 4g..4g+3 and 16+4g..16+4g+3 -- so that a
     // fragment is ONE 16-byte read at byte 16g of the row: keys 4a..4a+3 live in the 8-byte slot 2 (a & 3) + (a >> 2).
-    // A wave then reads sixteen consecutive rows as one linear KiB (no bank conflicts, no swizzle).
+    // A 16-byte read is served for lanes {0-7, 16-23} together (then {8-15, 24-31}, ...): rows j and j + 4 of a 64-byte
+    // pitch meet in the same banks, so rows with bit 2 set keep their chunks in the other half of the row (chunk ^ 2,
+    // i.e. 8-byte slot ^ 4) and the sixteen lanes of a phase cover all 64 banks.
     const int vr = ch >> 2, vc = ch & 3;
+    const int vx = 4 * ((vr >> 2) & 1);
     vsrc[i] = (uint32_t)vr * (uint32_t)a.max_len * 2u + vc * 16;
-    vdst0[i] = 8192 + vr * 64 + (2 * ((2 * vc) & 3) + (vc >> 1)) * 8;
-    vdst1[i] = 8192 + vr * 64 + (2 * ((2 * vc + 1) & 3) + (vc >> 1)) * 8;
+    vdst0[i] = 8192 + vr * 64 + ((2 * ((2 * vc) & 3) + (vc >> 1)) ^ vx) * 8;
+    vdst1[i] = 8192 + vr * 64 + ((2 * ((2 * vc + 1) & 3) + (vc >> 1)) ^ vx) * 8;
   }
+  // this (sequence, KV head)'s slice of each cache as a raw buffer (no stride, extent in bytes; the dispatcher keeps
+  // max_len small enough for 32-bit offsets)
+  const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(kbase), 0, a.max_len * (HD * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(vbase), 0, a.max_len * (HD * 2), 0x00020000);
   auto load_tile = [&](int tile, int set) __attribute__((always_inline)) {
     u32x4* kreg = kregs[set];
     u32x4* vreg = vregs[set];
     const int k0 = min(tile * 32, a.max_len - 32);  // max_len is a multiple of 32: never past the cache
-    const uint8_t* kt = kbase + (int64_t)k0 * (HD * 2);
-    const uint8_t* vt = vbase + (int64_t)k0 * 2;
+    // buffer loads: the descriptors (one per cache, in scalar registers) and the tile's byte offset are wave-uniform,
+    // the per-thread offsets are the constants formed above -- no vector instruction per load
+    const int ks = k0 * (HD * 2), vs = k0 * 2;
 #pragma unroll
     for (int i = 0; i < NCH; i++) {
       if (512 % NT == 0 || tid + i * NT < 512) {
-        kreg[i] = *reinterpret_cast<const u32x4*>(kt + (uint32_t)((tid + i * NT) * 16));
-        vreg[i] = *reinterpret_cast<const u32x4*>(vt + vsrc[i]);
+        kreg[i] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, (tid + i * NT) * 16, ks, 0);
+        vreg[i] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, (int)vsrc[i], vs, 0);
       }
     }
   };
@@ -254,11 +265,11 @@ __global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs 
 
   // LDS offsets of this lane's fragments inside a tile buffer, formed once: key row 16u + j of the K tile (256 bytes a
   // row, 16-byte chunk c*4 + g swizzled by the row; u adds 4096), channel row 16t + j of the V^T tile (64 bytes a row,
-  // the lane group's eight keys are the 16 bytes at 16g; t adds 1024)
+  // the lane group's eight keys are the 16-byte chunk g, or g ^ 2 in rows with bit 2 set; t adds 1024)
   uint32_t kofs[4];
 #pragma unroll
   for (int c = 0; c < 4; c++) kofs[c] = j * 256 + (((c * 4 + g) ^ (2 * (j & 7))) << 4);
-  const uint32_t vofs = 8192 + j * 64 + g * 16;
+  const uint32_t vofs = 8192 + j * 64 + (g ^ (2 * ((j >> 2) & 1))) * 16;
 
   const int ntiles = last_pos / 32 + 1;
   // loads past the last tile are clamped to a valid address and never used: issuing them unconditionally keeps the
@@ -336,13 +347,15 @@ int attention_dispatch(const void* q, const void* k_cache, const void* vt_cache,
   if (batch > 65535 || q_heads > 65535) return TBIK_ERR_INVALID;
   AttnArgs a{static_cast<const uint16_t*>(q), static_cast<const uint16_t*>(k_cache), static_cast<const uint16_t*>(vt_cache),
              static_cast<uint16_t*>(out), q_start, q_len, ctx_len, q_heads, kv_heads, max_len, scale * 1.4426950408889634f};
-  // the grouped kernel needs whole 32-key tiles in the caches and at most 8 query heads per KV head
+  // the grouped kernel needs whole 32-key tiles in the caches, at most 8 query heads per KV head and a (sequence, head)
+  // slice of a cache below 2 GiB (32-bit byte offsets)
   const int G = q_heads / kv_heads;
-  const bool grouped = (max_len & 31) == 0 && (G == 1 || G == 2 || G == 4 || G == 8) && kv_heads <= 65535;
+  const bool grouped = (max_len & 31) == 0 && (G == 1 || G == 2 || G == 4 || G == 8) && kv_heads <= 65535 && max_len <= (1 << 22);
   if (grouped) {
-    if ((int64_t)((max_q_len + 15) / 16) * kv_heads > 0x7fffffff) return TBIK_ERR_INVALID;
-    const dim3 grid((unsigned)((max_q_len + 15) / 16) * (unsigned)kv_heads, (unsigned)batch, 1u);
     const bool deep = max_q_len <= 16;  // decode: one block of queries per sequence
+    const int64_t gx = (int64_t)((max_q_len + 15) / 16) * kv_heads;
+    if (gx > 0x7fffffff) return TBIK_ERR_INVALID;
+    const dim3 grid((unsigned)gx, (unsigned)batch, 1u);
     if (G == 1) hipLaunchKernelGGL((attention_group_kernel<1, false>), grid, dim3(64), 0, stream, a);
     else if (G == 2 && deep) hipLaunchKernelGGL((attention_group_kernel<2, true>), grid, dim3(128), 0, stream, a);
     else if (G == 2) hipLaunchKernelGGL((attention_group_kernel<2, false>), grid, dim3(128), 0, stream, a);

@@ -85,6 +85,9 @@ struct Num16<true> {
 // operations are commutative, so the bits do not change.
 struct LaneSum { static __device__ __forceinline__ float f(float a, float b) { return a + b; } };
 struct LaneMax { static __device__ __forceinline__ float f(float a, float b) { return fmaxf(a, b); } };
+// the NaN-propagating maximum (v_maximum3_f32): equal to fmaxf unless an input is NaN, and one instruction where fmaxf
+// first quiets inputs the compiler cannot prove quiet (MFMA results, lane exchanges)
+struct LaneMaxNaN { static __device__ __forceinline__ float f(float a, float b) { return __builtin_elementwise_maximum(a, b); } };
 template <int OFF, typename Op>
 __device__ __forceinline__ float xor_step(float v) {
   const uint32_t u = __builtin_bit_cast(uint32_t, v);
