@@ -288,6 +288,12 @@ def table(steps, warmup, hot=False, settle_ms=20.0, full=False, only=None):
         gemm_row(f"tree matmul down_proj 8B M={M} K=12288 N=4096", M, 12288, 4096, 256, short=None if M == 2048 else f"tree dn8B M={M}")
     for M in (1, 128, 2048):
         library_row(M, 12288, 4096)
+    # the same product with B handed over as a row-major [K,N] matrix (a plain `x @ B`): consumed in place by the tiled
+    # kernels up to 1023 rows, repacked into the native [N,K] layout (inside the timed call) from 1024 rows on
+    for M in (128, 2048):
+        gemm_row(f"tree matmul down_proj 8B M={M}, B row-major [K,N] ({'repacked per call' if M >= 1024 else 'in place'})", M, 12288,
+                 4096, 256, lambda X, W: matmul_tp_persistent(X, W.view(W.shape[1], W.shape[0])),
+                 short=f"tree dn8B rowmajorB M={M}" if M == 2048 else None)
     for p in (2, 4, 8):
         gemm_row(f"tree matmul shard TP={p} M=2048 K={12288 // p} N=4096", 2048, 12288 // p, 4096, 256)
     for M in (1, 64, 512, 4096):

@@ -58,8 +58,10 @@ int tbik_tree_params(int K, int leaf_k, int* T, int* flb, int* level_k);
  *      (src/tbik/tree_based_matmul.py:259-264).  ldb_k == 1 (the nn.Linear weight [N,K], i.e. weight.t()) is the
  *      native layout of every kernel; ldb_n == 1 (row-major [K,N], what simple_matmul.py:11-14 hands over) is
  *      consumed in place by the tiled kernels, which transpose 8x8 blocks in registers on the way to LDS -- same
- *      MFMA chain, same bits, no copy (the large-M pipeline is built for [N,K] only, so big row-major problems run
- *      slower than their [N,K] form).  The contiguous dimension's partner stride must be a multiple of 8 elements;
+ *      MFMA chain, same bits, no copy (the large-M pipelines are built for [N,K] only: measured on MI355X,
+ *      [M,12288] x [12288,4096] row-major takes 60 / 762 us at M = 128 / 2048 against 32 / 200 us for the [N,K]
+ *      form, so a caller with many rows should hand over [N,K]; the Python wrappers repack from 1024
+ *      rows on).  The contiguous dimension's partner stride must be a multiple of 8 elements;
  *      neither stride equal to 1 returns TBIK_ERR_UNSUPPORTED.
  *      For ldb_n == 1 the workspace size is tbik_gemm_workspace_bytes_rowmajor_b(M,N,K,leaf_k,f16).
  *   C: element (m,n) at C[m*ldc + n]
@@ -84,6 +86,20 @@ int tbik_gemm_bf16(const void* A, int64_t lda,
 size_t tbik_gemm_workspace_bytes(int M, int N, int K, int leaf_k);
 /* The same for a row-major B[K,N] (ldb_n == 1); f16 != 0: for tbik_gemm_f16. */
 size_t tbik_gemm_workspace_bytes_rowmajor_b(int M, int N, int K, int leaf_k, int f16);
+/*
+ * How tbik_gemm_bf16 (f16 != 0: tbik_gemm_f16) would run this problem: the decision the workspace size above comes
+ * from, for callers and tests that want to see it (host only, launches nothing, no effect on any result).
+ *   out5[0] path: 0 one launch with K cut over the waves of a work-group (a few rows), 1 128x128 tiles,
+ *                 2 two column regions with a K split each, 3 one grid with one K split
+ *   out5[1] K split (of the first region for path 2, 0 if that region runs on 128x128 tiles; waves per strip for path 0)
+ *   out5[2] columns of the first region (path 2), else 0
+ *   out5[3] K split of the second region (path 2), else 0
+ *   out5[4] 1 when both regions go out as one launch
+ * Every choice yields the same bits (shard tree o leaf tree = full tree).
+ * Replaces: the fixed launch configuration of the reference, src/tbik/tree_based_matmul.py:206-238 (no counterpart
+ * for the K split: the reference cuts K only across GPUs).
+ */
+int tbik_gemm_plan_info(int M, int N, int K, int leaf_k, int f16, int rowmajor_b, int* out5);
 
 /*
  * tbik_gemm_bf16 for callers that cannot allocate device memory: code under HIP graph capture, tight serving loops,

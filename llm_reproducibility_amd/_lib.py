@@ -11,7 +11,7 @@ import os
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG_DIR, "libtbik_hip.so")
 
-ABI_VERSION = 12
+ABI_VERSION = 13
 TBIK_OK = 0
 TBIK_ERR_INVALID = 1
 TBIK_ERR_ALIGNMENT = 2
@@ -25,7 +25,7 @@ EXPORTS = (
     "tbik_tree_combine_bf16", "tbik_tree_combine_f32",
     "bi_gemm_bf16", "bi_rmsnorm_bf16", "bi_log_softmax_workspace_bytes", "bi_log_softmax_f32", "bi_mean_dim", "bi_attention_bf16", "bi_silu_mul_bf16",
     "tbik_gemm_f16", "tbik_gemm_f16_workspace_bytes", "tbik_tree_combine_f16", "bi_gemm_f16", "tbik_gemm_f32", "bi_gemm_f32", "bi_rmsnorm_f16", "bi_silu_mul_f16", "bi_qk_norm_rope_cache_bf16", "bi_argmax_bf16",
-    "tbik_gemm_bf16_static", "bi_log_softmax", "tbik_gemm_workspace_bytes_rowmajor_b",
+    "tbik_gemm_bf16_static", "bi_log_softmax", "tbik_gemm_workspace_bytes_rowmajor_b", "tbik_gemm_plan_info",
     "bi_rmsnorm_gemm_bf16", "tbik_gemm_silu_mul_bf16",
 )
 
@@ -62,6 +62,8 @@ def lib() -> ctypes.CDLL:
     L.tbik_gemm_bf16.restype = i32
     L.tbik_gemm_workspace_bytes_rowmajor_b.argtypes = [i32, i32, i32, i32, i32]
     L.tbik_gemm_workspace_bytes_rowmajor_b.restype = sz
+    L.tbik_gemm_plan_info.argtypes = [i32, i32, i32, i32, i32, i32, ctypes.POINTER(ctypes.c_int)]
+    L.tbik_gemm_plan_info.restype = i32
     L.tbik_tree_combine_bf16.argtypes = [ctypes.POINTER(vp), i32, vp, i64, vp]
     L.tbik_tree_combine_bf16.restype = i32
     L.bi_gemm_bf16.argtypes = [vp, i64, vp, i64, i64, vp, i64, i32, i32, i32, vp, vp]

@@ -7,6 +7,7 @@ int gemm_dispatch(bool tree, bool f16, const void* A, int64_t lda, const void* B
                   int64_t ldc, int M, int N, int K, int leaf_k, const void* bias, void* ws, size_t ws_bytes,
                   hipStream_t stream);
 size_t gemm_workspace_bytes(int M, int N, int K, int leaf_k, bool f16, bool rowmajor_b = false);
+int gemm_plan_info(int M, int N, int K, int leaf_k, bool f16, bool rowmajor_b, int out[5]);
 int tree_combine_dispatch(const void* const* parts, int nparts, void* out, int64_t numel, bool f16, hipStream_t stream);
 int tree_combine_f32_dispatch(const void* const* parts, int nparts, void* out, int64_t numel, hipStream_t stream);
 int rmsnorm_dispatch(const void* x, int64_t ldx, const void* res, int64_t ldr, const void* w, void* out, int64_t ldo,
@@ -36,7 +37,7 @@ int gemm_tree_gated_dispatch(const void* gate, const void* up, int64_t ld, const
 
 extern "C" {
 
-int tbik_abi_version(void) { return 12; }
+int tbik_abi_version(void) { return 13; }
 
 const char* tbik_error_string(int code) {
   switch (code) {
@@ -67,6 +68,9 @@ size_t tbik_gemm_workspace_bytes(int M, int N, int K, int leaf_k) { return tbik:
 size_t tbik_gemm_f16_workspace_bytes(int M, int N, int K, int leaf_k) { return tbik::gemm_workspace_bytes(M, N, K, leaf_k, true); }
 size_t tbik_gemm_workspace_bytes_rowmajor_b(int M, int N, int K, int leaf_k, int f16) {
   return tbik::gemm_workspace_bytes(M, N, K, leaf_k, f16 != 0, true);
+}
+int tbik_gemm_plan_info(int M, int N, int K, int leaf_k, int f16, int rowmajor_b, int* out5) {
+  return tbik::gemm_plan_info(M, N, K, leaf_k, f16 != 0, rowmajor_b != 0, out5);
 }
 
 int tbik_gemm_bf16(const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C, int64_t ldc, int M,

@@ -564,40 +564,101 @@ struct RegionPlan {
   size_t bytes_a, bytes_b, bytes;
 };
 
+// How a tree GEMM runs.  tree_plan() is the ONE place that decides it: the workspace query and the dispatcher both call
+// it, so the bytes the caller is told to bring are the bytes the launch uses.
+enum TreePath {
+  PATH_STRIP = 0,    // a few rows: one launch, K cut over the waves of a work-group, no workspace
+  PATH_NARROW = 1,   // 64 .. 512 rows, short shards: 128x128 tiles (narrow_plan)
+  PATH_REGIONS = 2,  // two column regions, each with a K split of its own (column_regions)
+  PATH_SINGLE = 3,   // one grid of 128x256 tiles or of the small tiles, one K split (make_plan)
+};
+struct TreePlan {
+  TreePath path;
+  int strip_waves;     // PATH_STRIP
+  NarrowPlan narrow;   // PATH_NARROW
+  RegionPlan regions;  // PATH_REGIONS
+  Plan single;         // PATH_SINGLE
+  size_t bytes;        // workspace of the chosen path
+};
+
+static bool tree_plan(int M, int N, int K, int leaf_k, bool f16, bool rowmajor_b, bool whole_problem, TreePlan* tp);
+
 static bool plan_regions(int M, int N, int K, int leaf_k, bool f16, RegionPlan* rp) {
   rp->na = column_regions(M, N, K, leaf_k, f16);
   if (!rp->na) return false;
+  // each region is planned as a problem of its own (never cut again): what it needs is what its launch will use
+  TreePlan ta, tb;
+  if (!tree_plan(M, rp->na, K, leaf_k, f16, false, false, &ta) || !tree_plan(M, N - rp->na, K, leaf_k, f16, false, false, &tb) ||
+      ta.path == PATH_STRIP || tb.path == PATH_STRIP) {
+    rp->na = 0;
+    return false;
+  }
+  // a region that qualifies for the 128x128 tiles takes them (o_proj 32B at M=512: the 1024 columns cut into sixteen
+  // become 32 tiles cut into eight)
+  rp->narrow_a = ta.path == PATH_NARROW;
+  rp->narrow_b = tb.path == PATH_NARROW;
   if (!make_plan(M, rp->na, K, leaf_k, f16, &rp->a) || !make_plan(M, N - rp->na, K, leaf_k, f16, &rp->b)) {
     rp->na = 0;
     return false;
   }
-  rp->bytes_a = (rp->a.partial_bytes + rp->a.parked_bytes + 255) & ~(size_t)255;
-  rp->bytes_b = (rp->b.partial_bytes + rp->b.parked_bytes + 255) & ~(size_t)255;
-  // a region that qualifies for the 128x128 tiles as a problem of its own takes them (o_proj 32B at M=512: the 1024
-  // columns cut into sixteen become 32 tiles cut into eight)
-  NarrowPlan np;
-  rp->narrow_a = narrow_plan(M, rp->na, K, leaf_k, f16, &np);
-  if (rp->narrow_a) rp->bytes_a = np.partial_bytes;
-  rp->narrow_b = narrow_plan(M, N - rp->na, K, leaf_k, f16, &np);
-  if (rp->narrow_b) rp->bytes_b = np.partial_bytes;
+  rp->bytes_a = (ta.bytes + 255) & ~(size_t)255;
+  rp->bytes_b = (tb.bytes + 255) & ~(size_t)255;
   rp->pair = !rp->narrow_a && !rp->narrow_b && rp->a.wide && rp->b.wide &&
              wide_uses_deep_kernel(leaf_k, f16, rp->a.flb, rp->a.lb) == wide_uses_deep_kernel(leaf_k, f16, rp->b.flb, rp->b.lb);
   rp->bytes = rp->pair ? rp->bytes_a + rp->bytes_b : std::max(rp->bytes_a, rp->bytes_b);
   return true;
 }
 
-size_t gemm_workspace_bytes(int M, int N, int K, int leaf_k, bool f16, bool rowmajor_b) {
+// whole_problem: the call may still be cut into column regions (false for a region itself).  Returns false for shapes
+// no tree exists for (K not a whole number of leaves).
+static bool tree_plan(int M, int N, int K, int leaf_k, bool f16, bool rowmajor_b, bool whole_problem, TreePlan* tp) {
+  int T, flb, level_k;
+  if (M <= 0 || N <= 0 || tbik_tree_params(K, leaf_k, &T, &flb, &level_k) != TBIK_OK) return false;
+  tp->bytes = 0;
+  tp->strip_waves = 0;
   if (!rowmajor_b) {
-    NarrowPlan np;
-    if (narrow_plan(M, N, K, leaf_k, f16, &np)) return np.partial_bytes;
-    RegionPlan rp;
-    if (plan_regions(M, N, K, leaf_k, f16, &rp)) return rp.bytes;
+    tp->strip_waves = gemm_tree_strip_waves(M, N, K, level_k - 1);
+    if (tp->strip_waves) {
+      tp->path = PATH_STRIP;
+      return true;
+    }
+    if (narrow_plan(M, N, K, leaf_k, f16, &tp->narrow)) {
+      tp->path = PATH_NARROW;
+      tp->bytes = tp->narrow.partial_bytes;
+      return true;
+    }
+    if (whole_problem && plan_regions(M, N, K, leaf_k, f16, &tp->regions)) {
+      tp->path = PATH_REGIONS;
+      tp->bytes = tp->regions.bytes;
+      return true;
+    }
   }
-  Plan pl;
-  if (!make_plan(M, N, K, leaf_k, f16, &pl, rowmajor_b)) return 0;
-  if (rowmajor_b) return pl.partial_bytes;
-  if (gemm_tree_strip_waves(M, N, K, pl.lb + (pl.split > 1 ? __builtin_ctz((unsigned)pl.split) : 0))) return 0;  // no workspace on that path
-  return pl.partial_bytes + pl.parked_bytes;
+  if (!make_plan(M, N, K, leaf_k, f16, &tp->single, rowmajor_b)) return false;
+  tp->path = PATH_SINGLE;
+  tp->bytes = tp->single.partial_bytes + tp->single.parked_bytes;
+  return true;
+}
+
+size_t gemm_workspace_bytes(int M, int N, int K, int leaf_k, bool f16, bool rowmajor_b) {
+  TreePlan tp;
+  return tree_plan(M, N, K, leaf_k, f16, rowmajor_b, true, &tp) ? tp.bytes : 0;
+}
+
+// What tree_plan() chose for a shape, for callers and tests that want to know (no effect on any result):
+// out[0] path (0 one-launch few-rows kernel, 1 128x128 tiles, 2 two column regions, 3 one grid), out[1] K split (of the
+// first region for path 2; waves per strip for path 0), out[2] columns of the first region (path 2, else 0), out[3] K
+// split of the second region (path 2, else 0), out[4] 1 when the two regions go out as one launch.
+int gemm_plan_info(int M, int N, int K, int leaf_k, bool f16, bool rowmajor_b, int out[5]) {
+  TreePlan tp;
+  if (!out) return TBIK_ERR_INVALID;
+  if (!tree_plan(M, N, K, leaf_k, f16, rowmajor_b, true, &tp)) return TBIK_ERR_INVALID;
+  out[0] = (int)tp.path;
+  out[1] = tp.path == PATH_STRIP ? tp.strip_waves : tp.path == PATH_NARROW ? tp.narrow.split
+           : tp.path == PATH_REGIONS ? (tp.regions.narrow_a ? 0 : tp.regions.a.split) : tp.single.split;
+  out[2] = tp.path == PATH_REGIONS ? tp.regions.na : 0;
+  out[3] = tp.path == PATH_REGIONS ? (tp.regions.narrow_b ? 0 : tp.regions.b.split) : 0;
+  out[4] = tp.path == PATH_REGIONS && tp.regions.pair ? 1 : 0;
+  return TBIK_OK;
 }
 
 static int gemm_dispatch_impl(bool tree, bool f16, const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n,
@@ -673,18 +734,17 @@ static int gemm_dispatch_impl(bool tree, bool f16, const void* A, int64_t lda, c
   }
 
   if (leaf_k != 256 && leaf_k != 128) return TBIK_ERR_UNSUPPORTED;
-  if (!rowmajor_b) {
+  TreePlan tp;
+  if (!tree_plan(M, N, K, leaf_k, f16, rowmajor_b, whole_problem, &tp)) return TBIK_ERR_INVALID;
+  if (tp.path == PATH_STRIP) {
     // a handful of rows: one launch, K cut over the waves of a work-group, nothing goes through the workspace
     int T, flb, level_k;
-    if (tbik_tree_params(K, leaf_k, &T, &flb, &level_k) != TBIK_OK) return TBIK_ERR_INVALID;
-    const int waves = gemm_tree_strip_waves(M, N, K, level_k - 1);
-    if (waves) {
-      StripArgs sa{a.X, a.W, a.C, a.bias, a.ldx, a.ldw, a.ldc, M, N, K, flb, level_k - 1, a.vec_store};
-      return gemm_tree_strip_launch(sa, leaf_k, waves, f16, stream);
-    }
+    tbik_tree_params(K, leaf_k, &T, &flb, &level_k);
+    StripArgs sa{a.X, a.W, a.C, a.bias, a.ldx, a.ldw, a.ldc, M, N, K, flb, level_k - 1, a.vec_store};
+    return gemm_tree_strip_launch(sa, leaf_k, tp.strip_waves, f16, stream);
   }
-  NarrowPlan np;
-  if (!rowmajor_b && narrow_plan(M, N, K, leaf_k, f16, &np)) {
+  if (tp.path == PATH_NARROW) {
+    const NarrowPlan& np = tp.narrow;
     if (np.partial_bytes > 0 && (!ws || ws_bytes < np.partial_bytes || !aligned16(ws))) return TBIK_ERR_WORKSPACE;
     WideArgs w{a.X, a.W, a.C, a.bias, nullptr, a.ldx, a.ldw, a.ldc, M, N, K / np.split, np.T, np.flb, np.lb, a.vec_store,
                (int64_t)(K / np.split), 0};
@@ -701,8 +761,8 @@ static int gemm_dispatch_impl(bool tree, bool f16, const void* A, int64_t lda, c
     for (int i = 0; i < np.split; i++) parts[i] = static_cast<uint8_t*>(ws) + (size_t)i * M * N * sizeof(uint16_t);
     return tree_combine_bias_dispatch(parts, np.split, C, (int64_t)M * N, bias, N, f16, stream, ldc);
   }
-  RegionPlan rp;
-  if (whole_problem && !rowmajor_b && plan_regions(M, N, K, leaf_k, f16, &rp)) {
+  if (tp.path == PATH_REGIONS) {
+    const RegionPlan& rp = tp.regions;
     const size_t esz = sizeof(uint16_t);
     const int na = rp.na;
     const void* Bb = static_cast<const uint8_t*>(B) + (size_t)na * ldb_n * esz;
@@ -753,10 +813,8 @@ static int gemm_dispatch_impl(bool tree, bool f16, const void* A, int64_t lda, c
     }
     return rc;
   }
-  Plan pl;
-  if (!make_plan(M, N, K, leaf_k, f16, &pl, rowmajor_b)) return TBIK_ERR_INVALID;
-  const size_t need = pl.partial_bytes + pl.parked_bytes;
-  if (need > 0 && (!ws || ws_bytes < need || !aligned16(ws))) return TBIK_ERR_WORKSPACE;
+  const Plan& pl = tp.single;
+  if (tp.bytes > 0 && (!ws || ws_bytes < tp.bytes || !aligned16(ws))) return TBIK_ERR_WORKSPACE;
   uint8_t* wsb = static_cast<uint8_t*>(ws);
   a.T = pl.T;
   a.flb = pl.flb;

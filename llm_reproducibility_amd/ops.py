@@ -89,16 +89,30 @@ def _rows16(t: torch.Tensor):
     return c, c.shape[1]
 
 
-def _weight_operand(B: torch.Tensor):
-    """How a [K,N] operand is handed to the kernels without a copy: (tensor whose data_ptr is passed, ldb_k, ldb_n).
+# Rows from which a row-major [K,N] operand is repacked into the native [N,K] layout instead of being consumed in
+# place.  In place it runs on the 64-row tiled kernels only (the pipelines with 128x256 tiles are built for [N,K]), so
+# the time grows with the rows; a repack costs one transposing copy of B (60 us for 4096 x 4096, 180 us for
+# 12288 x 4096 with the library's copy kernel) and then the fast kernels.  Measured on MI355X, bf16, B of 4096 x 4096 /
+# 12288 x 4096 / 4096 x 12288: the tree matmul in place wins up to 512 rows (74 / 199 / 197 us against 93 / 244 / 256)
+# and loses from 1024 on (133 / 382 / 393 against 110 / 305 / 303; at 4096 rows 523 / 1523 / 1567 against 205 / 594 /
+# 622); the single-accumulator mm, which cannot cut K, wins up to 1024 rows and loses from 2048 on (148 / 416 / 437
+# against 120 / 335 / 332).  Same bits either way.
+_REPACK_ROWS_TREE = 1024
+_REPACK_ROWS_MM = 2048
 
-    `weight.t()` of an nn.Linear weight ([N,K], K contiguous) is the native layout (ldb_k = 1); a row-major [K,N]
-    operand (N contiguous: a plain `x @ B`) is consumed in place too (ldb_n = 1).  Anything else -- neither dimension
-    contiguous, rows not 16-byte aligned -- is repacked once into the native layout."""
+
+def _weight_operand(B: torch.Tensor, rows: int = 0, tree: bool = True):
+    """How a [K,N] operand is handed to the kernels: (tensor whose data_ptr is passed, ldb_k, ldb_n).
+
+    `weight.t()` of an nn.Linear weight ([N,K], K contiguous) is the native layout (ldb_k = 1), used without a copy; a
+    row-major [K,N] operand (N contiguous: a plain `x @ B`) is consumed in place too (ldb_n = 1) unless the product has
+    so many rows (`rows`) that a repack into the native layout pays.  Anything else -- neither dimension contiguous,
+    rows not 16-byte aligned -- is repacked as well."""
     K, N = B.shape
     if B.stride(0) == 1 and _aligned16(B) and K % 8 == 0 and (N == 1 or (B.stride(1) >= K and B.stride(1) % 8 == 0)):
         return B, 1, (K if N == 1 else B.stride(1))
-    if B.stride(1) == 1 and _aligned16(B) and B.stride(0) >= N and B.stride(0) % 8 == 0:
+    in_place = rows < (_REPACK_ROWS_TREE if tree else _REPACK_ROWS_MM)
+    if in_place and B.stride(1) == 1 and _aligned16(B) and B.stride(0) >= N and B.stride(0) % 8 == 0:
         return B, B.stride(0), 1
     w, ldw = _rows16(B.t())
     return w, 1, ldw
@@ -114,7 +128,7 @@ def _gemm_tree_impl(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.Tenso
     M, K = A.shape
     N = B.shape[1]
     a, lda = _rows16(A)
-    w, ldb_k, ldb_n = _weight_operand(B)
+    w, ldb_k, ldb_n = _weight_operand(B, M, True)
     b = None if bias is None else bias.contiguous()
     f16 = _is_f16(A, B, bias)
     C = torch.empty((M, N), device=A.device, dtype=A.dtype)
@@ -192,7 +206,7 @@ def _bi_gemm_impl(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.Tensor]
         B = torch.nn.functional.pad(B, (0, 0, 0, pad))
         K += pad
     a, lda = _rows16(A)
-    w, ldb_k, ldb_n = _weight_operand(B)
+    w, ldb_k, ldb_n = _weight_operand(B, M, False)
     b = None if bias is None else bias.contiguous()
     C = torch.empty((M, N), device=A.device, dtype=A.dtype)
     L = _lib.lib()

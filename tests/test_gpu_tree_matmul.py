@@ -309,6 +309,27 @@ def test_row_major_b_simulated_tp_as_the_reference_script_runs_it(dev):
     assert_close_to_oracle(full, O.matmul_tree(A.cpu(), B.cpu()), "row-major B, Gaussian")
 
 
+def test_row_major_b_repacked_from_many_rows_on_gives_the_same_bits(dev):
+    """From 1024 rows on (2048 for the single-accumulator mm) the wrappers repack a row-major [K,N] operand into the
+    native layout, because the in-place path runs on the small tiles only; on either side of the switch the bits are
+    those of the [N,K] form."""
+    from llm_reproducibility_amd import ops
+    from llm_reproducibility_amd.bio import batch_invariant_ops as bio
+    K, N = 2048, 1536
+    B = O.gaussian_bf16((K, N), 0.02, 3).to(dev)                 # row-major [K,N]
+    Wt = B.t().contiguous().t()                                  # the same matrix as an [N,K] weight, transposed view
+    assert B.stride(1) == 1 and Wt.stride(0) == 1
+    for M in (ops._REPACK_ROWS_TREE - 1, ops._REPACK_ROWS_TREE, ops._REPACK_ROWS_MM - 1, ops._REPACK_ROWS_MM):
+        print("case row-major B rows", M, flush=True)
+        A = O.gaussian_bf16((M, K), 1.0, M).to(dev)
+        assert_bitwise(matmul_tp_persistent(A, B), matmul_tp_persistent(A, Wt), f"tree matmul, {M} rows")
+        assert torch.equal(bio.matmul_persistent(A, B), bio.matmul_persistent(A, Wt)), M
+    assert ops._weight_operand(B, ops._REPACK_ROWS_TREE - 1, True)[1] != 1      # in place
+    assert ops._weight_operand(B, ops._REPACK_ROWS_TREE, True)[1:] == (1, K)    # repacked: [N,K], K contiguous
+    assert ops._weight_operand(B, ops._REPACK_ROWS_MM - 1, False)[1] != 1
+    assert ops._weight_operand(B, ops._REPACK_ROWS_MM, False)[1:] == (1, K)
+
+
 @pytest.mark.parametrize("M,N,K", [(256, 4096, 4096), (128, 512, 12288), (16, 256, 12288), (1, 128, 8192)])
 def test_gaussian_inputs_within_one_ulp_of_oracle(dev, M, N, K):
     print("case", M, N, K, flush=True)

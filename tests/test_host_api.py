@@ -41,6 +41,52 @@ def test_tree_params_through_the_c_abi():
         _lib.tree_params(3200, 256)
 
 
+def test_workspace_query_and_plan_come_from_one_decision():
+    """The workspace a caller is told to bring and the way the dispatcher runs the problem are one host-side decision
+    (`tbik_gemm_plan_info` shows it): over a sweep of shapes the two agree on what each path needs -- nothing for the
+    one-launch few-rows kernel, the K-shard partials for the 128x128 tiles, at least the partials of every K split
+    otherwise -- and known shapes take the paths the design describes."""
+    L = _lib.lib()
+    out = (ctypes.c_int * 5)()
+
+    def plan(M, N, K, leaf, f16=0, rowmajor=0):
+        assert L.tbik_gemm_plan_info(M, N, K, leaf, f16, rowmajor, out) == _lib.TBIK_OK
+        return list(out)
+
+    seen = set()
+    for M in (1, 2, 4, 5, 16, 17, 64, 65, 100, 128, 129, 256, 300, 512, 1000, 2048, 4096, 8192):
+        for N in (64, 1000, 1024, 2048, 4096, 5120, 6144, 24576):
+            for K, leaf in ((256, 256), (1024, 256), (4096, 256), (8192, 256), (12288, 256), (1536, 256), (25600, 128), (3200, 128)):
+                path, split, na, split_b, pair = plan(M, N, K, leaf)
+                ws = L.tbik_gemm_workspace_bytes(M, N, K, leaf)
+                seen.add(path)
+                if path == 0:
+                    assert ws == 0 and M <= 16 and split in (2, 4, 8)
+                elif path == 1:
+                    assert 64 <= M <= 512 and leaf == 256 and ws == (0 if split == 1 else (split * M * N * 2 + 255) // 256 * 256)
+                elif path == 2:
+                    assert 0 < na < N and na % 256 == 0 and M >= 64
+                    parts = [(sp, n) for sp, n in ((split, na), (split_b, N - na)) if sp > 1]
+                    need = [sp * M * n * 2 for sp, n in parts]
+                    assert ws >= (sum(need) if pair else max(need, default=0))
+                else:
+                    assert split >= 1 and (split & (split - 1)) == 0 and ws >= (split * M * N * 2 if split > 1 else 0)
+                assert ws % 16 == 0
+                # a row-major B runs on the tiled kernels only: one grid, partial results only
+                rpath, rsplit, _, _, _ = plan(M, N, K, leaf, 0, 1)
+                assert rpath == 3
+                rws = L.tbik_gemm_workspace_bytes_rowmajor_b(M, N, K, leaf, 0)
+                assert rws == (0 if rsplit == 1 else (rsplit * M * N * 2 + 255) // 256 * 256)
+    assert seen == {0, 1, 2, 3}
+    assert plan(1, 4096, 12288, 256)[0] == 0                                # decode: one launch
+    assert plan(128, 4096, 12288, 256)[:2] == [1, 8]                        # down_proj 8B at 128 rows: 128x128 tiles, K in 8
+    assert plan(2048, 4096, 12288, 256) == [3, 1, 0, 0, 0]                  # the benchmark shape: one round of 256 tiles, no cut
+    p = plan(4096, 5120, 8192, 256)                                         # o_proj 32B: two regions in one launch
+    assert p[0] == 2 and p[2] == 1024 and p[4] == 1
+    assert L.tbik_gemm_plan_info(8, 8, 100, 256, 0, 0, out) == _lib.TBIK_ERR_INVALID   # K is not a whole number of leaves
+    assert L.tbik_gemm_plan_info(8, 8, 256, 256, 0, 0, None) == _lib.TBIK_ERR_INVALID
+
+
 def test_host_argument_checks_fire_before_any_launch():
     L = _lib.lib()
     # null pointers / bad sizes are rejected on the host, so these are safe without a GPU
