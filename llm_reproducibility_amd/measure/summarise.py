@@ -81,12 +81,12 @@ def counters(args) -> int:
             agg[key][r["Counter_Name"]].append(float(r["Counter_Value"]))
     scale = {}
     if args.copy_kib:
-        for k, cs in agg.items():
-            if "copyBuffer" in k:
-                for c in ("FETCH_SIZE", "WRITE_SIZE"):
-                    if c in cs:
-                        scale[c] = args.copy_kib / max(cs[c])
-                        print(f"plain copy of {args.copy_kib:g} KiB ({_short(k, 40)}): {c} reads {max(cs[c]):.0f} -> scale factor {scale[c]:.3f}")
+        # the calibration copies are the largest dispatches of the runtime's copy kernel (it also serves small copies)
+        for c in ("FETCH_SIZE", "WRITE_SIZE"):
+            reads = [max(cs[c]) for k, cs in agg.items() if "copyBuffer" in k and c in cs]
+            if reads:
+                scale[c] = args.copy_kib / max(reads)
+                print(f"plain copy of {args.copy_kib:g} KiB (__amd_rocclr_copyBuffer): {c} reads {max(reads):.0f} -> scale factor {scale[c]:.3f}")
     for k, cs in sorted(agg.items()):
         if args.kernel and args.kernel not in k:
             continue
