@@ -407,6 +407,53 @@ def test_qwen3_32b_shapes_match_the_oracle_bit_for_bit_at_full_size(dev, name, M
     assert want.float().abs().max() > 2048          # sums far beyond the 8 significant bits: the roundings matter
 
 
+def _plan_signatures():
+    """One small representative shape per distinct decision of the dispatcher over a sweep: (path, K splits, one or two
+    launches for column regions, leaf, class of row count) -> (M, N, K)."""
+    import ctypes
+    import itertools
+    from llm_reproducibility_amd import _lib
+    L = _lib.lib()
+    out = (ctypes.c_int * 5)()
+    Ms = (1, 2, 4, 8, 16, 17, 48, 64, 96, 128, 160, 256, 384, 512, 768, 1024, 2048, 4096)
+    Ns = (256, 512, 1024, 1536, 2048, 3072, 4096, 5120, 6144, 8192)
+    Ks = ((512, 256), (1024, 256), (1536, 256), (2048, 256), (3072, 256), (4096, 256), (6144, 256), (8192, 256), (12288, 256),
+          (16384, 256), (1280, 128), (3200, 128), (6400, 128), (25600, 128))
+    best = {}
+    for M, N, (K, leaf) in itertools.product(Ms, Ns, Ks):
+        assert L.tbik_gemm_plan_info(M, N, K, leaf, 0, 0, out) == 0
+        sig = (out[0], out[1], out[3], out[4], leaf, (M > 16) + (M > 64) + (M > 128) + (M > 512))
+        if sig not in best or M * N * K < best[sig][0] * best[sig][1] * best[sig][2]:
+            best[sig] = (M, N, K)
+    return best
+
+
+def test_every_decision_of_the_dispatcher_over_a_sweep_gives_the_same_bits(dev):
+    """Which kernel, which K split and which column regions serve a shape comes from measured thresholds; a threshold
+    that sends a shape to a pairing nobody tried must not change a bit.  For one representative of every distinct decision
+    in a sweep of 2520 shapes (all four paths, K cut into 1 .. 32, regions in one and in two launches, both leaf sizes):
+    the product equals the same product computed in column chunks of 128 and row chunks of 16 -- small problems that
+    take other paths -- bit for bit, and, where the CPU oracle is quick, the oracle on integer inputs."""
+    sigs = _plan_signatures()
+    assert {s[0] for s in sigs} == {0, 1, 2, 3} and len(sigs) >= 60
+    for sig, (M, N, K) in sorted(sigs.items()):
+        leaf = sig[4]
+        print("case plan", sig, "shape", M, N, K, flush=True)
+        A = O.gaussian_bf16((M, K), 1.0, M + K).to(dev)
+        Wt = O.gaussian_bf16((N, K), 0.02, N).to(dev).t()
+        got = matmul_tp_persistent(A, Wt, leaf_k=leaf)
+        ref = torch.empty_like(got)
+        for n0 in range(0, N, 128):                      # every element again, as part of a much smaller problem
+            for m0 in range(0, M, 16 if M <= 64 else 1024):
+                m1 = min(M, m0 + (16 if M <= 64 else 1024))
+                ref[m0:m1, n0:n0 + 128] = matmul_tp_persistent(A[m0:m1], Wt[:, n0:n0 + 128], leaf_k=leaf)
+        assert_bitwise(got, ref, f"plan {sig} on {M}x{N}x{K}")
+        if M * N * K <= 2e9:
+            Ai, Wi = O.integer_bf16((M, K), -9, 9, 1), O.integer_bf16((N, K), -7, 7, 2)
+            assert_bitwise(matmul_tp_persistent(Ai.to(dev), Wi.to(dev).t(), leaf_k=leaf), O.matmul_tree(Ai, Wi.t(), leaf=leaf),
+                           f"plan {sig} against the oracle")
+
+
 def test_invariance_qwen3_32b_o_proj(dev):
     _invariance(dev, 8192, 5120, (1, 64, 512), "gauss", 4096)
 
