@@ -256,6 +256,35 @@ def test_single_accumulator_mm_large_and_small_kernels_agree_bitwise(dev):
     assert torch.equal(bio.matmul_persistent(ai.to(dev), wi.to(dev).t()).cpu(), O.matmul_single_acc(ai, wi.t()))
 
 
+def test_single_accumulator_mm_every_shape_of_a_sweep_equals_its_small_pieces(dev):
+    """The mm picks among six kernel families and a dozen tile widths from measured cost models; none of it may change a
+    bit.  Over a seeded sweep of shapes (rows 1 .. 4096, the projection widths of the 8B and 32B configurations and ragged
+    ones, K a multiple of 64, of 32 and of 8 only) the product equals the same product computed in pieces of 16 rows by
+    128 columns, which the streaming kernels serve."""
+    g = torch.Generator().manual_seed(11)
+    Ms = (1, 5, 16, 31, 33, 64, 65, 100, 128, 129, 200, 256, 300, 512, 777, 1024, 1536, 2048, 4096)
+    Ns = (128, 1000, 1024, 3072, 4096, 5120, 6144, 8192, 10240, 24576)
+    Ks = (256, 320, 520, 1024, 2048, 4096, 5120)
+    picks = set()
+    while len(picks) < 48:
+        picks.add((Ms[int(torch.randint(len(Ms), (1,), generator=g))], Ns[int(torch.randint(len(Ns), (1,), generator=g))],
+                   Ks[int(torch.randint(len(Ks), (1,), generator=g))]))
+    for M, N, K in sorted(picks):
+        if M * N * K > 6e10:
+            continue
+        print("case mm sweep", M, N, K, flush=True)
+        A = O.gaussian_bf16((M, K), 1.0, M + N).to(dev)
+        Wt = O.gaussian_bf16((N, K), 0.02, K).to(dev).t()
+        got = bio.matmul_persistent(A, Wt)
+        # pieces: 16 rows (all rows of a small batch at once) by 128 columns
+        rows = range(0, M, 16) if M <= 64 else [int(r) for r in torch.randint(0, M - 15, (4,), generator=g)]
+        for m0 in rows:
+            m1 = min(M, m0 + 16)
+            for n0 in range(0, N, 1024 if N > 2048 else 128):
+                piece = bio.matmul_persistent(A[m0:m1], Wt[:, n0:n0 + 128])
+                assert torch.equal(piece, got[m0:m1, n0:n0 + 128]), (M, N, K, m0, n0)
+
+
 # (M, N, K) -> tile width the cost model picks: 64 / 96 / 192 / 128 / 256 / 32 columns, ragged edges in M and N
 @pytest.mark.parametrize("M,N,K", [(200, 6144, 1024), (500, 6100, 512), (700, 6144, 1024), (384, 8192, 2048), (1100, 8200, 256),
                                    (130, 40, 512), (257, 24576, 320)])
