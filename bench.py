@@ -333,6 +333,28 @@ def table(steps, warmup, hot=False, settle_ms=20.0, full=False, only=None):
     for r in (1, 256, 4096):
         add(f"silu_mul rows={r} inter=12288 (6 B/elem)", lambda r=r: (torch.randn((r, 2 * 12288), device=dev).to(torch.bfloat16),),
             ops.bi_silu_mul, 0.0, r * 12288 * 6, "hbm", short="silu_mul r=4096" if r == 4096 else None)
+    # decode-sized compositions: the producer inside the consuming matmul (one launch) against the two launches it
+    # stands for (same bits); algorithmic bytes = the weights once
+    for M in (1, 4):
+        def make_norm(M=M):
+            return (torch.randn((M, 4096), device=dev).to(torch.bfloat16), torch.randn((M, 4096), device=dev).to(torch.bfloat16),
+                    (torch.randn((24576, 4096), device=dev) * 0.02).to(torch.bfloat16))
+        by = 2.0 * 24576 * 4096
+        add(f"RMSNorm(+residual) inside the mm, gate_up 8B M={M} (one launch)", make_norm,
+            lambda x, r, W: ops.rmsnorm_gemm(x, w, 1e-6, r, W.t()), 2.0 * M * 24576 * 4096, by, "hbm", short=f"norm+mm gate_up M={M}")
+        add(f"  the same as two launches (rms_norm, then mm) M={M}", make_norm,
+            lambda x, r, W: bio.matmul_persistent(bio.rms_norm(x, w, 1e-6, residual=r)[0], W.t()), 2.0 * M * 24576 * 4096, by, "hbm",
+            short=f"norm, mm gate_up M={M}")
+
+        def make_gated(M=M):
+            return (torch.randn((M, 2 * 12288), device=dev).to(torch.bfloat16), (torch.randn((4096, 12288), device=dev) * 0.02).to(torch.bfloat16))
+        by = 2.0 * 4096 * 12288
+        add(f"SiLU*up inside the tree matmul, down_proj 8B M={M} (one launch)", make_gated,
+            lambda gu, W: ops.gemm_tree_silu_mul(gu[:, :12288], gu[:, 12288:], W.t(), None, 256), 2.0 * M * 4096 * 12288, by, "hbm",
+            short=f"silu+tree dn8B M={M}")
+        add(f"  the same as two launches (silu_mul, then tree matmul) M={M}", make_gated,
+            lambda gu, W: matmul_tp_persistent(ops.bi_silu_mul(gu), W.t()), 2.0 * M * 4096 * 12288, by, "hbm",
+            short=f"silu, tree dn8B M={M}")
     # fixed-order attention (Qwen3-8B heads: 32 query, 8 key/value, head_dim 128)
     Hq, Hkv, D = 32, 8, 128
 

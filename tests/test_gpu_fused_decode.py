@@ -69,8 +69,8 @@ def test_rmsnorm_inside_the_mm_declines_what_it_cannot_stage(dev):
     assert _raw_rmsnorm_gemm(x, x.clone(), w, 1e-6, W, C, x) == _lib.TBIK_ERR_INVALID
 
 
-@pytest.mark.parametrize("M,K,N,leaf", [(1, 12288, 4096, 256), (4, 12288, 4096, 256), (2, 1536, 4096, 256), (3, 6144, 4096, 256),
-                                        (1, 4096, 4096, 256), (2, 3072, 2048, 128), (4, 8192, 8192, 256)])
+@pytest.mark.parametrize("M,K,N,leaf", [(1, 12288, 4096, 256), (3, 12288, 4096, 256), (2, 1536, 4096, 256), (3, 6144, 4096, 256),
+                                        (1, 4096, 4096, 256), (2, 3072, 2048, 128), (4, 8192, 4096, 256)])
 def test_silu_mul_inside_the_tree_matmul_equals_the_two_launches(dev, M, K, N, leaf):
     gu = (torch.randn((M, 2 * K), generator=torch.Generator().manual_seed(M + K)) * 2).to(torch.bfloat16).to(dev)
     W = O.gaussian_bf16((N, K), 0.02, 5).to(dev)
@@ -108,13 +108,19 @@ def test_silu_mul_inside_the_tree_matmul_over_simulated_shards(dev):
             layer = SimulatedTPRowLinear(W, tp)
             assert torch.equal(layer.forward_gated(gu), want), (M, tp)
             assert torch.equal(layer(act), want), (M, tp)
-    # shapes the one-launch kernel declines (too many rows; a strip grid that does not balance the chip)
+    # shapes the one-launch kernel declines: too many rows; so many activations that forming them in every work-group
+    # costs more than a launch of its own (4 rows of 12288); more strips than CUs
     s = torch.cuda.current_stream().cuda_stream
     gu = torch.zeros((5, 2 * K), dtype=torch.bfloat16, device=dev)
     C = torch.empty((5, N), dtype=torch.bfloat16, device=dev)
     L = _lib.lib()
-    assert L.tbik_gemm_silu_mul_bf16(gu.data_ptr(), gu.data_ptr() + 2 * K, 2 * K, W.data_ptr(), 1, K, C.data_ptr(), N, 5, N, K,
-                                     256, None, s) == _lib.TBIK_ERR_UNSUPPORTED
+    for rows in (5, 4):
+        assert L.tbik_gemm_silu_mul_bf16(gu.data_ptr(), gu.data_ptr() + 2 * K, 2 * K, W.data_ptr(), 1, K, C.data_ptr(), N, rows, N, K,
+                                         256, None, s) == _lib.TBIK_ERR_UNSUPPORTED
+    Wwide = torch.zeros((8192, 4096), dtype=torch.bfloat16, device=dev)
+    Cw = torch.empty((1, 8192), dtype=torch.bfloat16, device=dev)
+    assert L.tbik_gemm_silu_mul_bf16(gu.data_ptr(), gu.data_ptr() + 4096, 2 * K, Wwide.data_ptr(), 1, 4096, Cw.data_ptr(), 8192, 1,
+                                     8192, 4096, 256, None, s) == _lib.TBIK_ERR_UNSUPPORTED
     W2 = O.gaussian_bf16((5120, 3200), 0.02, 8).to(dev)
     gu2 = (torch.randn((2, 6400), generator=torch.Generator().manual_seed(1))).to(torch.bfloat16).to(dev)
     got = ops.gemm_tree_silu_mul(gu2[:, :3200], gu2[:, 3200:], W2.t(), None, 128)
