@@ -20,7 +20,14 @@ from . import _lib
 _DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(t: torch.Tensor) -> int:
+    """The current stream of the tensor's device as a raw handle.  The private accessor (the one torch's own compiled code
+    uses) returns the handle without building a Stream object: 0.3 us instead of 3 us of host time per launch."""
+    if _raw_stream is not None and t.device.index is not None:
+        return _raw_stream(t.device.index)
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
