@@ -36,7 +36,7 @@ constexpr int HD = 128;
 // One online-softmax update of a query row for a tile of 32 keys, shared by all kernels of this file (one body: the same
 // bits).  Lane (j, g) holds the scores of query j for keys k0 + 16u + 4g + i in s[u][i]; on return p holds the four packed
 // probability pairs of the lane (the B operand of the P*V MFMA) and alpha the factor for the output accumulators of the
-// row (exactly 1.0 when the running maximum did not move).  MASK: apply the causal mask (needed only for tiles that
+// row (exactly 1.0 when the reference point of the exponentials did not move).  MASK: apply the causal mask (needed only for tiles that
 // reach beyond some row's horizon; the values are the same either way for the others).
 // 2^x is the hardware exponential: the arguments are <= 0, and a result below 2^-126 is dropped, which neither the
 // denominator (>= 1: the row's maximum contributes 2^0) nor a bf16 probability can show.
@@ -63,8 +63,16 @@ __device__ __forceinline__ void softmax_tile(const f32x4 (&s)[2], int k0, int g,
                              LaneMaxNaN::f(LaneMaxNaN::f(sv[4], sv[5]), LaneMaxNaN::f(sv[6], sv[7])));
   tmax = xor_step<16, LaneMaxNaN>(tmax);
   tmax = xor_step<32, LaneMaxNaN>(tmax);
-  const float m_new = LaneMaxNaN::f(m, tmax * scale_log2);  // key 0 is visible to every query: m_new is finite from tile 0 on
-  alpha = __builtin_amdgcn_exp2f(m - m_new);        // exactly 1.0 when the tile adds nothing new
+  // The reference point of the exponentials moves lazily: only when a score of this tile exceeds it by more than 2^kLazy
+  // (probabilities then stay below 2^kLazy instead of 1: no loss in fp32 sums or in the relative precision of a bf16
+  // probability, and out = o / l is the same quotient).  After the first tiles of a row it practically never moves, so
+  // the rescale of the output accumulators is skipped for whole rows of tiles.  The rule looks at a row's own scores
+  // in its fixed tile order only, so it is the same for prefill, chunked prefill and decode.
+  // Key 0 is visible to every query: the reference point is finite from tile 0 on.
+  constexpr float kLazy = 8.0f;
+  const float cand = tmax * scale_log2;
+  const float m_new = cand > m + kLazy ? cand : m;
+  alpha = __builtin_amdgcn_exp2f(m - m_new);        // exactly 1.0 when the reference point did not move
   float pv[8];
 #pragma unroll
   for (int e = 0; e < 8; e++) pv[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[e], scale_log2, -m_new));
@@ -108,7 +116,7 @@ __global__ __launch_bounds__(64) void attention_kernel(const AttnArgs a) {
   f32x4 o[8];  // output accumulators, transposed: lane (j, g) holds out[j][16t + 4g .. +3] for the channel tiles t
 #pragma unroll
   for (int t = 0; t < 8; t++) o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float m = -INFINITY;  // running maximum (base-2 domain), identical in the four lanes of a row
+  float m = -INFINITY;  // reference point of the exponentials (base-2 domain; a lazily updated running maximum), identical in the four lanes of a row
   float l = 0.f;        // running denominator
 
   const int ntiles = last_pos / 32 + 1;
@@ -309,7 +317,7 @@ __global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs 
     bf16x8 pf;
     if (!DEEP && __builtin_amdgcn_ballot_w64(k0 + 31 > qpos) == 0) softmax_tile<false>(s, k0, g, qpos, a.scale_log2, m, l, alpha, pf);
     else softmax_tile<true>(s, k0, g, qpos, a.scale_log2, m, l, alpha, pf);
-    // rescale the output accumulators only when some row's maximum moved (uniform over the wave): x * 1.0f is x bit
+    // rescale the output accumulators only when some row's reference point moved (uniform over the wave): x * 1.0f is x bit
     // for bit, and after the first tiles of a long row the maximum rarely moves (prefill only, as above)
     if (DEEP || __builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
 #pragma unroll
