@@ -1,6 +1,6 @@
 """Benchmark of the TBIK hot path on ONE MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--table] [--ceiling]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--table] [--no-ceiling]
 
 A step is one tree-ordered matmul (`matmul_tp_persistent`) over the headline batch: X[2048,12288]
 (SiLU-gated synthetic activations, bf16) times the down_proj weight W[4096,12288] (N(0,0.02), bf16,
@@ -8,7 +8,8 @@ stored [N,K] as nn.Linear does), inputs resident in HBM before the timed region.
 
 Order of a run: the step is timed twice -- right after the host-side set-up (`value_after_idle`: W warm-up steps, K
 timed steps, nothing else) and after `--settle-ms` of the same step run back to back (`value`: the settled rate);
-then the context figures (the vendor library and this library's plain mm on the same operands, and `context.table`:
+then the context figures (the vendor library and this library's plain mm on the same operands, `context.ceiling`: what
+the chip sustains on MFMAs alone and on a one-pass read, with the board power under each of these loops, and `context.table`:
 the other shapes of the workload family, each with its algorithmic flops or bytes and the fraction of the stated
 peak); the CPU baseline and the full-size parity check against it come last, so that they do not sit between the
 set-up and the timed region.  `--table` prints the long form of the table to stderr as well.
@@ -400,8 +401,10 @@ def main():
     ap.add_argument("--settle-ms", type=float, default=60.0,
                     help="continuous load (the step itself) in front of the warm-up steps of `value`, so that the timed "
                          "steps see the chip's settled state; `value_after_idle` is always measured without it")
-    ap.add_argument("--ceiling", action="store_true",
-                    help="also measure the MFMA-only and the one-pass-read ceilings of this chip (reported in `context`)")
+    ap.add_argument("--ceiling", action="store_true", help="kept for older command lines: the ceilings are measured by default")
+    ap.add_argument("--no-ceiling", action="store_true",
+                    help="skip `context.ceiling`: the MFMA-only and one-pass-read ceilings of this chip and the board power "
+                         "while the headline step, this library's plain mm, the vendor GEMM and the probes run (10 s)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run 5 plain device copies of X (50,331,648 B read + as many written each) so that a "
                          "counter run can scale FETCH_SIZE / WRITE_SIZE by what a copy of known size reads")
@@ -466,10 +469,14 @@ def main():
     from llm_reproducibility_amd.bio import batch_invariant_ops as bio
     mm_ms, _ = hip_time_ms(lambda: bio.matmul_persistent(X, Wt), args.steps, args.warmup, args.settle_ms)
     context["single_accumulator_mm_same_operands_TFLOPs"] = round(flops / (mm_ms * 1e-3) / 1e12, 2)
-    if args.ceiling:
-        context["ceiling"] = ceiling(args.settle_ms, (("tree_matmul_headline", step),
-                                                      ("single_accumulator_mm_same_operands", lambda: bio.matmul_persistent(X, Wt)),
-                                                      ("vendor_gemm_same_operands", lambda: torch.matmul(X, Wt))))
+    if not args.no_ceiling and (args.ceiling or not args.only):
+        from llm_reproducibility_amd.build import MEASURE_LIB_PATH
+        if not os.path.exists(MEASURE_LIB_PATH):
+            context["ceiling"] = {"skipped": "the measurement library is not built (python -m llm_reproducibility_amd.build)"}
+        else:
+            context["ceiling"] = ceiling(args.settle_ms, (("tree_matmul_headline", step),
+                                                          ("single_accumulator_mm_same_operands", lambda: bio.matmul_persistent(X, Wt)),
+                                                          ("vendor_gemm_same_operands", lambda: torch.matmul(X, Wt))))
     if args.table or not args.no_context_table:
         t0 = time.perf_counter()
         rows = table(12, 3, hot=args.table_hot, settle_ms=min(args.settle_ms, 10.0), full=args.table, only=args.only)

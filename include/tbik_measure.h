@@ -1,6 +1,6 @@
 /*
  * libtbik_measure.so -- machine probes of the benchmark.  NOT part of the drop-in boundary (include/tbik_hip.h is):
- * nothing here has a counterpart in the reference and no product code calls it; bench.py --ceiling loads the library
+ * nothing here has a counterpart in the reference and no product code calls it; bench.py loads the library for its ceiling figures
  * to read a roofline fraction against a ceiling measured on the box as well as against the published peak.
  * Return values are those of tbik_hip.h (0 = ok).
  *
