@@ -86,6 +86,14 @@ def test_attention_matches_fp32_reference_and_is_batch_and_phase_invariant(dev):
         oa = ops.bi_attention_bf16(torch.cat(q1), ca, va, i32(st), i32(lens[:3]), i32(lens[:3]), max(lens[:3]), scale)
         ob = ops.bi_attention_bf16(torch.cat(q1), cb, vb, i32(st), i32(lens[:3]), i32(lens[:3]), max(lens[:3]), scale)
         assert torch.equal(oa, ob), (hq, hkv)
+        # and against the oracle (a wrong query-head -> KV-head map would be the same mistake in both kernels), prefill
+        # and the decode kernel of this group size
+        dq = torch.stack([q[-1] for q in q1])
+        od = ops.bi_attention_bf16(dq, ca, va, i32([0, 1, 2]), i32([1, 1, 1]), i32(lens[:3]), 1, scale)
+        for b, n in enumerate(lens[:3]):
+            want = O.causal_attention(q1[b].cpu(), k1[b].cpu(), v1[b].cpu(), scale).to(torch.bfloat16)
+            assert not O.outside_tolerance(oa[st[b]: st[b] + n].cpu(), want).any(), (hq, hkv, b)
+            assert torch.equal(od[b], oa[st[b] + n - 1]), (hq, hkv, b)
 
 
 def _oracle_heads(q, k, v, heads, rep, scale):
