@@ -214,8 +214,8 @@ int bi_mean_dim(const void* x, void* out,
 
 /*
  * Causal grouped-query attention with a fixed key order (tiles of 32 keys, ascending, online softmax, one
- * pass, no split over keys), bf16, head_dim 128; the same kernel serves prefill and decode, and a
- * token's output does not depend on the batch it is computed in.
+ * pass, no split over keys), bf16, head_dim 128; prefill, chunked prefill and decode run the same arithmetic
+ * per row (whichever kernel takes the call), and a token's output does not depend on the batch it is computed in.
  *   q, out      [tokens, q_heads, 128]
  *   k_cache     [batch, kv_heads, max_len, 128]
  *   vt_cache    [batch, kv_heads, 128, max_len]   (V stored transposed; entries behind ctx_len must be finite)

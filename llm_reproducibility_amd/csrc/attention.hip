@@ -1,5 +1,11 @@
-// Fixed-order causal attention for gfx950 (bf16, head_dim 128, grouped-query heads), one wavefront per
-// (16 consecutive queries of one sequence, one query head).
+// Fixed-order causal attention for gfx950 (bf16, head_dim 128, grouped-query heads).  A query row is always the four
+// lanes {j, j+16, j+32, j+48} of one wavefront; three kernels differ in what else the wavefront and its work-group hold:
+//   attention_kernel        one wavefront per (16 consecutive queries of a sequence, query head), operands from global
+//                           memory (any cache length);
+//   attention_group_kernel  the G query heads of a KV head as the G wavefronts of a work-group, K/V tiles staged in LDS
+//                           once for all of them (prefill and chunked prefill);
+//   attention_decode_kernel the few new queries of a sequence times the G heads as the 16 rows of ONE tile, the output
+//                           channels split over four wavefronts (decode).
 //
 // Counterpart of the reference's fixed-tile attention for train/inference alignment
 // (_kernel_unified_attention_2d, src/patch/patch_training_inference_align.py:171-487: one pass over the
@@ -343,6 +349,174 @@ __global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs 
   }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Decode variant: every sequence brings so few new queries that all of them, for all G query heads of a KV head, fit
+// the 16 rows of one MFMA tile (row = query * G + head of the group).  One work-group per (KV head, sequence).  Its four
+// wavefronts all compute the scores and the softmax of the whole tile (the same instructions on the same values, so
+// the same bits in each) and each keeps the output accumulators of two of the eight 16-channel tiles: per key tile a
+// wave issues 8 + 2 MFMAs where a wave of the grouped kernel issues 16.  The scores of tile t + 1 are formed before the
+// softmax of tile t, so the MFMA chain of one tile runs beside the exponentials of the other.  A decode step is one
+// dependent chain of key tiles per sequence, and its length per tile is what the kernel's time consists of.
+// A row's arithmetic -- the lanes that own it, the MFMA chains over channels and key slots, the order of the softmax
+// updates -- is that of the kernels above: the same bits.
+// K tiles and V^T tiles have rings of their own (two slots each), because the K tile is needed one iteration earlier.
+// ------------------------------------------------------------------------------------------------
+template <int G>
+__global__ __launch_bounds__(256) void attention_decode_kernel(const AttnArgs a) {
+  __shared__ __attribute__((aligned(16))) uint8_t lds_k[2][8192];  // K tile [32][128], rows XOR-swizzled as above
+  __shared__ __attribute__((aligned(16))) uint8_t lds_v[2][8192];  // V^T tile [128][32] in fragment order as above
+  constexpr int QMAX = 16 / G;  // queries of a sequence that fit the tile
+  const int b = blockIdx.y;
+  const int kvh = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wv = tid >> 6;
+  const int j = lane & 15;
+  const int g = lane >> 4;
+  const uint8_t* kbase = reinterpret_cast<const uint8_t*>(a.k_cache + ((int64_t)b * a.kv_heads + kvh) * a.max_len * HD);
+  const uint8_t* vbase = reinterpret_cast<const uint8_t*>(a.vt_cache + ((int64_t)b * a.kv_heads + kvh) * (int64_t)HD * a.max_len);
+
+  // staging as in the grouped kernel: 512 16-byte chunks per tile and operand, two per thread, fetched four tiles ahead
+  // into four register sets (set = tile % 4)
+  constexpr int NT = 256, NCH = 2, DEPTH = 4;
+  constexpr int CT = 2;  // 16-channel tiles of the output per wave
+  u32x4 kregs[DEPTH][NCH], vregs[DEPTH][NCH];
+  uint32_t vsrc[NCH], kdst[NCH], vdst0[NCH], vdst1[NCH];
+#pragma unroll
+  for (int i = 0; i < NCH; i++) {
+    const int ch = tid + i * NT;
+    const int kr = ch >> 4, kc = ch & 15;
+    kdst[i] = kr * 256 + ((kc ^ (2 * (kr & 7))) << 4);
+    const int vr = ch >> 2, vc = ch & 3;
+    const int vx = 4 * ((vr >> 2) & 1);
+    vsrc[i] = (uint32_t)vr * (uint32_t)a.max_len * 2u + vc * 16;
+    vdst0[i] = vr * 64 + ((2 * ((2 * vc) & 3) + (vc >> 1)) ^ vx) * 8;
+    vdst1[i] = vr * 64 + ((2 * ((2 * vc + 1) & 3) + (vc >> 1)) ^ vx) * 8;
+  }
+  const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(kbase), 0, a.max_len * (HD * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(vbase), 0, a.max_len * (HD * 2), 0x00020000);
+  auto load_tile = [&](int tile, int set) __attribute__((always_inline)) {
+    const int k0 = min(tile * 32, a.max_len - 32);  // max_len is a multiple of 32: never past the cache
+    const int ks = k0 * (HD * 2), vs = k0 * 2;
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+      kregs[set][i] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, (tid + i * NT) * 16, ks, 0);
+      vregs[set][i] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, (int)vsrc[i], vs, 0);
+    }
+  };
+  auto store_k = [&](int slot, int set) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < NCH; i++) *reinterpret_cast<u32x4*>(&lds_k[slot][kdst[i]]) = kregs[set][i];
+  };
+  auto store_v = [&](int slot, int set) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+      *reinterpret_cast<uint2*>(&lds_v[slot][vdst0[i]]) = make_uint2(vregs[set][i][0], vregs[set][i][1]);
+      *reinterpret_cast<uint2*>(&lds_v[slot][vdst1[i]]) = make_uint2(vregs[set][i][2], vregs[set][i][3]);
+    }
+  };
+
+  bf16x8 qf[4];  // Q as the MFMA "B" operand: lane (j, g) holds channels 32c + 8g .. +7 of row j
+  uint32_t kofs[4];
+#pragma unroll
+  for (int c = 0; c < 4; c++) kofs[c] = j * 256 + (((c * 4 + g) ^ (2 * (j & 7))) << 4);
+  const uint32_t vofs = (CT * wv) * 1024 + j * 64 + (g ^ (2 * ((j >> 2) & 1))) * 16;
+  auto scores = [&](int slot, f32x4 (&s)[2]) __attribute__((always_inline)) {
+    const uint8_t* tb = &lds_k[slot][0];
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+      const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+      f32x4 acc;
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(tb + kofs[c] + u * 4096);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[c], c == 0 ? zero : acc, 0, 0, 0);
+      }
+      s[u] = acc;
+    }
+  };
+
+  f32x4 o[CT];  // channel tiles CT wv .. CT wv + CT - 1
+#pragma unroll
+  for (int i = 0; i < CT; i++) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY;
+  float l = 0.f;
+
+  // The first key tiles are requested before anything is known about the sequence: their addresses depend on the
+  // work-group only, and loads past the last tile are clamped to a valid address and never used (a static number of
+  // loads in flight).  The lengths and the queries arrive while those loads are on their way.
+#pragma unroll
+  for (int d = 0; d < DEPTH; d++) load_tile(d, d);
+  const int qlen = a.q_len[b];
+  if (qlen <= 0) return;  // uniform over the work-group
+  const int qi = j / G;                 // query of the sequence
+  const int h = kvh * G + j % G;        // query head
+  const int ctx = a.ctx_len[b];
+  const bool qvalid = qi < qlen;
+  const int qrow = min(qi, qlen - 1);
+  const int qpos = ctx - qlen + qrow;
+  const int last_pos = ctx - qlen + min(QMAX - 1, qlen - 1);
+  const int ntiles = last_pos / 32 + 1;
+  const int nfull = (ctx - qlen + 1) / 32;  // tiles whose keys are visible to every query: no mask needed
+  const uint16_t* qp = a.q + ((int64_t)(a.q_start[b] + qrow) * a.q_heads + h) * HD;
+#pragma unroll
+  for (int c = 0; c < 4; c++) qf[c] = *reinterpret_cast<const bf16x8*>(qp + c * 32 + g * 8);
+  store_k(0, 0);
+  __syncthreads();
+  f32x4 s_cur[2];
+  scores(0, s_cur);
+  store_k(1, 1);
+  store_v(0, 0);
+  __syncthreads();  // also: every wave has read K tile 0 before slot 0 is written again
+  // Iteration t: K tile t + 1 is in K slot (t + 1) & 1 and V^T tile t in V slot t & 1; it writes K tile t + 2 into K slot
+  // t & 1 (read during iteration t - 1) and V^T tile t + 1 into V slot (t + 1) & 1 (likewise), then meets the barrier.
+  // Register set t % 4 is free at the top of iteration t: its K tile went to LDS two iterations ago, its V^T tile one.
+  // The body covers four tiles, so that slots and sets are compile-time constants.
+  for (int t0 = 0; t0 < ntiles; t0 += DEPTH) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++) {
+      const int tile = t0 + d;
+      if (tile >= ntiles) break;
+      load_tile(tile + DEPTH, d);
+      // the V^T fragments are requested first: they have been in LDS since the barrier, and their latency passes
+      // during the scores and the softmax
+      bf16x8 vf[CT];
+#pragma unroll
+      for (int i = 0; i < CT; i++) vf[i] = *reinterpret_cast<const bf16x8*>(&lds_v[d & 1][vofs + i * 1024]);
+      // behind the last tile the slot holds an older tile: the scores are formed (no branch inside the chain) and unused
+      f32x4 s_next[2];
+      scores((d + 1) & 1, s_next);
+      float alpha;
+      bf16x8 pf;
+      // the mask is needed only where a tile reaches beyond some query's horizon (a scalar condition known long before;
+      // the values are the same either way)
+      if (tile < nfull) softmax_tile<false>(s_cur, tile * 32, g, qpos, a.scale_log2, m, l, alpha, pf);
+      else softmax_tile<true>(s_cur, tile * 32, g, qpos, a.scale_log2, m, l, alpha, pf);
+      // (always rescaled: a branch on the freshly computed factor costs more than the few multiplications)
+      {
+#pragma unroll
+        for (int i = 0; i < CT; i++) o[i] = f32x4{o[i][0] * alpha, o[i][1] * alpha, o[i][2] * alpha, o[i][3] * alpha};
+      }
+#pragma unroll
+      for (int i = 0; i < CT; i++) o[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[i], pf, o[i], 0, 0, 0);
+      if (tile + 2 < ntiles) store_k(d & 1, (d + 2) % DEPTH);
+      if (tile + 1 < ntiles) store_v((d + 1) & 1, (d + 1) % DEPTH);
+      __syncthreads();
+      s_cur[0] = s_next[0];
+      s_cur[1] = s_next[1];
+    }
+  }
+  if (!qvalid) return;
+  const float inv = 1.0f / l;
+  uint16_t* op = a.out + ((int64_t)(a.q_start[b] + qi) * a.q_heads + h) * HD + 16 * CT * wv;
+#pragma unroll
+  for (int i = 0; i < CT; i++) {
+    const uint32_t lo = pack_bf16x2(o[i][0] * inv, o[i][1] * inv);
+    const uint32_t hi = pack_bf16x2(o[i][2] * inv, o[i][3] * inv);
+    *reinterpret_cast<uint2*>(op + 16 * i + 4 * g) = make_uint2(lo, hi);
+  }
+}
+
 int attention_dispatch(const void* q, const void* k_cache, const void* vt_cache, void* out, const int* q_start,
                        const int* q_len, const int* ctx_len, int batch, int max_q_len, int q_heads, int kv_heads,
                        int head_dim, int max_len, float scale, hipStream_t stream) {
@@ -361,6 +535,14 @@ int attention_dispatch(const void* q, const void* k_cache, const void* vt_cache,
   const bool grouped = (max_len & 31) == 0 && (G == 1 || G == 2 || G == 4 || G == 8) && kv_heads <= 65535 && max_len <= (1 << 22);
   if (grouped) {
     const bool deep = max_q_len <= 16;  // decode: one block of queries per sequence
+    if ((int64_t)max_q_len * G <= 16) {  // all queries of a sequence and all heads of a group in one MFMA tile
+      const dim3 grid((unsigned)kv_heads, (unsigned)batch, 1u);
+      if (G == 1) hipLaunchKernelGGL(attention_decode_kernel<1>, grid, dim3(256), 0, stream, a);
+      else if (G == 2) hipLaunchKernelGGL(attention_decode_kernel<2>, grid, dim3(256), 0, stream, a);
+      else if (G == 4) hipLaunchKernelGGL(attention_decode_kernel<4>, grid, dim3(256), 0, stream, a);
+      else hipLaunchKernelGGL(attention_decode_kernel<8>, grid, dim3(256), 0, stream, a);
+      return hip_code(hipGetLastError());
+    }
     const int64_t gx = (int64_t)((max_q_len + 15) / 16) * kv_heads;
     if (gx > 0x7fffffff) return TBIK_ERR_INVALID;
     const dim3 grid((unsigned)gx, (unsigned)batch, 1u);

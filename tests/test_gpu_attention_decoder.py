@@ -96,6 +96,61 @@ def test_attention_matches_fp32_reference_and_is_batch_and_phase_invariant(dev):
             assert torch.equal(od[b], oa[st[b] + n - 1]), (hq, hkv, b)
 
 
+@pytest.mark.parametrize("hq,hkv,qlens,ctxs", [
+    (8, 2, [4, 1, 3, 2, 4], [70, 33, 128, 17, 4]),        # four heads per KV head: up to four new queries fit one tile
+    (16, 2, [2, 1, 2], [65, 1, 96]),                      # eight heads per KV head: two
+    (4, 2, [8, 5, 1], [40, 64, 97]),                      # two heads per KV head: eight
+    (2, 2, [16, 9, 1], [16, 100, 31]),                    # one head per KV head: sixteen
+    (32, 8, [3, 4, 1], [2272, 2304, 2239]),               # the decoder's heads; 71, 72 and 70 key tiles
+])
+def test_a_few_new_queries_per_sequence_equal_their_prefill_rows(dev, hq, hkv, qlens, ctxs):
+    """When the new queries of every sequence times the query heads of a KV head fit the 16 rows of one MFMA tile, a
+    kernel of its own takes the call (rows = query x head of the group, the score tiles formed one tile ahead, the
+    output channels split over the waves).  Its rows must be, bit for bit, the rows of the whole prefill of the same
+    sequences (the grouped kernel), ragged batches included, whatever the other sequences of the batch bring; and the
+    one-wave-per-head kernel (a cache length that is not a whole number of tiles) must agree as well."""
+    torch.manual_seed(hq * 100 + len(qlens))
+    D, scale = 128, 1.0 / math.sqrt(128)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)  # noqa: E731
+    ks = [torch.randn((n, hkv, D), device=dev).to(torch.bfloat16) for n in ctxs]
+    vs = [torch.randn((n, hkv, D), device=dev).to(torch.bfloat16) for n in ctxs]
+    qs = [torch.randn((n, hq, D), device=dev).to(torch.bfloat16) for n in ctxs]
+    max_len = (max(ctxs) + 31) // 32 * 32
+    kc, vt = _make_cache(ks, vs, max_len, dev)
+    starts = [sum(ctxs[:i]) for i in range(len(ctxs))]
+    print("case few new queries", hq, hkv, qlens, ctxs, flush=True)
+    full = ops.bi_attention_bf16(torch.cat(qs), kc, vt, i32(starts), i32(ctxs), i32(ctxs), max(ctxs), scale)
+    tails = torch.cat([q[-n:] for q, n in zip(qs, qlens)])
+    tstarts = [sum(qlens[:i]) for i in range(len(qlens))]
+    got = ops.bi_attention_bf16(tails, kc, vt, i32(tstarts), i32(qlens), i32(ctxs), max(qlens), scale)
+    for b, (n, c) in enumerate(zip(qlens, ctxs)):
+        assert torch.equal(got[tstarts[b]: tstarts[b] + n], full[starts[b] + c - n: starts[b] + c]), (b, n, c)
+    # a sequence on its own, and with a single new query where the batch had several
+    for b in (0, len(qlens) - 1):
+        kc1, vt1 = _make_cache([ks[b]], [vs[b]], max_len, dev)
+        alone = ops.bi_attention_bf16(qs[b][-qlens[b]:], kc1, vt1, i32([0]), i32([qlens[b]]), i32([ctxs[b]]), qlens[b], scale)
+        assert torch.equal(alone, got[tstarts[b]: tstarts[b] + qlens[b]]), b
+        one = ops.bi_attention_bf16(qs[b][-1:], kc1, vt1, i32([0]), i32([1]), i32([ctxs[b]]), 1, scale)
+        assert torch.equal(one[0], full[starts[b] + ctxs[b] - 1]), b
+    # a sequence without new tokens in the batch leaves the others as they are and writes nothing
+    q0 = list(qlens)
+    q0[1] = 0
+    t0 = [sum(q0[:i]) for i in range(len(q0))]
+    tails0 = torch.cat([q[-n:] for q, n in zip(qs, q0) if n])
+    out0 = ops.bi_attention_bf16(tails0, kc, vt, i32(t0), i32(q0), i32(ctxs), max(q0), scale)
+    for b, n in enumerate(q0):
+        assert torch.equal(out0[t0[b]: t0[b] + n], full[starts[b] + ctxs[b] - n: starts[b] + ctxs[b]]), b
+    kc2, vt2 = _make_cache(ks, vs, max_len + 4, dev)
+    assert torch.equal(ops.bi_attention_bf16(tails, kc2, vt2, i32(tstarts), i32(qlens), i32(ctxs), max(qlens), scale), got)
+    # and a row of each sequence against the float64 oracle (a wrong row -> (query, head) map would be the same mistake
+    # in nothing else: the prefill rows come from another kernel)
+    for b in range(len(qlens)):
+        if ctxs[b] > 300:
+            continue
+        want = O.causal_attention(qs[b].cpu(), ks[b].cpu(), vs[b].cpu(), scale).to(torch.bfloat16)
+        assert not O.outside_tolerance(got[tstarts[b]: tstarts[b] + qlens[b]].cpu(), want[-qlens[b]:]).any(), b
+
+
 def _oracle_heads(q, k, v, heads, rep, scale):
     """O.causal_attention for a subset of query heads (each with its own KV head), as [n, len(heads), D]."""
     outs = []
