@@ -342,6 +342,19 @@ int bi_qk_norm_rope_cache_bf16(const void* qkv, int64_t ld,
 int bi_argmax_bf16(const void* x, int64_t ld, void* out, int64_t rows, int cols, tbik_stream_t stream);
 
 /*
+ * bi_argmax_bf16 plus the bookkeeping of a decode step, in the same launch (a step of a small batch is a chain of
+ * short kernels, and each of the four updates below would be one more).  Row r's index goes to next_token[r] (int64)
+ * and, where given, to history[r * history_ld + count[r]] (int64; skipped once count[r] reaches history_ld); then
+ * count[r] (int64), positions[r] (int64) and ctx_len[r] (int32) advance by one.  history, count, positions and ctx_len
+ * may each be NULL (history needs count); all are device arrays of `rows` entries (history: rows x history_ld).
+ * Replaces: the sampler output and the per-sequence state update of the engine that the reference drives
+ *           (vllm_generate, simple_inference.py:62-105); same token choice as bi_argmax_bf16.
+ */
+int bi_argmax_advance_bf16(const void* x, int64_t ld, void* next_token, int64_t rows, int cols,
+                           void* history, int64_t history_ld, void* count, void* positions, void* ctx_len,
+                           tbik_stream_t stream);
+
+/*
  * One-launch compositions for decode-sized batches (a handful of rows): the producer of a matmul's activations runs
  * inside the matmul while it stages them, which saves a launch and a round trip of the activations through memory.
  * Both evaluate exactly the expressions of the two-launch forms (the same device functions, the same MFMA chains and

@@ -18,7 +18,8 @@ int log_softmax_dispatch(const void* x, int64_t ldx, int in_dtype, void* out, in
 int attention_dispatch(const void* q, const void* k_cache, const void* vt_cache, void* out, const int* q_start,
                        const int* q_len, const int* ctx_len, int batch, int max_q_len, int q_heads, int kv_heads,
                        int head_dim, int max_len, float scale, hipStream_t stream);
-int argmax_dispatch(const void* x, int64_t ld, void* out, int64_t rows, int cols, hipStream_t stream);
+int argmax_dispatch(const void* x, int64_t ld, void* out, int64_t rows, int cols, void* history, int64_t history_ld,
+                    void* count, void* positions, void* ctx_len, hipStream_t stream);
 int mean_dispatch(const void* x, void* out, int64_t outer, int64_t n, int64_t inner, int dtype_code, hipStream_t stream);
 int gemm_f32_dispatch(bool tree, const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C,
                       int64_t ldc, int M, int N, int K, int leaf_k, const void* bias, hipStream_t stream);
@@ -37,7 +38,7 @@ int gemm_tree_gated_dispatch(const void* gate, const void* up, int64_t ld, const
 
 extern "C" {
 
-int tbik_abi_version(void) { return 13; }
+int tbik_abi_version(void) { return 14; }
 
 const char* tbik_error_string(int code) {
   switch (code) {
@@ -195,7 +196,13 @@ int bi_qk_norm_rope_cache_bf16(const void* qkv, int64_t ld, const void* q_weight
 }
 
 int bi_argmax_bf16(const void* x, int64_t ld, void* out, int64_t rows, int cols, tbik_stream_t stream) {
-  return tbik::argmax_dispatch(x, ld, out, rows, cols, static_cast<hipStream_t>(stream));
+  return tbik::argmax_dispatch(x, ld, out, rows, cols, nullptr, 0, nullptr, nullptr, nullptr, static_cast<hipStream_t>(stream));
+}
+
+int bi_argmax_advance_bf16(const void* x, int64_t ld, void* next_token, int64_t rows, int cols, void* history,
+                           int64_t history_ld, void* count, void* positions, void* ctx_len, tbik_stream_t stream) {
+  return tbik::argmax_dispatch(x, ld, next_token, rows, cols, history, history_ld, count, positions, ctx_len,
+                               static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

@@ -586,7 +586,18 @@ __device__ __forceinline__ void argmax_take(float& bv, int& bi, float v, int i) 
   }
 }
 
-__global__ __launch_bounds__(1024) void argmax_rows_kernel(const uint16_t* x, int64_t ld, int64_t* out, int cols) {
+// Optional bookkeeping of a decode step, done by the work-group of a row once its index is known (all pointers may be
+// null): the index also goes to history[row * history_ld + count[row]] (skipped when the row's history is full) and
+// count[row], positions[row] and ctx_len[row] advance by one.
+struct ArgmaxAdvance {
+  int64_t* history;
+  int64_t history_ld;
+  int64_t* count;
+  int64_t* positions;
+  int* ctx_len;
+};
+
+__global__ __launch_bounds__(1024) void argmax_rows_kernel(const uint16_t* x, int64_t ld, int64_t* out, int cols, const ArgmaxAdvance adv) {
   __shared__ float sv[16];
   __shared__ int si[16];
   const uint16_t* xr = x + (int64_t)blockIdx.x * ld;
@@ -596,7 +607,8 @@ __global__ __launch_bounds__(1024) void argmax_rows_kernel(const uint16_t* x, in
   const bool vec = ((reinterpret_cast<uintptr_t>(xr) & 15) == 0);
   const int npacks = vec ? cols / 8 : 0;
   // eight packs in flight per thread (a pack past the end re-reads the last one and is skipped): one round trip
-  // covers 64 Ki elements of the row
+  // covers 64 Ki elements of the row.  A thread meets its elements in ascending index order, so inside the thread
+  // "strictly larger" keeps the lowest index of equal values; the full (value, index) order is needed only across lanes.
   for (int q0 = tid; q0 < npacks; q0 += 8 * 1024) {
     uint4 pk[8];
 #pragma unroll
@@ -608,8 +620,9 @@ __global__ __launch_bounds__(1024) void argmax_rows_kernel(const uint16_t* x, in
         const uint32_t w[4] = {pk[u].x, pk[u].y, pk[u].z, pk[u].w};
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-          argmax_take(bv, bi, bf16_lo(w[e]), q * 8 + 2 * e);
-          argmax_take(bv, bi, bf16_hi(w[e]), q * 8 + 2 * e + 1);
+          const float lo = bf16_lo(w[e]), hi = bf16_hi(w[e]);
+          if (lo > bv) { bv = lo; bi = q * 8 + 2 * e; }
+          if (hi > bv) { bv = hi; bi = q * 8 + 2 * e + 1; }
         }
       }
     }
@@ -629,17 +642,31 @@ __global__ __launch_bounds__(1024) void argmax_rows_kernel(const uint16_t* x, in
   if (tid == 0) {
 #pragma unroll
     for (int w = 1; w < 16; w++) argmax_take(bv, bi, sv[w], si[w]);
-    out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
+    const int64_t idx = bi == 0x7fffffff ? 0 : bi;
+    const int64_t r = blockIdx.x;
+    out[r] = idx;
+    if (adv.count) {
+      const int64_t c = adv.count[r];
+      if (adv.history && c >= 0 && c < adv.history_ld) adv.history[r * adv.history_ld + c] = idx;
+      adv.count[r] = c + 1;
+    }
+    if (adv.positions) adv.positions[r] += 1;
+    if (adv.ctx_len) adv.ctx_len[r] += 1;
   }
 }
 
-int argmax_dispatch(const void* x, int64_t ld, void* out, int64_t rows, int cols, hipStream_t stream) {
+int argmax_dispatch(const void* x, int64_t ld, void* out, int64_t rows, int cols, void* history, int64_t history_ld,
+                    void* count, void* positions, void* ctx_len, hipStream_t stream) {
   if (rows < 0 || cols <= 0 || ld < cols) return TBIK_ERR_INVALID;
+  if (history && (!count || history_ld <= 0)) return TBIK_ERR_INVALID;
   if (rows == 0) return TBIK_OK;
   if (!x || !out || rows > 0x7fffffff) return TBIK_ERR_INVALID;
-  if ((reinterpret_cast<uintptr_t>(x) & 1) || (reinterpret_cast<uintptr_t>(out) & 7)) return TBIK_ERR_ALIGNMENT;
+  auto mis = [](const void* p, uintptr_t m) { return (reinterpret_cast<uintptr_t>(p) & m) != 0; };
+  if (mis(x, 1) || mis(out, 7) || mis(history, 7) || mis(count, 7) || mis(positions, 7) || mis(ctx_len, 3)) return TBIK_ERR_ALIGNMENT;
+  const ArgmaxAdvance adv{static_cast<int64_t*>(history), history_ld, static_cast<int64_t*>(count),
+                          static_cast<int64_t*>(positions), static_cast<int*>(ctx_len)};
   hipLaunchKernelGGL(argmax_rows_kernel, dim3((unsigned)rows), dim3(1024), 0, stream, static_cast<const uint16_t*>(x), ld,
-                     static_cast<int64_t*>(out), cols);
+                     static_cast<int64_t*>(out), cols, adv);
   return hip_code(hipGetLastError());
 }
 

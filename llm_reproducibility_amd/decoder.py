@@ -148,12 +148,6 @@ class Qwen3Decoder:
         h, _ = rms_norm(x, self.final_norm, self.cfg.rms_eps, residual=residual)
         return matmul_persistent(h, self.lm_head.t())
 
-    @staticmethod
-    def _greedy(logits: torch.Tensor) -> torch.Tensor:
-        """argmax with ties resolved to the lowest index (a total order on (value, index): no dependence on how the
-        row is reduced)."""
-        return ops.bi_argmax(logits)
-
     # ------------------------------------------------------------------------------------------
     @torch.no_grad()
     def generate(self, prompts: List[List[int]], max_new_tokens: int, return_logits: bool = False):
@@ -178,27 +172,27 @@ class Qwen3Decoder:
         x, res = self._forward(tok, pos, seq, q_start, q_len, ctx, max(lens), cache)
         last = torch.tensor([s + n - 1 for s, n in zip(starts, lens)], dtype=torch.long, device=dev)
         logits = self._logits(x[last].contiguous(), res[last].contiguous())
-        out_ids = [self._greedy(logits)]
         all_logits = [logits] if return_logits else None
         # ---- decode: one token per sequence per step
         q_start = torch.arange(B, dtype=torch.int32, device=dev)
         q_len = torch.ones(B, dtype=torch.int32, device=dev)
         seq = torch.arange(B, dtype=torch.long, device=dev)
-        # the step works on static tensors, so that it can be captured once and replayed
-        tok_s = out_ids[-1].clone()
+        # The step works on static tensors, so that it can be captured once and replayed.  The token choice writes the
+        # next token, files it in the output and advances the positions and cache lengths in its own launch: at a
+        # small batch a step is a chain of short kernels, and each of those updates would be one more.
+        ids = torch.zeros((B, max_new_tokens), dtype=torch.long, device=dev)
+        n_out = torch.zeros(B, dtype=torch.long, device=dev)
+        tok_s = torch.empty(B, dtype=torch.long, device=dev)
         pos_s = torch.tensor(lens, dtype=torch.long, device=dev)
         ctx_s = (pos_s + 1).to(torch.int32)
+        ops.bi_argmax_advance(logits, tok_s, ids, n_out)       # the prompt's last position chooses the first new token
 
         def step():
             logits = self._logits(*self._forward(tok_s, pos_s, seq, q_start, q_len, ctx_s, 1, cache))
-            nxt = self._greedy(logits)
-            tok_s.copy_(nxt)
-            pos_s.add_(1)
-            ctx_s.add_(1)
-            return nxt, logits
+            ops.bi_argmax_advance(logits, tok_s, ids, n_out, pos_s, ctx_s)
+            return logits
 
-        def record(nxt, logits):
-            out_ids.append(nxt.clone())
+        def record(logits):
             if return_logits:
                 all_logits.append(logits.clone())
 
@@ -207,16 +201,15 @@ class Qwen3Decoder:
             side = torch.cuda.Stream(device=dev)
             side.wait_stream(torch.cuda.current_stream(dev))
             with torch.cuda.stream(side):
-                record(*step())          # first step eagerly on the capture stream (also warms every kernel up)
+                record(step())           # first step eagerly on the capture stream (also warms every kernel up)
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, stream=side):
-                static_next, static_logits = step()
+                static_logits = step()
             torch.cuda.current_stream(dev).wait_stream(side)
             for _ in range(steps - 1):
                 graph.replay()
-                record(static_next, static_logits)
+                record(static_logits)
         else:
             for _ in range(steps):
-                record(*step())
-        ids = torch.stack(out_ids, dim=1)
+                record(step())
         return (ids, torch.stack(all_logits, dim=1)) if return_logits else ids

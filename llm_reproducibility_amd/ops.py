@@ -544,3 +544,34 @@ def bi_argmax(logits: torch.Tensor) -> torch.Tensor:
     rc = _lib.lib().bi_argmax_bf16(x.data_ptr(), x.stride(0) if x.shape[0] > 1 else max(x.stride(0), x.shape[1]), out.data_ptr(), x.shape[0], x.shape[1], _stream(x))
     _lib.check(rc, "bi_argmax_bf16")
     return out
+
+
+def bi_argmax_advance(logits: torch.Tensor, next_token: torch.Tensor, history: Optional[torch.Tensor] = None,
+                      count: Optional[torch.Tensor] = None, positions: Optional[torch.Tensor] = None,
+                      ctx_len: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """bi_argmax written into `next_token` (int64 [rows]) plus the bookkeeping of a decode step in the same launch:
+    the index also goes to history[r, count[r]] (int64 [rows, T]; skipped once count[r] reaches T), then count[r]
+    (int64), positions[r] (int64) and ctx_len[r] (int32) advance by one.  All tensors are updated in place."""
+    _require_gpu(logits)
+    if logits.dim() != 2 or logits.dtype != torch.bfloat16:
+        raise NotImplementedError("bi_argmax_advance takes a 2-D bfloat16 tensor")
+    x = logits if logits.stride(1) == 1 else logits.contiguous()
+    rows = x.shape[0]
+
+    def arg(t, dtype, shape, name):
+        if t is None:
+            return 0
+        if t.dtype != dtype or tuple(t.shape) != shape or not t.is_contiguous() or t.device != x.device:
+            raise ValueError(f"{name}: a contiguous {dtype} tensor of shape {shape} on {x.device} is required")
+        return t.data_ptr()
+
+    if history is not None and (history.dim() != 2 or count is None):
+        raise ValueError("history is [rows, T] and needs count")
+    T = history.shape[1] if history is not None else 0
+    rc = _lib.lib().bi_argmax_advance_bf16(
+        x.data_ptr(), x.stride(0) if rows > 1 else max(x.stride(0), x.shape[1]),
+        arg(next_token, torch.int64, (rows,), "next_token"), rows, x.shape[1],
+        arg(history, torch.int64, (rows, T), "history"), T, arg(count, torch.int64, (rows,), "count"),
+        arg(positions, torch.int64, (rows,), "positions"), arg(ctx_len, torch.int32, (rows,), "ctx_len"), _stream(x))
+    _lib.check(rc, "bi_argmax_advance_bf16")
+    return next_token

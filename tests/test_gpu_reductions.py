@@ -551,6 +551,44 @@ def test_argmax_lowest_index_on_ties(dev):
     assert torch.equal(ops.bi_argmax(view), ops.bi_argmax(view.contiguous()))
 
 
+def test_argmax_with_step_bookkeeping_equals_argmax_and_the_separate_updates(dev):
+    """The token choice that also files the token and advances the sequence state (one launch of a decode step):
+    same index as bi_argmax / the oracle on rows full of ties, history written at each row's own count, a full
+    history left alone, and every optional argument may be absent."""
+    from llm_reproducibility_amd import ops
+    g = torch.Generator().manual_seed(11)
+    rows, cols, T = 5, 151936, 3
+    nxt = torch.full((rows,), -1, dtype=torch.int64, device=dev)
+    hist = torch.full((rows, T), -7, dtype=torch.int64, device=dev)
+    count = torch.tensor([0, 1, 2, 3, 0], dtype=torch.int64, device=dev)       # row 3: history already full
+    pos = torch.tensor([10, 0, 5, 99, 2 ** 40], dtype=torch.int64, device=dev)
+    ctx = torch.tensor([11, 1, 6, 100, 7], dtype=torch.int32, device=dev)
+    want_hist = hist.clone()
+    for stepno in range(2):
+        x = torch.randn((rows, cols), generator=g).to(torch.bfloat16)
+        want = O.argmax_lowest_index(x)
+        c0, p0, l0 = count.clone(), pos.clone(), ctx.clone()
+        got = ops.bi_argmax_advance(x.to(dev), nxt, hist, count, pos, ctx)
+        assert got is nxt and torch.equal(nxt.cpu(), want) and torch.equal(nxt, ops.bi_argmax(x.to(dev))), stepno
+        for r in range(rows):
+            if int(c0[r]) < T:
+                want_hist[r, int(c0[r])] = want[r]
+        assert torch.equal(hist, want_hist), stepno
+        assert torch.equal(count, c0 + 1) and torch.equal(pos, p0 + 1) and torch.equal(ctx, l0 + 1), stepno
+    # nothing but the token
+    x = torch.randn((2, 1000), generator=g).to(torch.bfloat16)
+    two = torch.empty(2, dtype=torch.int64, device=dev)
+    assert torch.equal(ops.bi_argmax_advance(x.to(dev), two).cpu(), O.argmax_lowest_index(x))
+    # positions only; and a history without its count is refused
+    p1 = torch.zeros(2, dtype=torch.int64, device=dev)
+    ops.bi_argmax_advance(x.to(dev), two, positions=p1)
+    assert p1.tolist() == [1, 1]
+    with pytest.raises(ValueError):
+        ops.bi_argmax_advance(x.to(dev), two, history=torch.zeros((2, 4), dtype=torch.int64, device=dev))
+    with pytest.raises(ValueError):
+        ops.bi_argmax_advance(x.to(dev), two, ctx_len=torch.zeros(2, dtype=torch.int64, device=dev))   # int32 required
+
+
 def test_aten_overrides_route_to_the_hip_kernels(dev):
     a = O.gaussian_bf16((20, 512), 1.0, 0).to(dev)
     w = O.gaussian_bf16((64, 512), 0.1, 1).to(dev)
