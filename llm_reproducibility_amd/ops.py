@@ -506,8 +506,14 @@ def gemm_tree_silu_mul(gate: torch.Tensor, up: torch.Tensor, B: torch.Tensor, bi
             return C
         if rc != _lib.TBIK_ERR_UNSUPPORTED:
             _lib.check(rc, "tbik_gemm_silu_mul_bf16")
-    act = bi_silu_mul(torch.cat((gate, up), dim=-1))
-    return gemm_tree(act, B, bias, leaf_k)
+    if (gate.dim() == 2 and up.shape == gate.shape and gate.stride(1) == 1 and up.stride(1) == 1 and gate.stride(0) == up.stride(0)
+            and gate.dtype == up.dtype and up.data_ptr() == gate.data_ptr() + K * gate.element_size()
+            and (M == 1 or gate.stride(0) >= 2 * K)):
+        # the two halves of one merged projection, side by side in memory: the activation kernel reads them in place
+        merged = torch.as_strided(gate, (M, 2 * K), (gate.stride(0), 1))
+    else:
+        merged = torch.cat((gate, up), dim=-1)
+    return gemm_tree(bi_silu_mul(merged), B, bias, leaf_k)
 
 
 # --------------------------------------------------------------------------------------------
