@@ -394,6 +394,46 @@ int tbik_gemm_silu_mul_bf16(const void* gate, const void* up, int64_t ld,
                             const void* bias_or_null,
                             tbik_stream_t stream);
 
+/*
+ * The consumer side of a row-split layer in the same launch as the layer's last pass: the (add-)RMSNorm that follows
+ * o_proj and down_proj in a decoder block, computed by the kernel that combines the K shards, so the layer's output
+ * never goes through memory un-normalised.  Both evaluate exactly the expressions of the separate calls (the shard
+ * tree of tbik_tree_combine_bf16 with the bias behind it, then the row function of bi_rmsnorm_bf16), so the results
+ * are bit-identical to those.
+ *
+ * tbik_gemm_rmsnorm_bf16:  out[M,N] = bi_rmsnorm_bf16( tbik_gemm_bf16(A, B, leaf_k) (+ bias) [+ residual], norm_weight, eps )
+ *   residual [M,N] or NULL; with a residual, residual_out [M,N] receives bf16(result + residual) (it may be the
+ *   residual itself).  workspace as for tbik_gemm_bf16 (tbik_gemm_workspace_bytes of the same M, N, K, leaf_k).
+ *   Returns TBIK_ERR_UNSUPPORTED (3), with nothing launched, where the matmul of this shape does not end in one shard
+ *   combine over whole rows (a handful of rows: the one-launch kernel; large M: column regions or no K split) or
+ *   N > 8192: the caller then runs tbik_gemm_bf16 and bi_rmsnorm_bf16.
+ *   Replaces: the patched RowParallelLinear forward (src/patch/patch_tp_invariant.py:10-48) followed by the model's
+ *             fused add-RMSNorm routed through the batch-invariant mean (src/patch/patch_batch_invariant.py:9-16).
+ *
+ * tbik_tree_combine_rmsnorm_bf16:  the same for partials that the caller holds (the ranks' results of a row-split layer
+ *   brought to one GPU): parts = nparts (2..32, a power of two) device pointers to contiguous [rows, hidden] arrays,
+ *   hidden a multiple of 8 and <= 8192, everything 16-byte aligned.
+ *   Replaces: tree_all_reduce_sum (src/tbik/tree_based_all_reduce.py:9-37) followed by that add-RMSNorm.
+ */
+int tbik_gemm_rmsnorm_bf16(const void* A, int64_t lda,
+                           const void* B, int64_t ldb_k, int64_t ldb_n,
+                           int M, int N, int K, int leaf_k,
+                           const void* bias_or_null,
+                           const void* residual_or_null, int64_t ldr,
+                           const void* norm_weight_or_null, float eps,
+                           void* residual_out_or_null, int64_t ldro,
+                           void* out, int64_t ldo,
+                           void* workspace, size_t workspace_bytes,
+                           tbik_stream_t stream);
+int tbik_tree_combine_rmsnorm_bf16(const void* const* parts, int nparts,
+                                   int64_t rows, int hidden,
+                                   const void* bias_or_null,
+                                   const void* residual_or_null, int64_t ldr,
+                                   const void* norm_weight_or_null, float eps,
+                                   void* residual_out_or_null, int64_t ldro,
+                                   void* out, int64_t ldo,
+                                   tbik_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

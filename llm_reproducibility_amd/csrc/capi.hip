@@ -32,13 +32,20 @@ int silu_mul_dispatch(const void* gate_up, int64_t ld_in, void* out, int64_t ld_
 int rmsnorm_gemm_dispatch(const void* x, int64_t ldx, const void* res, int64_t ldr, const void* norm_w, float eps,
                           void* res_out, int64_t ldro, const void* B, int64_t ldb_k, int64_t ldb_n, void* C, int64_t ldc,
                           int M, int N, int K, const void* bias, hipStream_t stream);
+int gemm_tree_rmsnorm_dispatch(bool f16, const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, int M, int N,
+                               int K, int leaf_k, const void* bias, const void* res, int64_t ldr, const void* norm_w, float eps,
+                               void* res_out, int64_t ldro, void* out, int64_t ldo, void* ws, size_t ws_bytes,
+                               hipStream_t stream);
+int tree_combine_rmsnorm_dispatch(const void* const* parts, int nparts, int64_t rows, int hidden, const void* bias,
+                                  const void* res, int64_t ldr, const void* w, float eps, void* out, int64_t ldo,
+                                  void* res_out, int64_t ldro, void* sum_out, int64_t lds, bool f16, hipStream_t stream);
 int gemm_tree_gated_dispatch(const void* gate, const void* up, int64_t ld, const void* B, int64_t ldb_k, int64_t ldb_n, void* C,
                              int64_t ldc, int M, int N, int K, int leaf_k, const void* bias, hipStream_t stream);
 }  // namespace tbik
 
 extern "C" {
 
-int tbik_abi_version(void) { return 14; }
+int tbik_abi_version(void) { return 15; }
 
 const char* tbik_error_string(int code) {
   switch (code) {
@@ -123,6 +130,23 @@ int tbik_gemm_silu_mul_bf16(const void* gate, const void* up, int64_t ld, const 
                             int64_t ldc, int M, int N, int K, int leaf_k, const void* bias_or_null, tbik_stream_t stream) {
   return tbik::gemm_tree_gated_dispatch(gate, up, ld, B, ldb_k, ldb_n, C, ldc, M, N, K, leaf_k, bias_or_null,
                                         static_cast<hipStream_t>(stream));
+}
+
+int tbik_gemm_rmsnorm_bf16(const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, int M, int N, int K,
+                           int leaf_k, const void* bias_or_null, const void* residual_or_null, int64_t ldr,
+                           const void* norm_weight_or_null, float eps, void* residual_out_or_null, int64_t ldro, void* out,
+                           int64_t ldo, void* workspace, size_t workspace_bytes, tbik_stream_t stream) {
+  return tbik::gemm_tree_rmsnorm_dispatch(false, A, lda, B, ldb_k, ldb_n, M, N, K, leaf_k, bias_or_null, residual_or_null, ldr,
+                                          norm_weight_or_null, eps, residual_out_or_null, ldro, out, ldo, workspace,
+                                          workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+int tbik_tree_combine_rmsnorm_bf16(const void* const* parts, int nparts, int64_t rows, int hidden, const void* bias_or_null,
+                                   const void* residual_or_null, int64_t ldr, const void* norm_weight_or_null, float eps,
+                                   void* residual_out_or_null, int64_t ldro, void* out, int64_t ldo, tbik_stream_t stream) {
+  return tbik::tree_combine_rmsnorm_dispatch(parts, nparts, rows, hidden, bias_or_null, residual_or_null, ldr,
+                                             norm_weight_or_null, eps, out, ldo, residual_out_or_null, ldro, nullptr, 0, false,
+                                             static_cast<hipStream_t>(stream));
 }
 
 int bi_rmsnorm_bf16(const void* x, int64_t ldx, const void* residual_or_null, int64_t ldr, const void* weight_or_null,

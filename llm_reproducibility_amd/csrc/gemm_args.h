@@ -105,4 +105,21 @@ int gemm_tree_strip_gated_launch(const StripArgs& a, int leaf_k, int waves, hipS
 int tree_combine_bias_dispatch(const void* const* parts, int nparts, void* out, int64_t numel, const void* bias, int N,
                                bool f16, hipStream_t stream, int64_t ldo = 0);
 
+// the shard combine with the (add-)RMSNorm of the combined rows behind it in the same launch: out = normalised rows,
+// res_out = combined + residual (with res), sum_out (optional) = the combined rows themselves
+int tree_combine_rmsnorm_dispatch(const void* const* parts, int nparts, int64_t rows, int hidden, const void* bias,
+                                  const void* res, int64_t ldr, const void* w, float eps, void* out, int64_t ldo,
+                                  void* res_out, int64_t ldro, void* sum_out, int64_t lds, bool f16, hipStream_t stream);
+
+// What follows a tree matmul whose K split ends in a shard combine, when the caller wants the (add-)RMSNorm of the result
+// in that combine's launch: the matmul's C / ldc arguments then name the NORMALISED output.
+struct NormEpilogue {
+  const void* res;   // optional residual [M, ldr]
+  int64_t ldr;
+  const void* w;     // optional norm weight [N]
+  float eps;
+  void* res_out;     // result + residual [M, ldro] (with res)
+  int64_t ldro;
+};
+
 }  // namespace tbik

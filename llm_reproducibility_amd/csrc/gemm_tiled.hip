@@ -663,7 +663,7 @@ int gemm_plan_info(int M, int N, int K, int leaf_k, bool f16, bool rowmajor_b, i
 
 static int gemm_dispatch_impl(bool tree, bool f16, const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n,
                               void* C, int64_t ldc, int M, int N, int K, int leaf_k, const void* bias, void* ws,
-                              size_t ws_bytes, hipStream_t stream, bool whole_problem);
+                              size_t ws_bytes, hipStream_t stream, bool whole_problem, const NormEpilogue* ep = nullptr);
 
 int gemm_dispatch(bool tree, bool f16, const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, void* C,
                   int64_t ldc, int M, int N, int K, int leaf_k, const void* bias, void* ws, size_t ws_bytes,
@@ -671,9 +671,24 @@ int gemm_dispatch(bool tree, bool f16, const void* A, int64_t lda, const void* B
   return gemm_dispatch_impl(tree, f16, A, lda, B, ldb_k, ldb_n, C, ldc, M, N, K, leaf_k, bias, ws, ws_bytes, stream, true);
 }
 
+// The tree matmul with the (add-)RMSNorm of its result inside the launch of its shard combine: `out` receives the
+// normalised rows, res_out the result + residual.  TBIK_ERR_UNSUPPORTED (nothing launched) where the matmul of this shape
+// has no shard combine over whole rows; the caller then runs the matmul and the norm as two calls.  Same bits either way.
+int gemm_tree_rmsnorm_dispatch(bool f16, const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, int M, int N,
+                               int K, int leaf_k, const void* bias, const void* res, int64_t ldr, const void* norm_w, float eps,
+                               void* res_out, int64_t ldro, void* out, int64_t ldo, void* ws, size_t ws_bytes,
+                               hipStream_t stream) {
+  if (res && !res_out) return TBIK_ERR_INVALID;
+  if (M <= 0 || N <= 0) return TBIK_ERR_UNSUPPORTED;
+  auto bad = [](const void* p, int64_t ld) { return (reinterpret_cast<uintptr_t>(p) & 15) != 0 || (ld & 7) != 0; };
+  if ((res && (bad(res, ldr) || bad(res_out, ldro) || ldr < N || ldro < N)) || (norm_w && bad(norm_w, 8))) return TBIK_ERR_ALIGNMENT;
+  const NormEpilogue ep{res, ldr, norm_w, eps, res ? res_out : nullptr, ldro};
+  return gemm_dispatch_impl(true, f16, A, lda, B, ldb_k, ldb_n, out, ldo, M, N, K, leaf_k, bias, ws, ws_bytes, stream, true, &ep);
+}
+
 static int gemm_dispatch_impl(bool tree, bool f16, const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n,
                               void* C, int64_t ldc, int M, int N, int K, int leaf_k, const void* bias, void* ws,
-                              size_t ws_bytes, hipStream_t stream, bool whole_problem) {
+                              size_t ws_bytes, hipStream_t stream, bool whole_problem, const NormEpilogue* ep) {
   if (M < 0 || N < 0 || K <= 0) return TBIK_ERR_INVALID;
   if (M == 0 || N == 0) return TBIK_OK;  // nothing to do (empty tensors may come with null pointers)
   if (!A || !B || !C) return TBIK_ERR_INVALID;
@@ -736,6 +751,18 @@ static int gemm_dispatch_impl(bool tree, bool f16, const void* A, int64_t lda, c
   if (leaf_k != 256 && leaf_k != 128) return TBIK_ERR_UNSUPPORTED;
   TreePlan tp;
   if (!tree_plan(M, N, K, leaf_k, f16, rowmajor_b, whole_problem, &tp)) return TBIK_ERR_INVALID;
+  if (ep) {
+    // the norm rides on the shard combine of ONE K split over all columns: nothing else has a pass over whole rows
+    const bool combines = (tp.path == PATH_NARROW && tp.narrow.split > 1) || (tp.path == PATH_SINGLE && tp.single.split > 1);
+    if (!combines || N > 16 * 512 || (N & 7) || !aligned16(C) || (ldc & 7)) return TBIK_ERR_UNSUPPORTED;
+  }
+  auto combine = [&](const void* const* parts, int nparts) {
+    if (ep)
+      return tree_combine_rmsnorm_dispatch(parts, nparts, M, N, bias, ep->res, ep->ldr, ep->w, ep->eps, C, ldc, ep->res_out,
+                                           ep->ldro, nullptr, 0, f16, stream);
+    // one launch adds the shards (and the bias) in tree order, into C's own row stride
+    return tree_combine_bias_dispatch(parts, nparts, C, (int64_t)M * N, bias, N, f16, stream, ldc);
+  };
   if (tp.path == PATH_STRIP) {
     // a handful of rows: one launch, K cut over the waves of a work-group, nothing goes through the workspace
     int T, flb, level_k;
@@ -759,7 +786,7 @@ static int gemm_dispatch_impl(bool tree, bool f16, const void* A, int64_t lda, c
     if (rc != TBIK_OK || np.split == 1) return rc;
     const void* parts[32];
     for (int i = 0; i < np.split; i++) parts[i] = static_cast<uint8_t*>(ws) + (size_t)i * M * N * sizeof(uint16_t);
-    return tree_combine_bias_dispatch(parts, np.split, C, (int64_t)M * N, bias, N, f16, stream, ldc);
+    return combine(parts, np.split);
   }
   if (tp.path == PATH_REGIONS) {
     const RegionPlan& rp = tp.regions;
@@ -846,8 +873,7 @@ static int gemm_dispatch_impl(bool tree, bool f16, const void* A, int64_t lda, c
   if (rc != TBIK_OK || pl.split == 1) return rc;
   const void* parts[32];
   for (int i = 0; i < pl.split; i++) parts[i] = wsb + (size_t)i * M * N * sizeof(uint16_t);
-  // one launch adds the shards (and the bias) in tree order, into C's own row stride
-  return tree_combine_bias_dispatch(parts, pl.split, C, (int64_t)M * N, bias, N, f16, stream, ldc);
+  return combine(parts, pl.split);
 }
 
 // ------------------------------------------------------------------------------------------------

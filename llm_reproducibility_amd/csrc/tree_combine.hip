@@ -4,6 +4,7 @@
 // mini_allreduce/tbik_kernel/csrc/allreduce/custom_all_reduce.cuh:203-234) applied to partials that
 // already sit in one GPU's memory.  HBM bound: (nparts + 1) * numel * 2 bytes.
 #include "common.h"
+#include "rmsnorm_row.h"
 
 namespace tbik {
 
@@ -28,6 +29,32 @@ __device__ __forceinline__ uint32_t tree_node(const uint32_t (&v)[NP]) {
   return w[0];
 }
 
+// The tree over the NP partial packs of one 16-byte pack (8 elements), and the bias added to it: one body for every
+// kernel that combines shards, so they all give the same bits.
+template <int NP, bool F16>
+__device__ __forceinline__ uint4 combine_pack(const uint4 (&in)[NP]) {
+  uint4 o;
+  uint32_t v[NP];
+#pragma unroll
+  for (int p = 0; p < NP; p++) v[p] = in[p].x;
+  o.x = tree_node<NP, F16>(v);
+#pragma unroll
+  for (int p = 0; p < NP; p++) v[p] = in[p].y;
+  o.y = tree_node<NP, F16>(v);
+#pragma unroll
+  for (int p = 0; p < NP; p++) v[p] = in[p].z;
+  o.z = tree_node<NP, F16>(v);
+#pragma unroll
+  for (int p = 0; p < NP; p++) v[p] = in[p].w;
+  o.w = tree_node<NP, F16>(v);
+  return o;
+}
+
+template <bool F16>
+__device__ __forceinline__ uint4 add_pack(const uint4& o, const uint4& bq) {
+  return make_uint4(Num16<F16>::add(o.x, bq.x), Num16<F16>::add(o.y, bq.y), Num16<F16>::add(o.z, bq.z), Num16<F16>::add(o.w, bq.w));
+}
+
 // One thread per 16-byte pack (8 bf16); grid-stride so any numel fits one launch.
 template <int NP, bool F16>
 __global__ __launch_bounds__(256) void combine_vec_kernel(const CombineArgs a, int64_t npacks) {
@@ -36,27 +63,9 @@ __global__ __launch_bounds__(256) void combine_vec_kernel(const CombineArgs a, i
     uint4 in[NP];
 #pragma unroll
     for (int p = 0; p < NP; p++) in[p] = reinterpret_cast<const uint4*>(a.parts[p])[i];
-    uint4 o;
-    uint32_t v[NP];
-#pragma unroll
-    for (int p = 0; p < NP; p++) v[p] = in[p].x;
-    o.x = tree_node<NP, F16>(v);
-#pragma unroll
-    for (int p = 0; p < NP; p++) v[p] = in[p].y;
-    o.y = tree_node<NP, F16>(v);
-#pragma unroll
-    for (int p = 0; p < NP; p++) v[p] = in[p].z;
-    o.z = tree_node<NP, F16>(v);
-#pragma unroll
-    for (int p = 0; p < NP; p++) v[p] = in[p].w;
-    o.w = tree_node<NP, F16>(v);
-    if (a.bias) {  // ncols % 8 == 0 on this path: the pack stays inside one row
-      const uint4 bq = *reinterpret_cast<const uint4*>(a.bias + (i * 8) % a.ncols);
-      o.x = Num16<F16>::add(o.x, bq.x);
-      o.y = Num16<F16>::add(o.y, bq.y);
-      o.z = Num16<F16>::add(o.z, bq.z);
-      o.w = Num16<F16>::add(o.w, bq.w);
-    }
+    uint4 o = combine_pack<NP, F16>(in);
+    // ncols % 8 == 0 on this path: the pack stays inside one row
+    if (a.bias) o = add_pack<F16>(o, *reinterpret_cast<const uint4*>(a.bias + (i * 8) % a.ncols));
     if (a.ldo) {  // ncols % 8 == 0 and aligned rows on this path
       const int64_t e = i * 8, r = e / a.ncols;
       *reinterpret_cast<uint4*>(a.out + r * a.ldo + (e - r * a.ncols)) = o;
@@ -141,6 +150,130 @@ int tree_combine_bias_dispatch(const void* const* parts, int nparts, void* out, 
     case 16: return launch_combine<16, false>(a, vec_ok, stream);
     default: return launch_combine<32, false>(a, vec_ok, stream);
   }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Shard combine followed by the (add-)RMSNorm of the combined rows, in one launch: one wavefront per row forms the
+// row's packs exactly as combine_vec_kernel does (tree over the partials, then the bias) and hands them, still in
+// registers, to the row function of the stand-alone RMSNorm (rmsnorm_row.h) in the lane layout that function expects.
+// Same bits as the two launches; a decode-sized batch saves a kernel per row-split layer.
+// ------------------------------------------------------------------------------------------------
+struct CombineNormArgs {
+  const uint16_t* parts[32];  // [rows, hidden] each, contiguous
+  const uint16_t* bias;       // optional [hidden]
+  const uint16_t* res;        // optional residual [rows, ldr]
+  const uint16_t* w;          // optional norm weight [hidden]
+  uint16_t* out;              // normalised rows [rows, ldo]
+  uint16_t* res_out;          // combined + residual [rows, ldro] (with res)
+  uint16_t* sum_out;          // optional: the combined rows themselves [rows, lds]
+  int64_t ldr, ldo, ldro, lds;
+  int64_t rows;
+  int hidden;
+  float eps;
+};
+
+template <int NP, int CPL, bool F16>
+__global__ __launch_bounds__(256) void combine_rmsnorm_kernel(const CombineNormArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= a.rows) return;
+  const int nchunks = a.hidden >> 3;
+  RmsnormRow<CPL, F16> r;
+  r.has_res = a.res != nullptr;
+  r.has_w = a.w != nullptr;
+  const uint4* wr = reinterpret_cast<const uint4*>(a.w);
+  const uint4* rr = a.res ? reinterpret_cast<const uint4*>(a.res + row * a.ldr) : nullptr;
+  const uint4* br = reinterpret_cast<const uint4*>(a.bias);
+  // every load of the row goes out before the first store (the residual output may alias the residual)
+#pragma unroll
+  for (int i = 0; i < CPL; i++) {
+    const int c = lane + 64 * i;
+    if (c < nchunks) {
+      if (wr) r.wq[i] = wr[c];
+      if (rr) r.rq[i] = rr[c];
+      uint4 in[NP];
+#pragma unroll
+      for (int p = 0; p < NP; p++) in[p] = reinterpret_cast<const uint4*>(a.parts[p] + row * a.hidden)[c];
+      uint4 o = combine_pack<NP, F16>(in);
+      if (br) o = add_pack<F16>(o, br[c]);
+      r.xq[i] = o;
+    }
+  }
+  if (a.sum_out) {
+    uint4* srow = reinterpret_cast<uint4*>(a.sum_out + row * a.lds);
+#pragma unroll
+    for (int i = 0; i < CPL; i++) {
+      const int c = lane + 64 * i;
+      if (c < nchunks) srow[c] = r.xq[i];
+    }
+  }
+  uint4* orow = reinterpret_cast<uint4*>(a.out + row * a.ldo);
+  r.finish(a.res_out ? a.res_out + row * a.ldro : nullptr, a.hidden, a.eps, lane, [&](int c, const uint4& o) { orow[c] = o; });
+}
+
+template <int NP, bool F16>
+static void launch_combine_rmsnorm(const CombineNormArgs& a, dim3 grid, hipStream_t stream) {
+  const int cpl = (a.hidden + 511) / 512;  // a function of the row length only
+  if (cpl <= 2) hipLaunchKernelGGL((combine_rmsnorm_kernel<NP, 2, F16>), grid, dim3(256), 0, stream, a);
+  else if (cpl <= 8) hipLaunchKernelGGL((combine_rmsnorm_kernel<NP, 8, F16>), grid, dim3(256), 0, stream, a);
+  else hipLaunchKernelGGL((combine_rmsnorm_kernel<NP, 16, F16>), grid, dim3(256), 0, stream, a);
+}
+
+int tree_combine_rmsnorm_dispatch(const void* const* parts, int nparts, int64_t rows, int hidden, const void* bias,
+                                  const void* res, int64_t ldr, const void* w, float eps, void* out, int64_t ldo,
+                                  void* res_out, int64_t ldro, void* sum_out, int64_t lds, bool f16, hipStream_t stream) {
+  if (rows < 0 || hidden <= 0) return TBIK_ERR_INVALID;
+  if (nparts < 2 || nparts > 32 || (nparts & (nparts - 1))) return TBIK_ERR_INVALID;
+  if (rows == 0) return TBIK_OK;
+  if (!parts || !out || (res && !res_out)) return TBIK_ERR_INVALID;
+  if (hidden & 7) return TBIK_ERR_ALIGNMENT;
+  if (hidden > 16 * 512) return TBIK_ERR_UNSUPPORTED;
+  auto bad = [](const void* p, int64_t ld) { return (reinterpret_cast<uintptr_t>(p) & 15) != 0 || (ld & 7) != 0; };
+  if (bad(out, ldo) || (res && (bad(res, ldr) || bad(res_out, ldro))) || (w && bad(w, 8)) || (bias && bad(bias, 8)) ||
+      (sum_out && bad(sum_out, lds)))
+    return TBIK_ERR_ALIGNMENT;
+  if (ldo < hidden || (res && (ldr < hidden || ldro < hidden)) || (sum_out && lds < hidden)) return TBIK_ERR_INVALID;
+  CombineNormArgs a;
+  for (int p = 0; p < 32; p++) a.parts[p] = nullptr;
+  for (int p = 0; p < nparts; p++) {
+    if (!parts[p]) return TBIK_ERR_INVALID;
+    if (reinterpret_cast<uintptr_t>(parts[p]) & 15) return TBIK_ERR_ALIGNMENT;
+    a.parts[p] = static_cast<const uint16_t*>(parts[p]);
+  }
+  a.bias = static_cast<const uint16_t*>(bias);
+  a.res = static_cast<const uint16_t*>(res);
+  a.w = static_cast<const uint16_t*>(w);
+  a.out = static_cast<uint16_t*>(out);
+  a.res_out = static_cast<uint16_t*>(res ? res_out : nullptr);
+  a.sum_out = static_cast<uint16_t*>(sum_out);
+  a.ldr = ldr;
+  a.ldo = ldo;
+  a.ldro = ldro;
+  a.lds = lds;
+  a.rows = rows;
+  a.hidden = hidden;
+  a.eps = eps;
+  const int64_t blocks = (rows + 3) / 4;
+  if (blocks > 0x7fffffff) return TBIK_ERR_INVALID;
+  const dim3 grid((unsigned)blocks);
+  if (f16) {
+    switch (nparts) {
+      case 2: launch_combine_rmsnorm<2, true>(a, grid, stream); break;
+      case 4: launch_combine_rmsnorm<4, true>(a, grid, stream); break;
+      case 8: launch_combine_rmsnorm<8, true>(a, grid, stream); break;
+      case 16: launch_combine_rmsnorm<16, true>(a, grid, stream); break;
+      default: launch_combine_rmsnorm<32, true>(a, grid, stream); break;
+    }
+  } else {
+    switch (nparts) {
+      case 2: launch_combine_rmsnorm<2, false>(a, grid, stream); break;
+      case 4: launch_combine_rmsnorm<4, false>(a, grid, stream); break;
+      case 8: launch_combine_rmsnorm<8, false>(a, grid, stream); break;
+      case 16: launch_combine_rmsnorm<16, false>(a, grid, stream); break;
+      default: launch_combine_rmsnorm<32, false>(a, grid, stream); break;
+    }
+  }
+  return hip_code(hipGetLastError());
 }
 
 int tree_combine_dispatch(const void* const* parts, int nparts, void* out, int64_t numel, bool f16, hipStream_t stream) {

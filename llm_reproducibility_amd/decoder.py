@@ -61,7 +61,8 @@ class _Layer:
 
 class Qwen3Decoder:
     def __init__(self, cfg: DecoderConfig, tp_size: int = 1, seed: int = 0, device="cuda:0", use_graphs: bool = False,
-                 fused_rope: bool = True, init_on_device: bool = False, fused_producers: bool = True):
+                 fused_rope: bool = True, init_on_device: bool = False, fused_producers: bool = True,
+                 fused_consumers: bool = True):
         assert cfg.head_dim == 128, "the attention kernel is built for head_dim 128"
         self.cfg, self.tp_size, self.device = cfg, tp_size, torch.device(device)
         # decode steps replayed from one captured HIP graph (same kernels, same order, same bits as eager; the
@@ -71,6 +72,9 @@ class Qwen3Decoder:
         # RMSNorm inside the projection that consumes it and SiLU*up inside down_proj (one launch each for a handful of
         # rows, the two launches otherwise; bit-identical either way, so the switch only exists for the tests)
         self.fused_producers = fused_producers
+        # beyond a handful of rows: the add-RMSNorm behind o_proj and down_proj inside the launch that combines the layer's
+        # K shards (bit-identical to the separate norm; the switch only exists for the tests)
+        self.fused_consumers = fused_consumers
         gen = torch.Generator(device=self.device if init_on_device else "cpu").manual_seed(seed)
         emb = lambda *shape: _normal_bf16(shape, gen, self.device)  # noqa: E731
         self.embed = emb(cfg.vocab_size, cfg.hidden_size)
@@ -104,18 +108,21 @@ class Qwen3Decoder:
         Hq, Hkv, D = cfg.num_q_heads, cfg.num_kv_heads, cfg.head_dim
         x = self.embed[token_ids]                                   # [tokens, H]
         residual: Optional[torch.Tensor] = None
-        fused = self.fused_producers
+        fused = self.fused_producers and (x.shape[0] <= 4 or not self.fused_consumers)   # the one-launch producers take a handful of rows
+        h: Optional[torch.Tensor] = None     # the layer's normalised input, when the previous layer's down_proj produced it
         for li, layer in enumerate(self.layers):
             if fused:
                 qkv, new_res = ops.rmsnorm_gemm(x, layer.input_norm, cfg.rms_eps, residual, layer.qkv_w.t())
                 residual = x if residual is None else new_res
             else:
-                if residual is None:
-                    residual = x
-                    h = rms_norm(x, layer.input_norm, cfg.rms_eps)
-                else:
-                    h, residual = rms_norm(x, layer.input_norm, cfg.rms_eps, residual=residual)
+                if h is None:
+                    if residual is None:
+                        residual = x
+                        h = rms_norm(x, layer.input_norm, cfg.rms_eps)
+                    else:
+                        h, residual = rms_norm(x, layer.input_norm, cfg.rms_eps, residual=residual)
                 qkv = matmul_persistent(h, layer.qkv_w.t())
+                h = None
             k_cache, vt_cache = cache[li]
             if self.fused_rope:
                 # per-head q/k norm, rotary embedding and the cache write in one kernel
@@ -130,13 +137,22 @@ class Qwen3Decoder:
                 k_cache[seq_of_token, :, positions] = k             # [tokens, Hkv, D] -> [B, Hkv, L, D]
                 vt_cache[seq_of_token, :, :, positions] = v         # stored transposed: [B, Hkv, D, L]
             attn = ops.bi_attention_bf16(q, k_cache, vt_cache, q_start, q_len, ctx_len, max_q_len, self.scale)
-            x = layer.o_proj(attn.reshape(-1, Hq * D))
             if fused:
+                x = layer.o_proj(attn.reshape(-1, Hq * D))
                 gu, residual = ops.rmsnorm_gemm(x, layer.post_norm, cfg.rms_eps, residual, layer.gate_up_w.t())
                 x = layer.down_proj.forward_gated(gu)
+            elif self.fused_consumers:
+                # the add-RMSNorm behind each row-split layer runs in the launch that combines the layer's K shards
+                hp, residual = layer.o_proj.forward_add_norm(attn.reshape(-1, Hq * D), residual, layer.post_norm, cfg.rms_eps)
+                act = ops.bi_silu_mul(matmul_persistent(hp, layer.gate_up_w.t()))
+                if li + 1 < len(self.layers):
+                    h, residual = layer.down_proj.forward_add_norm(act, residual, self.layers[li + 1].input_norm, cfg.rms_eps)
+                else:
+                    x = layer.down_proj(act)    # the final norm runs on the rows the caller selects
             else:
-                h, residual = rms_norm(x, layer.post_norm, cfg.rms_eps, residual=residual)
-                gu = matmul_persistent(h, layer.gate_up_w.t())
+                x = layer.o_proj(attn.reshape(-1, Hq * D))
+                hp, residual = rms_norm(x, layer.post_norm, cfg.rms_eps, residual=residual)
+                gu = matmul_persistent(hp, layer.gate_up_w.t())
                 act = ops.bi_silu_mul(gu)
                 x = layer.down_proj(act)
         return x, residual

@@ -114,6 +114,25 @@ class SimulatedTPRowLinear(nn.Module):
             out = out + self.bias
         return out.reshape(*lead, out.shape[-1])
 
+    def forward_add_norm(self, x: torch.Tensor, residual: Optional[torch.Tensor], norm_weight: Optional[torch.Tensor], eps: float):
+        """(rms_norm(forward(x) [+ residual]) * norm_weight, new residual or None): the add-RMSNorm that follows a
+        row-split layer in a decoder block, computed by the launch that combines the K shards where there is one
+        (inside the matmul for one rank, the shard combine for several); same bits as forward() and the norm."""
+        from . import ops
+        x2 = x.reshape(-1, x.shape[-1])
+        r2 = None if residual is None else residual.reshape(-1, residual.shape[-1])
+        K = x2.shape[1]
+        ks = K // self.tp_size
+        if self.tp_size == 1:
+            out, res = ops.gemm_tree_add_rmsnorm(x2, self.weight.t(), self.bias, self.leaf_k, r2, norm_weight, eps)
+        else:
+            parts = [matmul_tp_persistent(x2[:, r * ks:(r + 1) * ks], self.weight[:, r * ks:(r + 1) * ks].t(), leaf_k=self.leaf_k)
+                     for r in range(self.tp_size)]
+            out, res = ops.tree_combine_add_rmsnorm(parts, self.bias, r2, norm_weight, eps)
+        lead = x.shape[:-1]
+        out = out.reshape(*lead, out.shape[-1])
+        return out, (None if res is None else res.reshape(*lead, res.shape[-1]))
+
     def forward_gated(self, gate_up: torch.Tensor) -> torch.Tensor:
         """forward(silu(gate) * up) for the merged projection gate_up = [gate | up]: the activation is formed inside the
         per-shard tree matmul where that is one launch (a few rows), by its own kernel otherwise; same bits."""

@@ -517,6 +517,90 @@ def gemm_tree_silu_mul(gate: torch.Tensor, up: torch.Tensor, B: torch.Tensor, bi
 
 
 # --------------------------------------------------------------------------------------------
+# the (add-)RMSNorm behind a row-split layer, inside the launch that combines the layer's K shards
+# --------------------------------------------------------------------------------------------
+def _norm_after(y: torch.Tensor, residual: Optional[torch.Tensor], norm_weight: Optional[torch.Tensor], eps: float):
+    """The two-call form: (bi_rmsnorm(y [+ residual]), new residual or None)."""
+    if residual is None:
+        return bi_rmsnorm(y, norm_weight, eps), None
+    out, res = bi_add_rmsnorm(y, residual, norm_weight, eps)
+    return out, res
+
+
+def gemm_tree_add_rmsnorm(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch.Tensor], leaf_k: int,
+                          residual: Optional[torch.Tensor], norm_weight: Optional[torch.Tensor], eps: float):
+    """(rms_norm(gemm_tree(A, B, bias, leaf_k) [+ residual]) * norm_weight, new residual or None).
+
+    One call (`tbik_gemm_rmsnorm_bf16`: the norm runs in the launch that combines the matmul's K shards) where the matmul
+    of this shape ends in such a combine -- decode- and prefill-sized batches of a row-split layer; the matmul followed
+    by the norm otherwise.  Same bits either way."""
+    _require_gpu(A, B, bias, residual, norm_weight)
+    M, K = A.shape
+    N = B.shape[1]
+    fusable = (A.dtype == torch.bfloat16 and B.dtype == torch.bfloat16 and M > 0 and N % 8 == 0 and N <= 8192 and B.stride(0) == 1
+               and (residual is None or (residual.dtype == torch.bfloat16 and tuple(residual.shape) == (M, N)))
+               and (norm_weight is None or norm_weight.dtype == torch.bfloat16) and (bias is None or bias.dtype == torch.bfloat16)
+               and not torch.compiler.is_compiling())
+    if fusable:
+        a, lda = _rows16(A)
+        w, ldb_k, ldb_n = _weight_operand(B, M, True)
+        if ldb_k == 1:
+            L = _lib.lib()
+            b = None if bias is None else bias.contiguous()
+            nw = None if norm_weight is None else norm_weight.contiguous()
+            r2, ldr = (None, 0) if residual is None else _rows16(residual)
+            out = torch.empty((M, N), device=A.device, dtype=A.dtype)
+            rout = None if residual is None else torch.empty_like(out)
+            ws_bytes = L.tbik_gemm_workspace_bytes(M, N, K, leaf_k)
+            ws = torch.empty(ws_bytes, device=A.device, dtype=torch.uint8) if ws_bytes else None
+            rc = L.tbik_gemm_rmsnorm_bf16(a.data_ptr(), lda, w.data_ptr(), ldb_k, ldb_n, M, N, K, leaf_k,
+                                          None if b is None else b.data_ptr(), None if r2 is None else r2.data_ptr(), ldr,
+                                          None if nw is None else nw.data_ptr(), eps,
+                                          None if rout is None else rout.data_ptr(), 0 if rout is None else rout.stride(0),
+                                          out.data_ptr(), out.stride(0), None if ws is None else ws.data_ptr(), ws_bytes, _stream(A))
+            if rc == _lib.TBIK_OK:
+                return out, rout
+            if rc != _lib.TBIK_ERR_UNSUPPORTED:
+                _lib.check(rc, "tbik_gemm_rmsnorm_bf16")
+    return _norm_after(gemm_tree(A, B, bias, leaf_k), residual, norm_weight, eps)
+
+
+def tree_combine_add_rmsnorm(parts: List[torch.Tensor], bias: Optional[torch.Tensor], residual: Optional[torch.Tensor],
+                             norm_weight: Optional[torch.Tensor], eps: float):
+    """(rms_norm(tree_combine(parts) (+ bias) [+ residual]) * norm_weight, new residual or None) for 2-D partials: one
+    launch (`tbik_tree_combine_rmsnorm_bf16`) for bf16 rows of at most 8192 elements, the separate calls otherwise."""
+    _require_gpu(*parts, bias, residual, norm_weight)
+    p0 = parts[0]
+    n = len(parts)
+    fusable = (p0.dim() == 2 and n >= 2 and n <= 32 and (n & (n - 1)) == 0 and all(p.dtype == torch.bfloat16 and p.shape == p0.shape for p in parts)
+               and p0.shape[0] > 0 and p0.shape[1] % 8 == 0 and p0.shape[1] <= 8192
+               and (residual is None or (residual.dtype == torch.bfloat16 and residual.shape == p0.shape))
+               and (norm_weight is None or norm_weight.dtype == torch.bfloat16) and (bias is None or bias.dtype == torch.bfloat16)
+               and not torch.compiler.is_compiling())
+    if fusable:
+        ps = [p.contiguous() for p in parts]
+        if all(_aligned16(p) for p in ps):
+            M, N = p0.shape
+            arr = (ctypes.c_void_p * n)(*[p.data_ptr() for p in ps])
+            b = None if bias is None else bias.contiguous()
+            nw = None if norm_weight is None else norm_weight.contiguous()
+            r2, ldr = (None, 0) if residual is None else _rows16(residual)
+            out = torch.empty((M, N), device=p0.device, dtype=p0.dtype)
+            rout = None if residual is None else torch.empty_like(out)
+            rc = _lib.lib().tbik_tree_combine_rmsnorm_bf16(arr, n, M, N, None if b is None else b.data_ptr(),
+                                                           None if r2 is None else r2.data_ptr(), ldr,
+                                                           None if nw is None else nw.data_ptr(), eps,
+                                                           None if rout is None else rout.data_ptr(), 0 if rout is None else rout.stride(0),
+                                                           out.data_ptr(), out.stride(0), _stream(p0))
+            _lib.check(rc, "tbik_tree_combine_rmsnorm_bf16")
+            return out, rout
+    y = parts[0] if n == 1 else tree_combine(parts)
+    if bias is not None:
+        y = y + bias
+    return _norm_after(y, residual, norm_weight, eps)
+
+
+# --------------------------------------------------------------------------------------------
 # q/k norm + rotary embedding + KV-cache write in front of the attention
 # --------------------------------------------------------------------------------------------
 def bi_qk_norm_rope_cache_bf16(qkv: torch.Tensor, q_weight: torch.Tensor, k_weight: torch.Tensor, inv_freq: torch.Tensor,

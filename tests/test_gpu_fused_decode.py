@@ -1,6 +1,7 @@
 """One-launch compositions for decode-sized batches against the two-launch forms they stand for (bit for bit) and
 against the CPU oracle: RMSNorm inside the batch-invariant mm (`bi_rmsnorm_gemm_bf16`), SiLU * up inside the tree
-matmul of down_proj (`tbik_gemm_silu_mul_bf16`)."""
+matmul of down_proj (`tbik_gemm_silu_mul_bf16`), the add-RMSNorm behind a row-split layer inside the launch that combines
+the layer's K shards (`tbik_gemm_rmsnorm_bf16`, `tbik_tree_combine_rmsnorm_bf16`)."""
 import pytest
 import torch
 
@@ -136,9 +137,114 @@ def test_decoder_with_and_without_fused_producers_gives_the_same_bits(dev):
     prompts = [torch.randint(0, SMALL.vocab_size, (n,), generator=g).tolist() for n in (37, 5, 64, 21, 33, 16, 50, 48)]
     for tp in (1, 2, 8):
         fused = Qwen3Decoder(SMALL, tp_size=tp, seed=0, device=dev, fused_producers=True)
-        plain = Qwen3Decoder(SMALL, tp_size=tp, seed=0, device=dev, fused_producers=False)
+        plain = Qwen3Decoder(SMALL, tp_size=tp, seed=0, device=dev, fused_producers=False, fused_consumers=False)
         for batch in (1, 3, 4, 8):
             print("case decoder fused producers tp", tp, "batch", batch, flush=True)
+            a_ids, a_log = fused.generate(prompts[:batch], 6, return_logits=True)
+            b_ids, b_log = plain.generate(prompts[:batch], 6, return_logits=True)
+            assert torch.equal(a_ids, b_ids) and torch.equal(a_log, b_log), (tp, batch)
+        del fused, plain
+
+
+def _raw_gemm_rmsnorm(A, W, leaf, bias, res, w, eps, rout, out):
+    L = _lib.lib()
+    M, K = A.shape
+    N = W.shape[0]
+    ws_bytes = L.tbik_gemm_workspace_bytes(M, N, K, leaf)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=A.device)
+    p = lambda t: None if t is None else t.data_ptr()  # noqa: E731
+    return L.tbik_gemm_rmsnorm_bf16(A.data_ptr(), A.stride(0), W.data_ptr(), 1, W.stride(0), M, N, K, leaf, p(bias), p(res),
+                                    0 if res is None else res.stride(0), p(w), eps, p(rout), 0 if rout is None else rout.stride(0),
+                                    out.data_ptr(), out.stride(0), ws.data_ptr(), ws_bytes, torch.cuda.current_stream().cuda_stream)
+
+
+@pytest.mark.parametrize("M,K,N,leaf", [(5, 4096, 4096, 256), (32, 12288, 4096, 256), (128, 4096, 4096, 256), (77, 12288, 4096, 256),
+                                        (64, 8192, 5120, 256), (16, 6400, 5120, 128), (200, 4096, 1024, 256), (24, 4096, 8192, 256)])
+def test_add_rmsnorm_inside_the_shard_combine_of_the_tree_matmul_equals_the_two_calls(dev, M, K, N, leaf):
+    A = O.gaussian_bf16((M, K), 1.0, 40 + M).to(dev)
+    W = O.gaussian_bf16((N, K), 0.02, 41).to(dev)
+    res = O.gaussian_bf16((M, N), 1.0, 42 + M).to(dev)
+    w = (1.0 + 0.1 * torch.randn(N, generator=torch.Generator().manual_seed(5))).to(torch.bfloat16).to(dev)
+    bias = O.gaussian_bf16((N,), 0.5, 43).to(dev)
+    print("case tree matmul + add-rmsnorm", M, K, N, leaf, flush=True)
+    plan = (torch.zeros(5, dtype=torch.int32)).numpy()
+    import ctypes
+    assert _lib.lib().tbik_gemm_plan_info(M, N, K, leaf, 0, 0, plan.ctypes.data_as(ctypes.POINTER(ctypes.c_int))) == 0
+    assert plan[0] in (1, 3) and plan[1] > 1, plan          # a shape whose matmul ends in one shard combine
+    y = matmul_tp_persistent(A, W.t(), leaf_k=leaf)
+    for b in (None, bias):
+        yb = y if b is None else ops.gemm_tree(A, W.t(), b, leaf)
+        for r in (None, res):
+            for nw in (w, None):
+                want, want_res = bio.rms_norm(yb, nw, 1e-6, residual=r) if r is not None else (bio.rms_norm(yb, nw, 1e-6), None)
+                out = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+                rout = None if r is None else torch.empty_like(out)
+                assert _raw_gemm_rmsnorm(A, W, leaf, b, r, nw, 1e-6, rout, out) == _lib.TBIK_OK
+                assert torch.equal(out, want), (b is None, r is None, nw is None)
+                assert r is None or torch.equal(rout, want_res)
+                got, got_res = ops.gemm_tree_add_rmsnorm(A, W.t(), b, leaf, r, nw, 1e-6)
+                assert torch.equal(got, want) and (r is None or torch.equal(got_res, want_res))
+    # the new residual may be written over the old one
+    r2 = res.clone()
+    out = torch.empty((M, N), dtype=torch.bfloat16, device=dev)
+    assert _raw_gemm_rmsnorm(A, W, leaf, None, r2, w, 1e-6, r2, out) == _lib.TBIK_OK
+    want, want_res = bio.rms_norm(y, w, 1e-6, residual=res)
+    assert torch.equal(out, want) and torch.equal(r2, want_res)
+    # and the whole against the oracle's norm of the oracle-checked product (rounding points as documented: within 2 ulp)
+    ref, ref_res = O.rmsnorm(y.cpu(), w.cpu(), 1e-6, residual=res.cpu())
+    assert torch.equal(r2.cpu(), ref_res) and O.bf16_ulp_distance(out.cpu(), ref).max() <= 2
+
+
+def test_add_rmsnorm_behind_the_tree_matmul_falls_back_where_there_is_no_shard_combine(dev):
+    W = O.gaussian_bf16((4096, 4096), 0.02, 50).to(dev)
+    w = torch.ones(4096, dtype=torch.bfloat16, device=dev)
+    for M in (1, 4, 4096):                 # the one-launch few-rows kernel; a grid that needs no K split
+        A = O.gaussian_bf16((M, 4096), 1.0, 51).to(dev)
+        res = O.gaussian_bf16((M, 4096), 1.0, 52).to(dev)
+        out = torch.empty((M, 4096), dtype=torch.bfloat16, device=dev)
+        rout = torch.empty_like(out)
+        rc = _raw_gemm_rmsnorm(A, W, 256, None, res, w, 1e-6, rout, out)
+        want, want_res = bio.rms_norm(matmul_tp_persistent(A, W.t()), w, 1e-6, residual=res)
+        if rc != _lib.TBIK_OK:
+            assert rc == _lib.TBIK_ERR_UNSUPPORTED, (M, rc)
+        else:
+            assert torch.equal(out, want) and torch.equal(rout, want_res), M
+        got, got_res = ops.gemm_tree_add_rmsnorm(A, W.t(), None, 256, res, w, 1e-6)
+        assert torch.equal(got, want) and torch.equal(got_res, want_res), M
+    assert _raw_gemm_rmsnorm(O.gaussian_bf16((1, 4096), 1.0, 53).to(dev), W, 256, None, None, w, 1e-6, None,
+                             torch.empty((1, 4096), dtype=torch.bfloat16, device=dev)) == _lib.TBIK_ERR_UNSUPPORTED
+
+
+@pytest.mark.parametrize("rows,hidden,nparts", [(1, 4096, 2), (33, 4096, 8), (7, 1024, 4), (5, 8192, 2), (130, 1000, 4), (3, 5120, 32)])
+def test_add_rmsnorm_inside_the_shard_combine_equals_the_separate_calls(dev, rows, hidden, nparts):
+    parts = [O.gaussian_bf16((rows, hidden), 1.0, 60 + i).to(dev) for i in range(nparts)]
+    res = O.gaussian_bf16((rows, hidden), 1.0, 59).to(dev)
+    w = (1.0 + 0.1 * torch.randn(hidden, generator=torch.Generator().manual_seed(6))).to(torch.bfloat16).to(dev)
+    bias = O.gaussian_bf16((hidden,), 0.5, 58).to(dev)
+    print("case shard combine + add-rmsnorm", rows, hidden, nparts, flush=True)
+    y = ops.tree_combine(parts)
+    assert torch.equal(y.cpu(), O.tree_combine([p.cpu() for p in parts]))
+    for b in (None, bias):
+        yb = y if b is None else y + b
+        for r in (None, res):
+            want, want_res = bio.rms_norm(yb, w, 1e-6, residual=r) if r is not None else (bio.rms_norm(yb, w, 1e-6), None)
+            got, got_res = ops.tree_combine_add_rmsnorm(parts, b, r, w, 1e-6)
+            assert torch.equal(got, want), (b is None, r is None)
+            assert r is None or torch.equal(got_res, want_res)
+    # what the one-launch kernel does not take goes through the separate calls (fp16 partials here)
+    half = [O.gaussian_bf16((2, 512), 1.0, 70 + i).to(torch.float16).to(dev) for i in range(2)]
+    g, _ = ops.tree_combine_add_rmsnorm(half, None, None, None, 1e-6)
+    assert torch.equal(g, bio.rms_norm(ops.tree_combine(half), None, 1e-6))
+
+
+def test_decoder_with_and_without_fused_consumers_gives_the_same_bits(dev):
+    g = torch.Generator().manual_seed(4)
+    prompts = [torch.randint(0, SMALL.vocab_size, (n,), generator=g).tolist() for n in (37, 5, 64, 21, 33, 16, 50, 48, 9, 12)]
+    for tp in (1, 2, 4):
+        fused = Qwen3Decoder(SMALL, tp_size=tp, seed=0, device=dev, fused_consumers=True)
+        plain = Qwen3Decoder(SMALL, tp_size=tp, seed=0, device=dev, fused_consumers=False)
+        for batch in (1, 5, 10):
+            print("case decoder fused consumers tp", tp, "batch", batch, flush=True)
             a_ids, a_log = fused.generate(prompts[:batch], 6, return_logits=True)
             b_ids, b_log = plain.generate(prompts[:batch], 6, return_logits=True)
             assert torch.equal(a_ids, b_ids) and torch.equal(a_log, b_log), (tp, batch)
