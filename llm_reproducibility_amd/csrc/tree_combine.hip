@@ -153,9 +153,9 @@ int tree_combine_bias_dispatch(const void* const* parts, int nparts, void* out, 
 }
 
 // ------------------------------------------------------------------------------------------------
-// Shard combine followed by the (add-)RMSNorm of the combined rows, in one launch: one wavefront per row forms the
-// row's packs exactly as combine_vec_kernel does (tree over the partials, then the bias) and hands them, still in
-// registers, to the row function of the stand-alone RMSNorm (rmsnorm_row.h) in the lane layout that function expects.
+// Shard combine followed by the (add-)RMSNorm of the combined rows, in one launch: the row's packs are formed exactly
+// as combine_vec_kernel forms them (tree over the partials, then the bias) and handed, without a trip through memory,
+// to the row function of the stand-alone RMSNorm (rmsnorm_row.h) in the lane layout that function expects.
 // Same bits as the two launches; a decode-sized batch saves a kernel per row-split layer.
 // ------------------------------------------------------------------------------------------------
 struct CombineNormArgs {
@@ -172,51 +172,58 @@ struct CombineNormArgs {
   float eps;
 };
 
+// One work-group per row, CPL wavefronts: wave w forms the chunks lane + 64 w of the row (all its partial loads in
+// flight at once) and leaves them in LDS; wave 0, which asked for the residual and the weights first, then takes the
+// whole row in the lane layout of the row function (lane l: chunks l, l + 64, ...) and finishes it.
 template <int NP, int CPL, bool F16>
-__global__ __launch_bounds__(256) void combine_rmsnorm_kernel(const CombineNormArgs a) {
+__global__ __launch_bounds__(64 * CPL) void combine_rmsnorm_kernel(const CombineNormArgs a) {
+  __shared__ uint4 xs[64 * CPL];
   const int lane = threadIdx.x & 63;
-  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (row >= a.rows) return;
+  const int wave = threadIdx.x >> 6;
+  const int64_t row = blockIdx.x;
   const int nchunks = a.hidden >> 3;
   RmsnormRow<CPL, F16> r;
   r.has_res = a.res != nullptr;
   r.has_w = a.w != nullptr;
-  const uint4* wr = reinterpret_cast<const uint4*>(a.w);
-  const uint4* rr = a.res ? reinterpret_cast<const uint4*>(a.res + row * a.ldr) : nullptr;
-  const uint4* br = reinterpret_cast<const uint4*>(a.bias);
-  // every load of the row goes out before the first store (the residual output may alias the residual)
-#pragma unroll
-  for (int i = 0; i < CPL; i++) {
-    const int c = lane + 64 * i;
-    if (c < nchunks) {
-      if (wr) r.wq[i] = wr[c];
-      if (rr) r.rq[i] = rr[c];
-      uint4 in[NP];
-#pragma unroll
-      for (int p = 0; p < NP; p++) in[p] = reinterpret_cast<const uint4*>(a.parts[p] + row * a.hidden)[c];
-      uint4 o = combine_pack<NP, F16>(in);
-      if (br) o = add_pack<F16>(o, br[c]);
-      r.xq[i] = o;
-    }
-  }
-  if (a.sum_out) {
-    uint4* srow = reinterpret_cast<uint4*>(a.sum_out + row * a.lds);
+  if (wave == 0) {
+    const uint4* wr = reinterpret_cast<const uint4*>(a.w);
+    const uint4* rr = a.res ? reinterpret_cast<const uint4*>(a.res + row * a.ldr) : nullptr;
 #pragma unroll
     for (int i = 0; i < CPL; i++) {
       const int c = lane + 64 * i;
-      if (c < nchunks) srow[c] = r.xq[i];
+      if (c < nchunks) {
+        if (wr) r.wq[i] = wr[c];
+        if (rr) r.rq[i] = rr[c];
+      }
     }
   }
+  const int c = lane + 64 * wave;
+  if (c < nchunks) {
+    uint4 in[NP];
+#pragma unroll
+    for (int p = 0; p < NP; p++) in[p] = reinterpret_cast<const uint4*>(a.parts[p] + row * a.hidden)[c];
+    uint4 o = combine_pack<NP, F16>(in);
+    if (a.bias) o = add_pack<F16>(o, reinterpret_cast<const uint4*>(a.bias)[c]);
+    if (a.sum_out) reinterpret_cast<uint4*>(a.sum_out + row * a.lds)[c] = o;
+    xs[c] = o;
+  }
+  __syncthreads();
+  if (wave != 0) return;
+#pragma unroll
+  for (int i = 0; i < CPL; i++) {
+    const int ci = lane + 64 * i;
+    if (ci < nchunks) r.xq[i] = xs[ci];
+  }
   uint4* orow = reinterpret_cast<uint4*>(a.out + row * a.ldo);
-  r.finish(a.res_out ? a.res_out + row * a.ldro : nullptr, a.hidden, a.eps, lane, [&](int c, const uint4& o) { orow[c] = o; });
+  r.finish(a.res_out ? a.res_out + row * a.ldro : nullptr, a.hidden, a.eps, lane, [&](int cc, const uint4& o) { orow[cc] = o; });
 }
 
 template <int NP, bool F16>
 static void launch_combine_rmsnorm(const CombineNormArgs& a, dim3 grid, hipStream_t stream) {
   const int cpl = (a.hidden + 511) / 512;  // a function of the row length only
-  if (cpl <= 2) hipLaunchKernelGGL((combine_rmsnorm_kernel<NP, 2, F16>), grid, dim3(256), 0, stream, a);
-  else if (cpl <= 8) hipLaunchKernelGGL((combine_rmsnorm_kernel<NP, 8, F16>), grid, dim3(256), 0, stream, a);
-  else hipLaunchKernelGGL((combine_rmsnorm_kernel<NP, 16, F16>), grid, dim3(256), 0, stream, a);
+  if (cpl <= 2) hipLaunchKernelGGL((combine_rmsnorm_kernel<NP, 2, F16>), grid, dim3(128), 0, stream, a);
+  else if (cpl <= 8) hipLaunchKernelGGL((combine_rmsnorm_kernel<NP, 8, F16>), grid, dim3(512), 0, stream, a);
+  else hipLaunchKernelGGL((combine_rmsnorm_kernel<NP, 16, F16>), grid, dim3(1024), 0, stream, a);
 }
 
 int tree_combine_rmsnorm_dispatch(const void* const* parts, int nparts, int64_t rows, int hidden, const void* bias,
@@ -253,9 +260,8 @@ int tree_combine_rmsnorm_dispatch(const void* const* parts, int nparts, int64_t 
   a.rows = rows;
   a.hidden = hidden;
   a.eps = eps;
-  const int64_t blocks = (rows + 3) / 4;
-  if (blocks > 0x7fffffff) return TBIK_ERR_INVALID;
-  const dim3 grid((unsigned)blocks);
+  if (rows > 0x7fffffff) return TBIK_ERR_INVALID;
+  const dim3 grid((unsigned)rows);
   if (f16) {
     switch (nparts) {
       case 2: launch_combine_rmsnorm<2, true>(a, grid, stream); break;

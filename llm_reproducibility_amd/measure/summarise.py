@@ -106,6 +106,7 @@ _KINDS = [("gemm_single_acc_stream", "batch-invariant mm (streaming kernels; RMS
           ("gemm_tree_strip", "tree GEMM o_proj / down_proj (one-launch kernel; SiLU*up inside where fused)"),
           ("gemm_tree", "tree GEMM o_proj / down_proj (tile kernels)"),
           ("gemm_kernel<", "mm / tree GEMM (small-tile kernel)"),
+          ("combine_rmsnorm", "shard combine of the K-cut tree GEMM with the add-RMSNorm of the result"),
           ("combine_", "shard combine of the K-cut tree GEMM"),
           ("attention", "attention"), ("rmsnorm", "RMSNorm (+ residual add)"), ("argmax", "token choice (arg-max kernel)"),
           ("silu_mul", "silu_mul"), ("qk_norm_rope", "q/k norm + rotary + cache write")]
