@@ -347,6 +347,8 @@ def table(steps, warmup, hot=False, settle_ms=20.0, full=False, only=None):
             lambda x, r, W: bio.matmul_persistent(bio.rms_norm(x, w, 1e-6, residual=r)[0], W.t()), 2.0 * M * 24576 * 4096, by, "hbm",
             short=f"norm, mm gate_up M={M}")
 
+        M = min(M, 3)   # 4 rows of 12288 activations are past what the one-launch kernel forms in every work-group
+
         def make_gated(M=M):
             return (torch.randn((M, 2 * 12288), device=dev).to(torch.bfloat16), (torch.randn((4096, 12288), device=dev) * 0.02).to(torch.bfloat16))
         by = 2.0 * 4096 * 12288
@@ -356,6 +358,19 @@ def table(steps, warmup, hot=False, settle_ms=20.0, full=False, only=None):
         add(f"  the same as two launches (silu_mul, then tree matmul) M={M}", make_gated,
             lambda gu, W: matmul_tp_persistent(ops.bi_silu_mul(gu), W.t()), 2.0 * M * 4096 * 12288, by, "hbm",
             short=f"silu, tree dn8B M={M}")
+    # from five rows on the consumer runs inside the producer: the add-RMSNorm behind a row-split layer in the launch that
+    # combines the layer's K shards, against the matmul followed by the norm (same bits)
+    for M in (32, 128):
+        def make_tn(M=M):
+            return (torch.randn((M, 12288), device=dev).to(torch.bfloat16), torch.randn((M, 4096), device=dev).to(torch.bfloat16),
+                    (torch.randn((4096, 12288), device=dev) * 0.02).to(torch.bfloat16))
+        by = 2.0 * 4096 * 12288
+        add(f"add-RMSNorm inside the shard combine of the tree matmul, down_proj 8B M={M}", make_tn,
+            lambda x, r, W: ops.gemm_tree_add_rmsnorm(x, W.t(), None, 256, r, w, 1e-6), 2.0 * M * 4096 * 12288, by, "hbm",
+            short=f"tree+norm dn8B M={M}")
+        add(f"  the same as separate calls (tree matmul, then add-RMSNorm) M={M}", make_tn,
+            lambda x, r, W: bio.rms_norm(matmul_tp_persistent(x, W.t()), w, 1e-6, residual=r), 2.0 * M * 4096 * 12288, by, "hbm",
+            short=f"tree, norm dn8B M={M}")
     # fixed-order attention (Qwen3-8B heads: 32 query, 8 key/value, head_dim 128)
     Hq, Hkv, D = 32, 8, 128
 

@@ -449,6 +449,11 @@ def _(gate_up):
 # --------------------------------------------------------------------------------------------
 # one-launch compositions for decode-sized batches (bit-identical to the two-launch forms they fall back to)
 # --------------------------------------------------------------------------------------------
+# Shapes for which a one-launch entry point answered 'unsupported': whether it applies depends on the shape alone, so the
+# next call of the same shape goes to the separate calls at once (no output allocated for a call that will not run).
+_declined: set = set()
+
+
 def rmsnorm_gemm(x: torch.Tensor, norm_weight: Optional[torch.Tensor], eps: float, residual: Optional[torch.Tensor],
                  B: torch.Tensor, bias: Optional[torch.Tensor] = None):
     """(bi_gemm(rms_norm(x [+ residual]) * norm_weight, B) (+ bias), new residual or None).
@@ -459,7 +464,7 @@ def rmsnorm_gemm(x: torch.Tensor, norm_weight: Optional[torch.Tensor], eps: floa
     M, K = x.shape
     N = B.shape[1]
     fusable = (x.dtype == torch.bfloat16 and B.dtype == torch.bfloat16 and M * K <= 32768 and K <= 8192 and K % 32 == 0
-               and B.stride(0) == 1 and not torch.compiler.is_compiling())
+               and B.stride(0) == 1 and not torch.compiler.is_compiling() and ("norm_mm", M, N, K) not in _declined)
     if fusable:
         x2, ldx = _rows16(x)
         r2, ldr = (None, 0) if residual is None else _rows16(residual)
@@ -476,6 +481,7 @@ def rmsnorm_gemm(x: torch.Tensor, norm_weight: Optional[torch.Tensor], eps: floa
             return C, rout
         if rc != _lib.TBIK_ERR_UNSUPPORTED:
             _lib.check(rc, "bi_rmsnorm_gemm_bf16")
+        _declined.add(("norm_mm", M, N, K))
     if residual is None:
         h, rout = bi_rmsnorm(x, norm_weight, eps), None
     else:
@@ -494,7 +500,8 @@ def gemm_tree_silu_mul(gate: torch.Tensor, up: torch.Tensor, B: torch.Tensor, bi
     N = B.shape[1]
     fusable = (gate.dtype == torch.bfloat16 and B.dtype == torch.bfloat16 and M <= 4 and up.shape == gate.shape
                and gate.stride(1) == 1 and up.stride(1) == 1 and gate.stride(0) == up.stride(0) and gate.stride(0) % 8 == 0
-               and _aligned16(gate) and _aligned16(up) and B.stride(0) == 1 and not torch.compiler.is_compiling())
+               and _aligned16(gate) and _aligned16(up) and B.stride(0) == 1 and not torch.compiler.is_compiling()
+               and ("silu_tree", M, N, K, leaf_k) not in _declined)
     if fusable:
         w, ldb_k, ldb_n = _weight_operand(B)
         b = None if bias is None else bias.contiguous()
@@ -506,6 +513,7 @@ def gemm_tree_silu_mul(gate: torch.Tensor, up: torch.Tensor, B: torch.Tensor, bi
             return C
         if rc != _lib.TBIK_ERR_UNSUPPORTED:
             _lib.check(rc, "tbik_gemm_silu_mul_bf16")
+        _declined.add(("silu_tree", M, N, K, leaf_k))
     if (gate.dim() == 2 and up.shape == gate.shape and gate.stride(1) == 1 and up.stride(1) == 1 and gate.stride(0) == up.stride(0)
             and gate.dtype == up.dtype and up.data_ptr() == gate.data_ptr() + K * gate.element_size()
             and (M == 1 or gate.stride(0) >= 2 * K)):
@@ -540,7 +548,7 @@ def gemm_tree_add_rmsnorm(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch
     fusable = (A.dtype == torch.bfloat16 and B.dtype == torch.bfloat16 and M > 0 and N % 8 == 0 and N <= 8192 and B.stride(0) == 1
                and (residual is None or (residual.dtype == torch.bfloat16 and tuple(residual.shape) == (M, N)))
                and (norm_weight is None or norm_weight.dtype == torch.bfloat16) and (bias is None or bias.dtype == torch.bfloat16)
-               and not torch.compiler.is_compiling())
+               and not torch.compiler.is_compiling() and ("tree_norm", M, N, K, leaf_k) not in _declined)
     if fusable:
         a, lda = _rows16(A)
         w, ldb_k, ldb_n = _weight_operand(B, M, True)
@@ -562,6 +570,7 @@ def gemm_tree_add_rmsnorm(A: torch.Tensor, B: torch.Tensor, bias: Optional[torch
                 return out, rout
             if rc != _lib.TBIK_ERR_UNSUPPORTED:
                 _lib.check(rc, "tbik_gemm_rmsnorm_bf16")
+            _declined.add(("tree_norm", M, N, K, leaf_k))
     return _norm_after(gemm_tree(A, B, bias, leaf_k), residual, norm_weight, eps)
 
 
