@@ -5,7 +5,7 @@
 //   attention_group_kernel  the G query heads of a KV head as the G wavefronts of a work-group, K/V tiles staged in LDS
 //                           once for all of them (prefill and chunked prefill);
 //   attention_decode_kernel the few new queries of a sequence times the G heads as the 16 rows of ONE tile, the output
-//                           channels split over four wavefronts (decode).
+//                           channels split over four wavefronts, four more wavefronts bringing the tiles in (decode).
 //
 // Counterpart of the reference's fixed-tile attention for train/inference alignment
 // (_kernel_unified_attention_2d, src/patch/patch_training_inference_align.py:171-487: one pass over the
@@ -22,6 +22,7 @@
 // [batch, kv_heads, 128, max_len] so that the P*V MFMA operand (8 consecutive keys of one channel) is a
 // contiguous load.  Cache entries behind ctx_len must be finite (they are multiplied by an exact 0).
 #include "common.h"
+#include "lds_direct.h"
 
 namespace tbik {
 
@@ -351,76 +352,129 @@ __global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs 
 
 // ------------------------------------------------------------------------------------------------
 // Decode variant: every sequence brings so few new queries that all of them, for all G query heads of a KV head, fit
-// the 16 rows of one MFMA tile (row = query * G + head of the group).  One work-group per (KV head, sequence).  Its four
-// wavefronts all compute the scores and the softmax of the whole tile (the same instructions on the same values, so
-// the same bits in each) and each keeps the output accumulators of two of the eight 16-channel tiles: per key tile a
-// wave issues 8 + 2 MFMAs where a wave of the grouped kernel issues 16.  The scores of tile t + 1 are formed before the
-// softmax of tile t, so the MFMA chain of one tile runs beside the exponentials of the other.  A decode step is one
-// dependent chain of key tiles per sequence, and its length per tile is what the kernel's time consists of.
+// the 16 rows of one MFMA tile (row = query * G + head of the group).  One work-group of eight wavefronts per
+// (KV head, sequence):
+//   * waves 0-3 compute.  All four form the scores and the softmax of the whole tile (the same instructions on the same
+//     values, so the same bits in each) and each keeps the output accumulators of two of the eight 16-channel tiles: per
+//     key tile a wave issues 8 + 2 MFMAs where a wave of the grouped kernel issues 16.  The scores of tile t + 1 are formed
+//     before the softmax of tile t, so the MFMA chain of one tile runs beside the exponentials of the other.
+//   * waves 4-7 do nothing but bring tiles in, with direct global->LDS loads (no staging registers, no LDS writes by a
+//     wave): a decode step is one dependent chain of key tiles per sequence, and every load a computing wave issues is a
+//     piece of that chain.  Loader i issues two of the eight 1 KiB load instructions of every K tile and V^T tile.
+// A direct load puts lane l's 16 bytes at (wave-uniform address) + 16 l, so the LDS layout is made on the global side:
+// each lane fetches the chunk that belongs at its fixed place.
+//   K tile [32 keys][256 bytes]: chunk position pc of key row kr holds chunk pc ^ 2 (kr & 7) (the swizzle of the grouped
+//     kernel, read the same way);
+//   V^T tile [128 channels][64 bytes = 32 keys]: chunk position pc of channel row r holds chunk pc ^ ((r >> 2) & 3); a
+//     P*V fragment (keys 4g .. 4g+3 and 16+4g .. 16+4g+3 of channel row 16t + j) is two 8-byte reads, and the sixteen
+//     rows x two lane groups of a read pass cover all 64 banks.
+// K tiles and V^T tiles have rings of NS slots each.  Iteration t reads K tile t + 1 and V^T tile t; the loaders request
+// K tile t + NS (slot t % NS, read during iteration t - 1) and V^T tile t + NS - 1 (slot (t - 1) % NS, likewise), wait
+// until what they requested NS - 2 iterations ago has landed (K tile t + 2, V^T tile t + 1: what iteration t + 1 reads),
+// and all eight waves meet at the barrier.  Tiles behind the last one are clamped to the last tile of the cache and
+// never used, so the number of loads in flight is static; nothing is in flight when a wave ends.
 // A row's arithmetic -- the lanes that own it, the MFMA chains over channels and key slots, the order of the softmax
 // updates -- is that of the kernels above: the same bits.
-// K tiles and V^T tiles have rings of their own (two slots each), because the K tile is needed one iteration earlier.
 // ------------------------------------------------------------------------------------------------
 template <int G>
-__global__ __launch_bounds__(256) void attention_decode_kernel(const AttnArgs a) {
-  __shared__ __attribute__((aligned(16))) uint8_t lds_k[2][8192];  // K tile [32][128], rows XOR-swizzled as above
-  __shared__ __attribute__((aligned(16))) uint8_t lds_v[2][8192];  // V^T tile [128][32] in fragment order as above
-  constexpr int QMAX = 16 / G;  // queries of a sequence that fit the tile
+__global__ __launch_bounds__(512) void attention_decode_kernel(const AttnArgs a) {
+  constexpr int NS = 4;               // ring slots per operand (2 x 4 x 8 KiB of LDS)
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds_dyn[];
+  uint8_t (*lds_k)[8192] = reinterpret_cast<uint8_t (*)[8192]>(lds_dyn);
+  uint8_t (*lds_v)[8192] = reinterpret_cast<uint8_t (*)[8192]>(lds_dyn + NS * 8192);
+  constexpr int QMAX = 16 / G;
+  constexpr int CT = 2;
+  constexpr int NL = 4;               // loader waves
+  constexpr int PI = 8 / NL;          // load instructions per tile, operand and loader wave
   const int b = blockIdx.y;
   const int kvh = blockIdx.x;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wv = tid >> 6;
+  const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int j = lane & 15;
   const int g = lane >> 4;
   const uint8_t* kbase = reinterpret_cast<const uint8_t*>(a.k_cache + ((int64_t)b * a.kv_heads + kvh) * a.max_len * HD);
   const uint8_t* vbase = reinterpret_cast<const uint8_t*>(a.vt_cache + ((int64_t)b * a.kv_heads + kvh) * (int64_t)HD * a.max_len);
-
-  // staging as in the grouped kernel: 512 16-byte chunks per tile and operand, two per thread, fetched four tiles ahead
-  // into four register sets (set = tile % 4)
-  constexpr int NT = 256, NCH = 2, DEPTH = 4;
-  constexpr int CT = 2;  // 16-channel tiles of the output per wave
-  u32x4 kregs[DEPTH][NCH], vregs[DEPTH][NCH];
-  uint32_t vsrc[NCH], kdst[NCH], vdst0[NCH], vdst1[NCH];
+  if (wv >= 4) {
+    // ---------------- loader waves: loader li issues instructions li*PI .. li*PI+PI-1 of every K tile and V^T tile
+    const int li = wv - 4;
+    // K: instruction q covers key rows 4q .. 4q+3 (1 KiB): lane -> row 4q + (lane >> 4), chunk position lane & 15
+    // V^T: instruction q covers channel rows 16q .. 16q+15: lane -> row 16q + (lane >> 2), chunk position lane & 3
+    uint32_t kvoff[PI], vvoff[PI];
 #pragma unroll
-  for (int i = 0; i < NCH; i++) {
-    const int ch = tid + i * NT;
-    const int kr = ch >> 4, kc = ch & 15;
-    kdst[i] = kr * 256 + ((kc ^ (2 * (kr & 7))) << 4);
-    const int vr = ch >> 2, vc = ch & 3;
-    const int vx = 4 * ((vr >> 2) & 1);
-    vsrc[i] = (uint32_t)vr * (uint32_t)a.max_len * 2u + vc * 16;
-    vdst0[i] = vr * 64 + ((2 * ((2 * vc) & 3) + (vc >> 1)) ^ vx) * 8;
-    vdst1[i] = vr * 64 + ((2 * ((2 * vc + 1) & 3) + (vc >> 1)) ^ vx) * 8;
+    for (int i = 0; i < PI; i++) {
+      const int q = li * PI + i;
+      const int kr = 4 * q + (lane >> 4), pc = lane & 15;
+      const int r = 16 * q + (lane >> 2), vc = (lane & 3) ^ ((lane >> 4) & 3);
+      kvoff[i] = (uint32_t)(kr * 256 + ((pc ^ (2 * (kr & 7))) << 4));
+      vvoff[i] = (uint32_t)r * (uint32_t)a.max_len * 2u + vc * 16;
+    }
+    const uint32_t lk = (uint32_t)(uintptr_t)&lds_k[0][0] + li * PI * 1024;
+    const uint32_t lv = (uint32_t)(uintptr_t)&lds_v[0][0] + li * PI * 1024;
+    auto load_k = [&](int tile, int slot) __attribute__((always_inline)) {
+      const uint8_t* src = kbase + (int64_t)min(tile * 32, a.max_len - 32) * (HD * 2);
+#pragma unroll
+      for (int i = 0; i < PI; i++) dma16(lk + slot * 8192 + i * 1024, kvoff[i], src);
+    };
+    auto load_v = [&](int tile, int slot) __attribute__((always_inline)) {
+      const uint8_t* src = vbase + (int64_t)min(tile * 32, a.max_len - 32) * 2;
+#pragma unroll
+      for (int i = 0; i < PI; i++) dma16(lv + slot * 8192 + i * 1024, vvoff[i], src);
+    };
+    load_k(0, 0);
+#pragma unroll
+    for (int i = 0; i < NS - 1; i++) {
+      load_k(i + 1, i + 1);
+      load_v(i, i);
+    }
+    const int qlen = a.q_len[b];
+    if (qlen <= 0) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      return;
+    }
+    const int ctx = a.ctx_len[b];
+    const int last_pos = ctx - qlen + min(QMAX - 1, qlen - 1);
+    const int ntiles = last_pos / 32 + 1;
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * PI * (NS - 1)) : "memory");  // K tile 0
+    __syncthreads();
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * PI * (NS - 2)) : "memory");  // K tile 1, V^T tile 0
+    __syncthreads();
+    for (int t0 = 0; t0 < ntiles; t0 += NS) {
+#pragma unroll
+      for (int d = 0; d < NS; d++) {
+        const int tile = t0 + d;
+        if (tile >= ntiles) break;
+        load_k(tile + NS, d);                          // slot t % NS, read during iteration t - 1
+        load_v(tile + NS - 1, (d + NS - 1) % NS);      // slot (t - 1) % NS, likewise
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * PI * (NS - 2)) : "memory");  // K tile t + 2, V^T tile t + 1
+        __syncthreads();
+      }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    return;
   }
-  const __amdgpu_buffer_rsrc_t krsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(kbase), 0, a.max_len * (HD * 2), 0x00020000);
-  const __amdgpu_buffer_rsrc_t vrsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(vbase), 0, a.max_len * (HD * 2), 0x00020000);
-  auto load_tile = [&](int tile, int set) __attribute__((always_inline)) {
-    const int k0 = min(tile * 32, a.max_len - 32);  // max_len is a multiple of 32: never past the cache
-    const int ks = k0 * (HD * 2), vs = k0 * 2;
+  // ---------------- computing waves
+  const int qlen = a.q_len[b];
+  if (qlen <= 0) return;
+  const int qi = j / G;
+  const int h = kvh * G + j % G;
+  const int ctx = a.ctx_len[b];
+  const bool qvalid = qi < qlen;
+  const int qrow = min(qi, qlen - 1);
+  const int qpos = ctx - qlen + qrow;
+  const int last_pos = ctx - qlen + min(QMAX - 1, qlen - 1);
+  const int ntiles = last_pos / 32 + 1;
+  const int nfull = (ctx - qlen + 1) / 32;
+  const uint16_t* qp = a.q + ((int64_t)(a.q_start[b] + qrow) * a.q_heads + h) * HD;
+  bf16x8 qf[4];
 #pragma unroll
-    for (int i = 0; i < NCH; i++) {
-      kregs[set][i] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, (tid + i * NT) * 16, ks, 0);
-      vregs[set][i] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, (int)vsrc[i], vs, 0);
-    }
-  };
-  auto store_k = [&](int slot, int set) __attribute__((always_inline)) {
-#pragma unroll
-    for (int i = 0; i < NCH; i++) *reinterpret_cast<u32x4*>(&lds_k[slot][kdst[i]]) = kregs[set][i];
-  };
-  auto store_v = [&](int slot, int set) __attribute__((always_inline)) {
-#pragma unroll
-    for (int i = 0; i < NCH; i++) {
-      *reinterpret_cast<uint2*>(&lds_v[slot][vdst0[i]]) = make_uint2(vregs[set][i][0], vregs[set][i][1]);
-      *reinterpret_cast<uint2*>(&lds_v[slot][vdst1[i]]) = make_uint2(vregs[set][i][2], vregs[set][i][3]);
-    }
-  };
-
-  bf16x8 qf[4];  // Q as the MFMA "B" operand: lane (j, g) holds channels 32c + 8g .. +7 of row j
+  for (int c = 0; c < 4; c++) qf[c] = *reinterpret_cast<const bf16x8*>(qp + c * 32 + g * 8);
   uint32_t kofs[4];
 #pragma unroll
   for (int c = 0; c < 4; c++) kofs[c] = j * 256 + (((c * 4 + g) ^ (2 * (j & 7))) << 4);
-  const uint32_t vofs = (CT * wv) * 1024 + j * 64 + (g ^ (2 * ((j >> 2) & 1))) * 16;
+  const int vsw = (j >> 2) & 3;
+  const uint32_t vofs0 = (CT * wv) * 1024 + j * 64 + (((g >> 1) ^ vsw) << 4) + (g & 1) * 8;
+  const uint32_t vofs1 = (CT * wv) * 1024 + j * 64 + (((2 + (g >> 1)) ^ vsw) << 4) + (g & 1) * 8;
   auto scores = [&](int slot, f32x4 (&s)[2]) __attribute__((always_inline)) {
     const uint8_t* tb = &lds_k[slot][0];
 #pragma unroll
@@ -435,72 +489,37 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(const AttnArgs a)
       s[u] = acc;
     }
   };
-
-  f32x4 o[CT];  // channel tiles CT wv .. CT wv + CT - 1
+  f32x4 o[CT];
 #pragma unroll
   for (int i = 0; i < CT; i++) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY;
   float l = 0.f;
-
-  // The first key tiles are requested before anything is known about the sequence: their addresses depend on the
-  // work-group only, and loads past the last tile are clamped to a valid address and never used (a static number of
-  // loads in flight).  The lengths and the queries arrive while those loads are on their way.
-#pragma unroll
-  for (int d = 0; d < DEPTH; d++) load_tile(d, d);
-  const int qlen = a.q_len[b];
-  if (qlen <= 0) return;  // uniform over the work-group
-  const int qi = j / G;                 // query of the sequence
-  const int h = kvh * G + j % G;        // query head
-  const int ctx = a.ctx_len[b];
-  const bool qvalid = qi < qlen;
-  const int qrow = min(qi, qlen - 1);
-  const int qpos = ctx - qlen + qrow;
-  const int last_pos = ctx - qlen + min(QMAX - 1, qlen - 1);
-  const int ntiles = last_pos / 32 + 1;
-  const int nfull = (ctx - qlen + 1) / 32;  // tiles whose keys are visible to every query: no mask needed
-  const uint16_t* qp = a.q + ((int64_t)(a.q_start[b] + qrow) * a.q_heads + h) * HD;
-#pragma unroll
-  for (int c = 0; c < 4; c++) qf[c] = *reinterpret_cast<const bf16x8*>(qp + c * 32 + g * 8);
-  store_k(0, 0);
   __syncthreads();
   f32x4 s_cur[2];
   scores(0, s_cur);
-  store_k(1, 1);
-  store_v(0, 0);
-  __syncthreads();  // also: every wave has read K tile 0 before slot 0 is written again
-  // Iteration t: K tile t + 1 is in K slot (t + 1) & 1 and V^T tile t in V slot t & 1; it writes K tile t + 2 into K slot
-  // t & 1 (read during iteration t - 1) and V^T tile t + 1 into V slot (t + 1) & 1 (likewise), then meets the barrier.
-  // Register set t % 4 is free at the top of iteration t: its K tile went to LDS two iterations ago, its V^T tile one.
-  // The body covers four tiles, so that slots and sets are compile-time constants.
-  for (int t0 = 0; t0 < ntiles; t0 += DEPTH) {
+  __syncthreads();
+  for (int t0 = 0; t0 < ntiles; t0 += NS) {
 #pragma unroll
-    for (int d = 0; d < DEPTH; d++) {
+    for (int d = 0; d < NS; d++) {
       const int tile = t0 + d;
       if (tile >= ntiles) break;
-      load_tile(tile + DEPTH, d);
-      // the V^T fragments are requested first: they have been in LDS since the barrier, and their latency passes
-      // during the scores and the softmax
       bf16x8 vf[CT];
 #pragma unroll
-      for (int i = 0; i < CT; i++) vf[i] = *reinterpret_cast<const bf16x8*>(&lds_v[d & 1][vofs + i * 1024]);
-      // behind the last tile the slot holds an older tile: the scores are formed (no branch inside the chain) and unused
+      for (int i = 0; i < CT; i++) {
+        const uint2 va = *reinterpret_cast<const uint2*>(&lds_v[d][vofs0 + i * 1024]);
+        const uint2 vb = *reinterpret_cast<const uint2*>(&lds_v[d][vofs1 + i * 1024]);
+        vf[i] = __builtin_bit_cast(bf16x8, u32x4{va.x, va.y, vb.x, vb.y});
+      }
       f32x4 s_next[2];
-      scores((d + 1) & 1, s_next);
+      scores((d + 1) % NS, s_next);
       float alpha;
       bf16x8 pf;
-      // the mask is needed only where a tile reaches beyond some query's horizon (a scalar condition known long before;
-      // the values are the same either way)
       if (tile < nfull) softmax_tile<false>(s_cur, tile * 32, g, qpos, a.scale_log2, m, l, alpha, pf);
       else softmax_tile<true>(s_cur, tile * 32, g, qpos, a.scale_log2, m, l, alpha, pf);
-      // (always rescaled: a branch on the freshly computed factor costs more than the few multiplications)
-      {
 #pragma unroll
-        for (int i = 0; i < CT; i++) o[i] = f32x4{o[i][0] * alpha, o[i][1] * alpha, o[i][2] * alpha, o[i][3] * alpha};
-      }
+      for (int i = 0; i < CT; i++) o[i] = f32x4{o[i][0] * alpha, o[i][1] * alpha, o[i][2] * alpha, o[i][3] * alpha};
 #pragma unroll
       for (int i = 0; i < CT; i++) o[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[i], pf, o[i], 0, 0, 0);
-      if (tile + 2 < ntiles) store_k(d & 1, (d + 2) % DEPTH);
-      if (tile + 1 < ntiles) store_v((d + 1) & 1, (d + 1) % DEPTH);
       __syncthreads();
       s_cur[0] = s_next[0];
       s_cur[1] = s_next[1];
@@ -537,10 +556,11 @@ int attention_dispatch(const void* q, const void* k_cache, const void* vt_cache,
     const bool deep = max_q_len <= 16;  // decode: one block of queries per sequence
     if ((int64_t)max_q_len * G <= 16) {  // all queries of a sequence and all heads of a group in one MFMA tile
       const dim3 grid((unsigned)kv_heads, (unsigned)batch, 1u);
-      if (G == 1) hipLaunchKernelGGL(attention_decode_kernel<1>, grid, dim3(256), 0, stream, a);
-      else if (G == 2) hipLaunchKernelGGL(attention_decode_kernel<2>, grid, dim3(256), 0, stream, a);
-      else if (G == 4) hipLaunchKernelGGL(attention_decode_kernel<4>, grid, dim3(256), 0, stream, a);
-      else hipLaunchKernelGGL(attention_decode_kernel<8>, grid, dim3(256), 0, stream, a);
+      constexpr size_t lds = 2 * 4 * 8192;
+      if (G == 1) hipLaunchKernelGGL(attention_decode_kernel<1>, grid, dim3(512), lds, stream, a);
+      else if (G == 2) hipLaunchKernelGGL(attention_decode_kernel<2>, grid, dim3(512), lds, stream, a);
+      else if (G == 4) hipLaunchKernelGGL(attention_decode_kernel<4>, grid, dim3(512), lds, stream, a);
+      else hipLaunchKernelGGL(attention_decode_kernel<8>, grid, dim3(512), lds, stream, a);
       return hip_code(hipGetLastError());
     }
     const int64_t gx = (int64_t)((max_q_len + 15) / 16) * kv_heads;
