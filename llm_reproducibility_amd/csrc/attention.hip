@@ -178,9 +178,12 @@ __global__ __launch_bounds__(64) void attention_kernel(const AttnArgs a) {
 // by every wave.  A row's arithmetic -- the lanes that own it, the MFMA chain, the order of the softmax updates --
 // is exactly that of attention_kernel above, so both kernels produce the same bits; this one just moves 1/G of
 // the bytes and hides the load latency behind the previous tile.
+// NLD > 0: that many more wavefronts in the work-group do all the staging (loads, LDS writes) at the same barriers and
+// the G computing waves none of it: for launches that leave the chip short of work-groups, where a work-group's time is
+// its own chain of tiles rather than its share of a CU.
 // ------------------------------------------------------------------------------------------------
-template <int G, bool DEEP>
-__global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs a) {
+template <int G, bool DEEP, int NLD = 0>
+__global__ __launch_bounds__(64 * (G + NLD)) void attention_group_kernel(const AttnArgs a) {
   __shared__ __attribute__((aligned(16))) uint8_t lds[2][16384];  // per buffer: K tile [32][128] (8 KiB), V^T tile [128][32] (8 KiB)
   const int b = blockIdx.y;
   // Work-groups are dealt to the eight XCDs round robin, each with an L2 of its own: with the KV head as the fastest
@@ -203,16 +206,13 @@ __global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs 
   const int qpos = ctx - qlen + min(qrow, qlen - 1);
   const int last_pos = ctx - qlen + min(qb * 16 + 15, qlen - 1);
 
-  const uint16_t* qp = a.q + ((int64_t)(a.q_start[b] + min(qrow, qlen - 1)) * a.q_heads + h) * HD;
-  bf16x8 qf[4];
-#pragma unroll
-  for (int c = 0; c < 4; c++) qf[c] = *reinterpret_cast<const bf16x8*>(qp + c * 32 + g * 8);
-
   const uint8_t* kbase = reinterpret_cast<const uint8_t*>(a.k_cache + ((int64_t)b * a.kv_heads + kvh) * a.max_len * HD);
   const uint8_t* vbase = reinterpret_cast<const uint8_t*>(a.vt_cache + ((int64_t)b * a.kv_heads + kvh) * (int64_t)HD * a.max_len);
 
   // cooperative staging: 512 16-byte chunks per tile and operand, NCH per thread
-  constexpr int NT = 64 * G;
+  // (NLD loader waves, where the kernel has them, do all of it; the computing waves then neither load nor store tiles)
+  constexpr int NT = NLD ? 64 * NLD : 64 * G;
+  const int stid = NLD ? tid - 64 * G : tid;   // staging thread
   constexpr int NCH = (512 + NT - 1) / NT;
   // Key tiles are fetched DEPTH tiles ahead into DEPTH register sets (set = tile % DEPTH).  DEEP is for decode: a
   // single block of queries per sequence makes the kernel a chain of memory round trips, and one tile of arithmetic
@@ -225,7 +225,7 @@ __global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs 
   uint32_t vsrc[NCH], kdst[NCH], vdst0[NCH], vdst1[NCH];
 #pragma unroll
   for (int i = 0; i < NCH; i++) {
-    const int ch = min(tid + i * NT, 511);
+    const int ch = min(max(stid, 0) + i * NT, 511);
     const int kr = ch >> 4, kc = ch & 15;   // key row, 16-byte chunk of its 256 bytes
     kdst[i] = kr * 256 + ((kc ^ (2 * (kr & 7))) << 4);
     // V^T: channel row vr (64 bytes = 32 keys), 16-byte chunk vc = keys 8vc .. 8vc+7.  The keys of a row are stored
@@ -253,8 +253,8 @@ __global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs 
     const int ks = k0 * (HD * 2), vs = k0 * 2;
 #pragma unroll
     for (int i = 0; i < NCH; i++) {
-      if (512 % NT == 0 || tid + i * NT < 512) {
-        kreg[i] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, (tid + i * NT) * 16, ks, 0);
+      if (512 % NT == 0 || stid + i * NT < 512) {
+        kreg[i] = __builtin_amdgcn_raw_buffer_load_b128(krsrc, (stid + i * NT) * 16, ks, 0);
         vreg[i] = __builtin_amdgcn_raw_buffer_load_b128(vrsrc, (int)vsrc[i], vs, 0);
       }
     }
@@ -264,13 +264,38 @@ __global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs 
     const u32x4* vreg = vregs[set];
 #pragma unroll
     for (int i = 0; i < NCH; i++) {
-      if (512 % NT == 0 || tid + i * NT < 512) {
+      if (512 % NT == 0 || stid + i * NT < 512) {
         *reinterpret_cast<u32x4*>(&lds[buf][kdst[i]]) = kreg[i];
         *reinterpret_cast<uint2*>(&lds[buf][vdst0[i]]) = make_uint2(vreg[i][0], vreg[i][1]);
         *reinterpret_cast<uint2*>(&lds[buf][vdst1[i]]) = make_uint2(vreg[i][2], vreg[i][3]);
       }
     }
   };
+
+  const int ntiles = last_pos / 32 + 1;
+  constexpr int UNROLL = DEPTH < 2 ? 2 : DEPTH;
+  if (NLD && stid >= 0) {
+    // ---- loader waves: the staging half of the loop below, at the same barriers
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++) load_tile(d, d);
+    store_tile(0, 0);
+    __syncthreads();
+    for (int t0 = 0; t0 < ntiles; t0 += UNROLL) {
+#pragma unroll
+      for (int d = 0; d < UNROLL; d++) {
+        const int tile = t0 + d;
+        if (tile >= ntiles) break;
+        load_tile(tile + DEPTH, d % DEPTH);
+        if (tile + 1 < ntiles) store_tile((d & 1) ^ 1, (d + 1) % DEPTH);
+        __syncthreads();
+      }
+    }
+    return;
+  }
+  const uint16_t* qp = a.q + ((int64_t)(a.q_start[b] + min(qrow, qlen - 1)) * a.q_heads + h) * HD;
+  bf16x8 qf[4];
+#pragma unroll
+  for (int c = 0; c < 4; c++) qf[c] = *reinterpret_cast<const bf16x8*>(qp + c * 32 + g * 8);
 
   f32x4 o[8];
 #pragma unroll
@@ -286,23 +311,23 @@ __global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs 
   for (int c = 0; c < 4; c++) kofs[c] = j * 256 + (((c * 4 + g) ^ (2 * (j & 7))) << 4);
   const uint32_t vofs = 8192 + j * 64 + (g ^ (2 * ((j >> 2) & 1))) * 16;
 
-  const int ntiles = last_pos / 32 + 1;
   // loads past the last tile are clamped to a valid address and never used: issuing them unconditionally keeps the
   // number of loads in flight static, so the waits below can leave the newer tiles in flight
+  if (!NLD) {
 #pragma unroll
-  for (int d = 0; d < DEPTH; d++) load_tile(d, d);
-  store_tile(0, 0);
+    for (int d = 0; d < DEPTH; d++) load_tile(d, d);
+    store_tile(0, 0);
+  }
   __syncthreads();
   // the loop body covers UNROLL (an even number of) tiles, so that the LDS buffer of each is a compile-time constant and
   // every LDS address is a per-thread offset plus an immediate
-  constexpr int UNROLL = DEPTH < 2 ? 2 : DEPTH;
   for (int t0 = 0; t0 < ntiles; t0 += UNROLL) {
 #pragma unroll
    for (int d = 0; d < UNROLL; d++) {
     const int tile = t0 + d;
     if (tile >= ntiles) break;
     const int cur = d & 1;
-    load_tile(tile + DEPTH, d % DEPTH);  // that set held this tile and went to LDS a tile ago
+    if (!NLD) load_tile(tile + DEPTH, d % DEPTH);  // that set held this tile and went to LDS a tile ago
     const int k0 = tile * 32;
     const uint8_t* tb = &lds[cur][0];
     f32x4 s[2];
@@ -335,7 +360,7 @@ __global__ __launch_bounds__(64 * G) void attention_group_kernel(const AttnArgs 
       const bf16x8 vf = *reinterpret_cast<const bf16x8*>(tb + vofs + t * 1024);
       o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[t], 0, 0, 0);
     }
-    if (tile + 1 < ntiles) store_tile(cur ^ 1, (d + 1) % DEPTH);
+    if (!NLD && tile + 1 < ntiles) store_tile(cur ^ 1, (d + 1) % DEPTH);
     __syncthreads();
    }
   }
@@ -566,13 +591,23 @@ int attention_dispatch(const void* q, const void* k_cache, const void* vt_cache,
     const int64_t gx = (int64_t)((max_q_len + 15) / 16) * kv_heads;
     if (gx > 0x7fffffff) return TBIK_ERR_INVALID;
     const dim3 grid((unsigned)gx, (unsigned)batch, 1u);
-    if (G == 1) hipLaunchKernelGGL((attention_group_kernel<1, false>), grid, dim3(64), 0, stream, a);
-    else if (G == 2 && deep) hipLaunchKernelGGL((attention_group_kernel<2, true>), grid, dim3(128), 0, stream, a);
-    else if (G == 2) hipLaunchKernelGGL((attention_group_kernel<2, false>), grid, dim3(128), 0, stream, a);
-    else if (G == 4 && deep) hipLaunchKernelGGL((attention_group_kernel<4, true>), grid, dim3(256), 0, stream, a);
-    else if (G == 4) hipLaunchKernelGGL((attention_group_kernel<4, false>), grid, dim3(256), 0, stream, a);
-    else if (deep) hipLaunchKernelGGL((attention_group_kernel<8, true>), grid, dim3(512), 0, stream, a);
-    else hipLaunchKernelGGL((attention_group_kernel<8, false>), grid, dim3(512), 0, stream, a);
+    // Two more waves per work-group that only stage the tiles (NLD = 2) take the loads and LDS writes out of the computing
+    // waves' instruction streams.  That pays while the launch leaves CUs short of work-groups (a chunk of a prompt, a few
+    // sequences: up to two work-groups per CU: 3 - 18 % faster) and costs once the chip is full, where the extra waves
+    // take the place of a whole work-group (from three per CU on: 35 % slower).  Same bits either way.
+    const bool few = gx * batch <= 512;
+#define TBIK_ATTN_GROUP(GG)                                                                                              \
+  do {                                                                                                                   \
+    if (few && deep) hipLaunchKernelGGL((attention_group_kernel<GG, true, 2>), grid, dim3(64 * (GG + 2)), 0, stream, a);   \
+    else if (few) hipLaunchKernelGGL((attention_group_kernel<GG, false, 2>), grid, dim3(64 * (GG + 2)), 0, stream, a);    \
+    else if (deep) hipLaunchKernelGGL((attention_group_kernel<GG, true, 0>), grid, dim3(64 * GG), 0, stream, a);          \
+    else hipLaunchKernelGGL((attention_group_kernel<GG, false, 0>), grid, dim3(64 * GG), 0, stream, a);                   \
+  } while (0)
+    if (G == 1) TBIK_ATTN_GROUP(1);
+    else if (G == 2) TBIK_ATTN_GROUP(2);
+    else if (G == 4) TBIK_ATTN_GROUP(4);
+    else TBIK_ATTN_GROUP(8);
+#undef TBIK_ATTN_GROUP
   } else {
     const dim3 grid((unsigned)((max_q_len + 15) / 16), (unsigned)q_heads, (unsigned)batch);
     hipLaunchKernelGGL(attention_kernel, grid, dim3(64), 0, stream, a);
