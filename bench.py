@@ -403,6 +403,40 @@ def print_table(rows, hot):
               f"{r['GBps']:9.1f} {100 * r['GBps'] / PEAK_HBM_GBS:6.1f} {r['bound']:>6s}", file=sys.stderr)
 
 
+def decode_step(layers=12, prompt_len=512, batches=(1, 32, 128)):
+    """Wall time of a greedy decode step of the Qwen3-8B-architecture decoder (random weights, `layers` of its 36 layers,
+    TP = 1), per layer: two generate() calls that differ only in the number of new tokens, so the prefill cancels.
+    lm_head, the token choice and the embedding lookup run once per step and are in the figure (spread over `layers`)."""
+    import torch
+    from llm_reproducibility_amd.decoder import DecoderConfig, Qwen3Decoder
+    cfg = DecoderConfig(num_layers=layers)
+    t0 = time.perf_counter()
+    model = Qwen3Decoder(cfg, tp_size=1, seed=0, init_on_device=True)
+    g = torch.Generator().manual_seed(1)
+    prompts = torch.randint(0, cfg.vocab_size, (max(batches), prompt_len), generator=g).tolist()
+    out = {}
+    short, long_ = 9, 41
+
+    def run(bs, n):
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        model.generate(prompts[:bs], n)
+        torch.cuda.synchronize()
+        return time.perf_counter() - t
+    for bs in batches:
+        run(bs, short)                                   # warm-up (first use of every kernel at this batch size)
+        a = min(run(bs, short) for _ in range(2))
+        b = min(run(bs, long_) for _ in range(2))
+        step_us = (b - a) / (long_ - short) * 1e6
+        out[f"batch_{bs}"] = {"us_per_step": round(step_us, 1), "us_per_layer": round(step_us / layers, 1)}
+    out["config"] = (f"{layers} layers of the 8B architecture (hidden 4096, 32/8 heads, intermediate 12288, vocabulary 151936), prompts of "
+                     f"{prompt_len} tokens, wall time between the steps {short} and {long_} of greedy decoding, host launches included; "
+                     f"{time.perf_counter() - t0:.0f} s")
+    del model
+    torch.cuda.empty_cache()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -420,6 +454,7 @@ def main():
     ap.add_argument("--no-ceiling", action="store_true",
                     help="skip `context.ceiling`: the MFMA-only and one-pass-read ceilings of this chip and the board power "
                          "while the headline step, this library's plain mm, the vendor GEMM and the probes run (10 s)")
+    ap.add_argument("--no-decode-step", action="store_true", help="leave the decode-step timing of the 12-layer decoder out")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run 5 plain device copies of X (50,331,648 B read + as many written each) so that a "
                          "counter run can scale FETCH_SIZE / WRITE_SIZE by what a copy of known size reads")
@@ -504,6 +539,11 @@ def main():
         context["table_cols"] = ("[us per call (Python operator, HIP events, 12 calls after 10 ms of load, inputs "
                                  + ("reused" if args.table_hot else "cycled: cold") + "), algorithmic flop (m) or bytes (h), share of "
                                  f"{PEAK_BF16_TFLOPS:g} TFLOP/s (m) or {PEAK_HBM_GBS:g} GB/s (h), bound]; {time.perf_counter() - t0:.0f} s")
+
+    # (with the compact per-shape table only: the profiler commands that switch the table off or ask for its long form stay
+    # free of the decoder's kernels)
+    if not args.no_decode_step and not args.no_context_table and not args.table and not args.only:
+        context["decode_step"] = decode_step()
 
     # ---- not timed: what was timed equals the simulated TP=4 run bit for bit and agrees with the CPU oracle on the same
     # inputs within the stated tolerance (1 bf16 ulp, or 2^-8 of the output scale); the oracle run is also the CPU baseline
