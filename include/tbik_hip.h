@@ -332,6 +332,25 @@ int bi_qk_norm_rope_cache_bf16(const void* qkv, int64_t ld,
                                float eps, tbik_stream_t stream);
 
 /*
+ * One decode step of an attention block in one launch: bi_qk_norm_rope_cache_bf16 followed by bi_attention_bf16 for
+ * sequences that each bring ONE new token.  Row b of qkv [batch, (q_heads + 2*kv_heads) * 128] (row stride ld) is
+ * sequence b's token at position ctx_len[b] - 1 (ctx_len: cache length including it, device int32 [batch]; a sequence
+ * with ctx_len <= 0 is skipped).  The work-group of a (sequence, KV head) forms its query heads, the key and the value
+ * itself, files key and value in the caches and attends: out [batch, q_heads, 128].  Bit-identical to the two calls
+ * (the same per-head function, the same attention kernel).
+ * Returns TBIK_ERR_UNSUPPORTED (3), with nothing launched, where the decode attention kernel does not apply (max_len
+ * not a multiple of 32, query heads per KV head not 1, 2, 4 or 8): the caller then makes the two calls.
+ * Replaces: the rotary-embedding patch and the attention kernel of the alignment mode for a decode step,
+ *           src/patch/patch_training_inference_align.py:35-44 and :171-487.
+ */
+int bi_attention_decode_qkv_bf16(const void* qkv, int64_t ld,
+                                 const void* q_weight, const void* k_weight, const float* inv_freq,
+                                 void* k_cache, void* vt_cache, void* out,
+                                 const int32_t* ctx_len,
+                                 int batch, int q_heads, int kv_heads, int head_dim, int max_len,
+                                 float scale, float eps, tbik_stream_t stream);
+
+/*
  * Greedy sampling: out[r] (int64) = index of the largest element of row r of x [rows, cols] (bf16, row stride ld
  * elements), ties resolved to the lowest index; the pair order (value, then lowest index) is total, so the result
  * does not depend on how a row is split over lanes.  A NaN is never selected (a row of NaNs gives 0).

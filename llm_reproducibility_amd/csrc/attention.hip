@@ -23,6 +23,7 @@
 // contiguous load.  Cache entries behind ctx_len must be finite (they are multiplied by an exact 0).
 #include "common.h"
 #include "lds_direct.h"
+#include "qk_norm_rope.h"
 
 namespace tbik {
 
@@ -39,6 +40,19 @@ struct AttnArgs {
 };
 
 constexpr int HD = 128;
+
+// The decode kernel that forms its own queries and the new key/value (FUSED): sequence b's one new token is row b of the
+// fused qkv projection output, at position ctx_len[b] - 1.
+struct QkvArgs {
+  const uint16_t* qkv;    // [batch, (q_heads + 2 kv_heads) * 128], row stride ld
+  int64_t ld;
+  const uint16_t* qw;     // per-head q norm weight [128]
+  const uint16_t* kw;     // per-head k norm weight [128]
+  const float* inv_freq;  // [64]
+  uint16_t* k_cache;      // the caches of AttnArgs, writable: the new key and value are filed here as well
+  uint16_t* vt_cache;
+  float eps;
+};
 
 // One online-softmax update of a query row for a tile of 32 keys, shared by all kernels of this file (one body: the same
 // bits).  Lane (j, g) holds the scores of query j for keys k0 + 16u + 4g + i in s[u][i]; on return p holds the four packed
@@ -401,8 +415,8 @@ __global__ __launch_bounds__(64 * (G + NLD)) void attention_group_kernel(const A
 // A row's arithmetic -- the lanes that own it, the MFMA chains over channels and key slots, the order of the softmax
 // updates -- is that of the kernels above: the same bits.
 // ------------------------------------------------------------------------------------------------
-template <int G>
-__global__ __launch_bounds__(512) void attention_decode_kernel(const AttnArgs a) {
+template <int G, bool FUSED>
+__global__ __launch_bounds__(512) void attention_decode_kernel(const AttnArgs a, const QkvArgs f) {
   constexpr int NS = 4;               // ring slots per operand (2 x 4 x 8 KiB of LDS)
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds_dyn[];
   uint8_t (*lds_k)[8192] = reinterpret_cast<uint8_t (*)[8192]>(lds_dyn);
@@ -452,14 +466,15 @@ __global__ __launch_bounds__(512) void attention_decode_kernel(const AttnArgs a)
       load_k(i + 1, i + 1);
       load_v(i, i);
     }
-    const int qlen = a.q_len[b];
+    const int ctx = a.ctx_len[b];
+    const int qlen = FUSED ? (ctx > 0 ? 1 : 0) : a.q_len[b];
     if (qlen <= 0) {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       return;
     }
-    const int ctx = a.ctx_len[b];
     const int last_pos = ctx - qlen + min(QMAX - 1, qlen - 1);
     const int ntiles = last_pos / 32 + 1;
+    if (FUSED) __syncthreads();  // the computing waves exchange the heads they formed
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * PI * (NS - 1)) : "memory");  // K tile 0
     __syncthreads();
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * PI * (NS - 2)) : "memory");  // K tile 1, V^T tile 0
@@ -479,21 +494,66 @@ __global__ __launch_bounds__(512) void attention_decode_kernel(const AttnArgs a)
     return;
   }
   // ---------------- computing waves
-  const int qlen = a.q_len[b];
+  const int ctx = a.ctx_len[b];
+  const int qlen = FUSED ? (ctx > 0 ? 1 : 0) : a.q_len[b];
   if (qlen <= 0) return;
   const int qi = j / G;
   const int h = kvh * G + j % G;
-  const int ctx = a.ctx_len[b];
   const bool qvalid = qi < qlen;
   const int qrow = min(qi, qlen - 1);
   const int qpos = ctx - qlen + qrow;
   const int last_pos = ctx - qlen + min(QMAX - 1, qlen - 1);
   const int ntiles = last_pos / 32 + 1;
   const int nfull = (ctx - qlen + 1) / 32;
-  const uint16_t* qp = a.q + ((int64_t)(a.q_start[b] + qrow) * a.q_heads + h) * HD;
   bf16x8 qf[4];
+  // FUSED: the G query heads, the key head and the value head of this (sequence, KV head) are formed here, one head per
+  // wave at a time (per-head RMSNorm and rotary embedding as the stand-alone kernel does them), left in LDS for all four
+  // waves and, the key and the value, filed in the caches for the steps to come.  This step takes them from LDS: the tile
+  // that a loader brings in for their position holds whatever the cache held there, and is patched below.
+  uint16_t* hs = reinterpret_cast<uint16_t*>(lds_dyn + 2 * NS * 8192);  // [G + 2][128]: q heads, k, v
+  const int pos = ctx - 1;
+  if (FUSED) {
+    const uint16_t* row = f.qkv + (int64_t)b * f.ld;
+    for (int u = wv; u < G + 2; u += 4) {  // wave-uniform
+      const int head = u < G ? kvh * G + u : (u == G ? a.q_heads + kvh : a.q_heads + a.kv_heads + kvh);
+      const uint16_t* src = row + (int64_t)head * HD;
+      const uint16_t r1 = src[lane], r2 = src[lane + 64];
+      uint32_t o = (uint32_t)r1 | ((uint32_t)r2 << 16);
+      if (u <= G) o = qk_norm_rope_head(r1, r2, u < G ? f.qw : f.kw, pos, f.inv_freq, f.eps, lane);
+      hs[u * HD + lane] = (uint16_t)(o & 0xffffu);
+      hs[u * HD + lane + 64] = (uint16_t)(o >> 16);
+      if (u == G && pos < a.max_len) {
+        uint16_t* dst = f.k_cache + (((int64_t)b * a.kv_heads + kvh) * a.max_len + pos) * HD;
+        dst[lane] = (uint16_t)(o & 0xffffu);
+        dst[lane + 64] = (uint16_t)(o >> 16);
+      }
+      if (u == G + 1 && pos < a.max_len) {
+        uint16_t* dst = f.vt_cache + ((int64_t)b * a.kv_heads + kvh) * (int64_t)HD * a.max_len + pos;
+        dst[(int64_t)lane * a.max_len] = r1;
+        dst[(int64_t)(lane + 64) * a.max_len] = r2;
+      }
+    }
+    __syncthreads();
 #pragma unroll
-  for (int c = 0; c < 4; c++) qf[c] = *reinterpret_cast<const bf16x8*>(qp + c * 32 + g * 8);
+    for (int c = 0; c < 4; c++) qf[c] = *reinterpret_cast<const bf16x8*>(hs + (j % G) * HD + c * 32 + g * 8);
+  } else {
+    const uint16_t* qp = a.q + ((int64_t)(a.q_start[b] + qrow) * a.q_heads + h) * HD;
+#pragma unroll
+    for (int c = 0; c < 4; c++) qf[c] = *reinterpret_cast<const bf16x8*>(qp + c * 32 + g * 8);
+  }
+  // the new key's row of the K tile in `slot` and the new value's column of this wave's rows of the V^T tile, from LDS
+  // (each wave patches what it reads itself, right before it reads it: a wave's LDS operations keep their order)
+  const int lt = pos >> 5, pr = pos & 31;
+  auto patch_k = [&](int slot) __attribute__((always_inline)) {
+    if (lane < 16)
+      *reinterpret_cast<u32x4*>(&lds_k[slot][pr * 256 + ((lane ^ (2 * (pr & 7))) << 4)]) = *reinterpret_cast<const u32x4*>(hs + G * HD + lane * 8);
+  };
+  auto patch_v = [&](int slot) __attribute__((always_inline)) {
+    if (lane < 16 * CT) {
+      const int ch = 16 * CT * wv + lane;
+      *reinterpret_cast<uint16_t*>(&lds_v[slot][ch * 64 + (((pr >> 3) ^ ((ch >> 2) & 3)) << 4) + (pr & 7) * 2]) = hs[(G + 1) * HD + ch];
+    }
+  };
   uint32_t kofs[4];
 #pragma unroll
   for (int c = 0; c < 4; c++) kofs[c] = j * 256 + (((c * 4 + g) ^ (2 * (j & 7))) << 4);
@@ -520,6 +580,7 @@ __global__ __launch_bounds__(512) void attention_decode_kernel(const AttnArgs a)
   float m = -INFINITY;
   float l = 0.f;
   __syncthreads();
+  if (FUSED && lt == 0) patch_k(0);
   f32x4 s_cur[2];
   scores(0, s_cur);
   __syncthreads();
@@ -528,6 +589,8 @@ __global__ __launch_bounds__(512) void attention_decode_kernel(const AttnArgs a)
     for (int d = 0; d < NS; d++) {
       const int tile = t0 + d;
       if (tile >= ntiles) break;
+      if (FUSED && tile == lt) patch_v(d);
+      if (FUSED && tile + 1 == lt) patch_k((d + 1) % NS);
       bf16x8 vf[CT];
 #pragma unroll
       for (int i = 0; i < CT; i++) {
@@ -552,7 +615,7 @@ __global__ __launch_bounds__(512) void attention_decode_kernel(const AttnArgs a)
   }
   if (!qvalid) return;
   const float inv = 1.0f / l;
-  uint16_t* op = a.out + ((int64_t)(a.q_start[b] + qi) * a.q_heads + h) * HD + 16 * CT * wv;
+  uint16_t* op = a.out + ((int64_t)(FUSED ? b : a.q_start[b] + qi) * a.q_heads + h) * HD + 16 * CT * wv;
 #pragma unroll
   for (int i = 0; i < CT; i++) {
     const uint32_t lo = pack_bf16x2(o[i][0] * inv, o[i][1] * inv);
@@ -582,10 +645,11 @@ int attention_dispatch(const void* q, const void* k_cache, const void* vt_cache,
     if ((int64_t)max_q_len * G <= 16) {  // all queries of a sequence and all heads of a group in one MFMA tile
       const dim3 grid((unsigned)kv_heads, (unsigned)batch, 1u);
       constexpr size_t lds = 2 * 4 * 8192;
-      if (G == 1) hipLaunchKernelGGL(attention_decode_kernel<1>, grid, dim3(512), lds, stream, a);
-      else if (G == 2) hipLaunchKernelGGL(attention_decode_kernel<2>, grid, dim3(512), lds, stream, a);
-      else if (G == 4) hipLaunchKernelGGL(attention_decode_kernel<4>, grid, dim3(512), lds, stream, a);
-      else hipLaunchKernelGGL(attention_decode_kernel<8>, grid, dim3(512), lds, stream, a);
+      const QkvArgs none{};
+      if (G == 1) hipLaunchKernelGGL((attention_decode_kernel<1, false>), grid, dim3(512), lds, stream, a, none);
+      else if (G == 2) hipLaunchKernelGGL((attention_decode_kernel<2, false>), grid, dim3(512), lds, stream, a, none);
+      else if (G == 4) hipLaunchKernelGGL((attention_decode_kernel<4, false>), grid, dim3(512), lds, stream, a, none);
+      else hipLaunchKernelGGL((attention_decode_kernel<8, false>), grid, dim3(512), lds, stream, a, none);
       return hip_code(hipGetLastError());
     }
     const int64_t gx = (int64_t)((max_q_len + 15) / 16) * kv_heads;
@@ -612,6 +676,38 @@ int attention_dispatch(const void* q, const void* k_cache, const void* vt_cache,
     const dim3 grid((unsigned)((max_q_len + 15) / 16), (unsigned)q_heads, (unsigned)batch);
     hipLaunchKernelGGL(attention_kernel, grid, dim3(64), 0, stream, a);
   }
+  return hip_code(hipGetLastError());
+}
+
+// One decode step of an attention block from the fused qkv projection output: per-head q/k RMSNorm, rotary embedding, the
+// cache write and the attention of every sequence's one new token (row b of qkv, position ctx_len[b] - 1) in one launch.
+// The bits of qk_norm_rope_cache_dispatch followed by attention_dispatch.  TBIK_ERR_UNSUPPORTED where the decode kernel
+// does not apply (cache length not a whole number of tiles, more than 8 or an odd number of query heads per KV head):
+// the caller makes the two calls.
+int attention_decode_qkv_dispatch(const void* qkv, int64_t ld, const void* q_weight, const void* k_weight, const float* inv_freq,
+                                  void* k_cache, void* vt_cache, void* out, const int* ctx_len, int batch, int q_heads,
+                                  int kv_heads, int head_dim, int max_len, float scale, float eps, hipStream_t stream) {
+  if (!qkv || !q_weight || !k_weight || !inv_freq || !k_cache || !vt_cache || !out || !ctx_len) return TBIK_ERR_INVALID;
+  if (batch <= 0 || q_heads <= 0 || kv_heads <= 0 || q_heads % kv_heads != 0) return TBIK_ERR_INVALID;
+  if (head_dim != HD) return TBIK_ERR_UNSUPPORTED;
+  if (ld < (int64_t)(q_heads + 2 * kv_heads) * HD) return TBIK_ERR_INVALID;
+  if (max_len < 32 || (max_len & 3)) return TBIK_ERR_ALIGNMENT;
+  auto mis = [](const void* p, uintptr_t m) { return (reinterpret_cast<uintptr_t>(p) & m) != 0; };
+  if (mis(k_cache, 15) || mis(vt_cache, 15) || mis(out, 15) || mis(qkv, 1) || mis(q_weight, 1) || mis(k_weight, 1) || mis(inv_freq, 3))
+    return TBIK_ERR_ALIGNMENT;
+  if (batch > 65535 || kv_heads > 65535) return TBIK_ERR_INVALID;
+  const int G = q_heads / kv_heads;
+  if ((max_len & 31) != 0 || !(G == 1 || G == 2 || G == 4 || G == 8) || max_len > (1 << 22)) return TBIK_ERR_UNSUPPORTED;
+  AttnArgs a{nullptr, static_cast<const uint16_t*>(k_cache), static_cast<const uint16_t*>(vt_cache), static_cast<uint16_t*>(out),
+             nullptr, nullptr, ctx_len, q_heads, kv_heads, max_len, scale * 1.4426950408889634f};
+  const QkvArgs f{static_cast<const uint16_t*>(qkv), ld, static_cast<const uint16_t*>(q_weight), static_cast<const uint16_t*>(k_weight),
+                  inv_freq, static_cast<uint16_t*>(k_cache), static_cast<uint16_t*>(vt_cache), eps};
+  const dim3 grid((unsigned)kv_heads, (unsigned)batch, 1u);
+  const size_t lds = 2 * 4 * 8192 + (size_t)(G + 2) * HD * 2;
+  if (G == 1) hipLaunchKernelGGL((attention_decode_kernel<1, true>), grid, dim3(512), lds, stream, a, f);
+  else if (G == 2) hipLaunchKernelGGL((attention_decode_kernel<2, true>), grid, dim3(512), lds, stream, a, f);
+  else if (G == 4) hipLaunchKernelGGL((attention_decode_kernel<4, true>), grid, dim3(512), lds, stream, a, f);
+  else hipLaunchKernelGGL((attention_decode_kernel<8, true>), grid, dim3(512), lds, stream, a, f);
   return hip_code(hipGetLastError());
 }
 

@@ -32,6 +32,9 @@ int silu_mul_dispatch(const void* gate_up, int64_t ld_in, void* out, int64_t ld_
 int rmsnorm_gemm_dispatch(const void* x, int64_t ldx, const void* res, int64_t ldr, const void* norm_w, float eps,
                           void* res_out, int64_t ldro, const void* B, int64_t ldb_k, int64_t ldb_n, void* C, int64_t ldc,
                           int M, int N, int K, const void* bias, hipStream_t stream);
+int attention_decode_qkv_dispatch(const void* qkv, int64_t ld, const void* q_weight, const void* k_weight, const float* inv_freq,
+                                  void* k_cache, void* vt_cache, void* out, const int* ctx_len, int batch, int q_heads,
+                                  int kv_heads, int head_dim, int max_len, float scale, float eps, hipStream_t stream);
 int gemm_tree_rmsnorm_dispatch(bool f16, const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, int M, int N,
                                int K, int leaf_k, const void* bias, const void* res, int64_t ldr, const void* norm_w, float eps,
                                void* res_out, int64_t ldro, void* out, int64_t ldo, void* ws, size_t ws_bytes,
@@ -45,7 +48,7 @@ int gemm_tree_gated_dispatch(const void* gate, const void* up, int64_t ld, const
 
 extern "C" {
 
-int tbik_abi_version(void) { return 15; }
+int tbik_abi_version(void) { return 16; }
 
 const char* tbik_error_string(int code) {
   switch (code) {
@@ -217,6 +220,13 @@ int bi_qk_norm_rope_cache_bf16(const void* qkv, int64_t ld, const void* q_weight
   return tbik::qk_norm_rope_cache_dispatch(qkv, ld, q_weight, k_weight, inv_freq, positions, seq_of_token, q_out, k_cache,
                                            vt_cache, tokens, q_heads, kv_heads, head_dim, max_len, batch, eps,
                                            static_cast<hipStream_t>(stream));
+}
+
+int bi_attention_decode_qkv_bf16(const void* qkv, int64_t ld, const void* q_weight, const void* k_weight, const float* inv_freq,
+                                 void* k_cache, void* vt_cache, void* out, const int32_t* ctx_len, int batch, int q_heads,
+                                 int kv_heads, int head_dim, int max_len, float scale, float eps, tbik_stream_t stream) {
+  return tbik::attention_decode_qkv_dispatch(qkv, ld, q_weight, k_weight, inv_freq, k_cache, vt_cache, out, ctx_len, batch,
+                                             q_heads, kv_heads, head_dim, max_len, scale, eps, static_cast<hipStream_t>(stream));
 }
 
 int bi_argmax_bf16(const void* x, int64_t ld, void* out, int64_t rows, int cols, tbik_stream_t stream) {

@@ -6,6 +6,7 @@
 // then the product rounded to bf16 -- two roundings, as an unfused `F.silu(gate) * up` on bf16 tensors
 // gives.  Elementwise, so batch invariant by construction.  HBM bound: 6 bytes per output element.
 #include "common.h"
+#include "qk_norm_rope.h"
 #include "silu_mul.h"
 
 namespace tbik {
@@ -105,15 +106,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_cache_kernel(const QkRopeArg
   }
   const bool is_q = hh < a.q_heads;
   const uint16_t* w = is_q ? a.qw : a.kw;
-  const float x1 = bf16_bits_to_f32(r1), x2 = bf16_bits_to_f32(r2);
-  const float ss = wave_sum(fmaf(x1, x1, x2 * x2));
-  const float rs = 1.0f / sqrtf(ss * (1.0f / 128.0f) + a.eps);
-  const uint32_t nrm = pack_bf16x2(x1 * rs, x2 * rs);
-  const uint32_t wv = pack_bf16x2(bf16_lo(nrm) * bf16_bits_to_f32(w[lane]), bf16_hi(nrm) * bf16_bits_to_f32(w[lane + 64]));
-  const float y1 = bf16_lo(wv), y2 = bf16_hi(wv);
-  const float ang = (float)pos * a.inv_freq[lane];
-  const float c = cosf(ang), s = sinf(ang);
-  const uint32_t o = pack_bf16x2(y1 * c - y2 * s, y2 * c + y1 * s);
+  const uint32_t o = qk_norm_rope_head(r1, r2, w, pos, a.inv_freq, a.eps, lane);
   uint16_t* dst;
   if (is_q) {
     dst = a.q_out + (tok * a.q_heads + hh) * 128;

@@ -62,7 +62,7 @@ class _Layer:
 class Qwen3Decoder:
     def __init__(self, cfg: DecoderConfig, tp_size: int = 1, seed: int = 0, device="cuda:0", use_graphs: bool = False,
                  fused_rope: bool = True, init_on_device: bool = False, fused_producers: bool = True,
-                 fused_consumers: bool = True):
+                 fused_consumers: bool = True, fused_attention_step: bool = True):
         assert cfg.head_dim == 128, "the attention kernel is built for head_dim 128"
         self.cfg, self.tp_size, self.device = cfg, tp_size, torch.device(device)
         # decode steps replayed from one captured HIP graph (same kernels, same order, same bits as eager; the
@@ -75,6 +75,9 @@ class Qwen3Decoder:
         # beyond a handful of rows: the add-RMSNorm behind o_proj and down_proj inside the launch that combines the layer's
         # K shards (bit-identical to the separate norm; the switch only exists for the tests)
         self.fused_consumers = fused_consumers
+        # decode steps (one new token per sequence): q/k norm, rotary embedding, cache write and attention in one launch
+        # (bit-identical to the two launches; the switch only exists for the tests)
+        self.fused_attention_step = fused_attention_step and fused_rope
         gen = torch.Generator(device=self.device if init_on_device else "cpu").manual_seed(seed)
         emb = lambda *shape: _normal_bf16(shape, gen, self.device)  # noqa: E731
         self.embed = emb(cfg.vocab_size, cfg.hidden_size)
@@ -124,7 +127,11 @@ class Qwen3Decoder:
                 qkv = matmul_persistent(h, layer.qkv_w.t())
                 h = None
             k_cache, vt_cache = cache[li]
-            if self.fused_rope:
+            if self.fused_attention_step and max_q_len == 1 and qkv.shape[0] == ctx_len.numel():
+                # a decode step: token b is sequence b's, at position ctx_len[b] - 1
+                attn = ops.bi_attention_decode_qkv(qkv, layer.q_norm, layer.k_norm, self.inv_freq, k_cache, vt_cache, ctx_len,
+                                                   Hq, Hkv, self.scale, cfg.rms_eps)
+            elif self.fused_rope:
                 # per-head q/k norm, rotary embedding and the cache write in one kernel
                 q = ops.bi_qk_norm_rope_cache_bf16(qkv, layer.q_norm, layer.k_norm, self.inv_freq, positions, seq_of_token,
                                                    k_cache, vt_cache, Hq, Hkv, cfg.rms_eps)
@@ -136,7 +143,8 @@ class Qwen3Decoder:
                 k = self._rope(rms_norm(k.contiguous(), layer.k_norm, cfg.rms_eps), positions)
                 k_cache[seq_of_token, :, positions] = k             # [tokens, Hkv, D] -> [B, Hkv, L, D]
                 vt_cache[seq_of_token, :, :, positions] = v         # stored transposed: [B, Hkv, D, L]
-            attn = ops.bi_attention_bf16(q, k_cache, vt_cache, q_start, q_len, ctx_len, max_q_len, self.scale)
+            if not (self.fused_attention_step and max_q_len == 1 and qkv.shape[0] == ctx_len.numel()):
+                attn = ops.bi_attention_bf16(q, k_cache, vt_cache, q_start, q_len, ctx_len, max_q_len, self.scale)
             if fused:
                 x = layer.o_proj(attn.reshape(-1, Hq * D))
                 gu, residual = ops.rmsnorm_gemm(x, layer.post_norm, cfg.rms_eps, residual, layer.gate_up_w.t())

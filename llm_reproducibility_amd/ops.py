@@ -633,6 +633,36 @@ def bi_qk_norm_rope_cache_bf16(qkv: torch.Tensor, q_weight: torch.Tensor, k_weig
     return q_out
 
 
+def bi_attention_decode_qkv(qkv: torch.Tensor, q_weight: torch.Tensor, k_weight: torch.Tensor, inv_freq: torch.Tensor,
+                            k_cache: torch.Tensor, vt_cache: torch.Tensor, ctx_len: torch.Tensor, q_heads: int, kv_heads: int,
+                            scale: float, eps: float) -> torch.Tensor:
+    """A decode step of an attention block for sequences with one new token each (row b of qkv = sequence b's token at
+    position ctx_len[b] - 1): per-head q/k norm, rotary embedding, cache write (in place) and attention in one launch
+    (`bi_attention_decode_qkv_bf16`), the two calls where that kernel does not apply.  Same bits either way."""
+    _require_gpu(qkv, q_weight, k_weight, inv_freq, k_cache, vt_cache, ctx_len)
+    B = qkv.shape[0]
+    assert qkv.dtype == torch.bfloat16 and qkv.stride(1) == 1 and qkv.shape[1] == (q_heads + 2 * kv_heads) * 128
+    assert k_cache.is_contiguous() and vt_cache.is_contiguous() and k_cache.shape[1] == kv_heads and k_cache.shape[3] == 128
+    assert ctx_len.dtype == torch.int32 and ctx_len.numel() == B and k_cache.shape[0] == B and inv_freq.dtype == torch.float32
+    max_len = k_cache.shape[2]
+    if ("attn_qkv", q_heads, kv_heads, max_len % 32) not in _declined:
+        out = torch.empty((B, q_heads, 128), device=qkv.device, dtype=qkv.dtype)
+        rc = _lib.lib().bi_attention_decode_qkv_bf16(
+            qkv.data_ptr(), qkv.stride(0) if B > 1 else max(qkv.stride(0), qkv.shape[1]), q_weight.contiguous().data_ptr(),
+            k_weight.contiguous().data_ptr(), inv_freq.contiguous().data_ptr(), k_cache.data_ptr(), vt_cache.data_ptr(),
+            out.data_ptr(), ctx_len.data_ptr(), B, q_heads, kv_heads, 128, max_len, scale, eps, _stream(qkv))
+        if rc == _lib.TBIK_OK:
+            return out
+        if rc != _lib.TBIK_ERR_UNSUPPORTED:
+            _lib.check(rc, "bi_attention_decode_qkv_bf16")
+        _declined.add(("attn_qkv", q_heads, kv_heads, max_len % 32))
+    pos = (ctx_len - 1).to(torch.int64)
+    seq = torch.arange(B, device=qkv.device, dtype=torch.int64)
+    q = bi_qk_norm_rope_cache_bf16(qkv, q_weight, k_weight, inv_freq, pos, seq, k_cache, vt_cache, q_heads, kv_heads, eps)
+    one = torch.ones(B, dtype=torch.int32, device=qkv.device)
+    return bi_attention_bf16(q, k_cache, vt_cache, torch.arange(B, dtype=torch.int32, device=qkv.device), one, ctx_len, 1, scale)
+
+
 def bi_argmax(logits: torch.Tensor) -> torch.Tensor:
     """Index (int64) of the largest element of each row of a 2-D bf16 tensor, ties resolved to the lowest index."""
     _require_gpu(logits)

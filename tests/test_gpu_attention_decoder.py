@@ -307,6 +307,86 @@ def test_fused_qk_norm_rope_cache_matches_the_unfused_composition(dev):
     assert (a[1].float() - b[1].float()).abs().max() < 0.05 * b[1].float().abs().max()
 
 
+@pytest.mark.parametrize("hq,hkv,ctxs,max_len", [
+    (32, 8, [1, 32, 33, 64, 65, 96, 128, 129, 160, 161, 577, 700, 736], 736),   # the new key in tile 0 .. 22, at tile edges
+    (8, 2, [5, 31, 100, 128, 0, 200], 224),                                      # a sequence without tokens is skipped
+    (16, 2, [40, 129, 7], 160),
+    (4, 2, [64, 1, 97], 128),
+    (2, 2, [33, 160, 2, 95], 160),
+])
+def test_decode_step_in_one_launch_equals_norm_rope_cache_write_then_attention(dev, hq, hkv, ctxs, max_len):
+    """q/k norm + rotary embedding + cache write + attention of one new token per sequence in ONE launch (the work-group
+    of a (sequence, KV head) forms its heads itself and patches the new key and value into the tiles its loaders bring in)
+    against the two launches: outputs and both caches bit for bit, wherever the new key falls in its tile and whichever
+    tile of the prefetch ring it is."""
+    from llm_reproducibility_amd import _lib
+    from llm_reproducibility_amd.patch.patch_training_inference_align import compute_inv_freq
+    torch.manual_seed(hq + len(ctxs))
+    D, B, scale, eps = 128, len(ctxs), 1.0 / math.sqrt(128), 1e-6
+    qkv = torch.randn((B, (hq + 2 * hkv) * D), device=dev).to(torch.bfloat16)
+    qw = (1 + 0.1 * torch.randn(D, device=dev)).to(torch.bfloat16)
+    kw = (1 + 0.1 * torch.randn(D, device=dev)).to(torch.bfloat16)
+    inv = compute_inv_freq(D, 1e6, dev)
+    kc0 = torch.randn((B, hkv, max_len, D), device=dev).to(torch.bfloat16)      # the history (and junk behind it)
+    vt0 = torch.randn((B, hkv, D, max_len), device=dev).to(torch.bfloat16)
+    ctx = torch.tensor(ctxs, dtype=torch.int32, device=dev)
+    live = [b for b, c in enumerate(ctxs) if c > 0]
+    print("case one-launch decode step", hq, hkv, ctxs, max_len, flush=True)
+    # the two launches, on the live sequences
+    kc_a, vt_a = kc0.clone(), vt0.clone()
+    pos = (ctx[live] - 1).to(torch.int64)
+    seq = torch.tensor(live, dtype=torch.int64, device=dev)
+    q = ops.bi_qk_norm_rope_cache_bf16(qkv[live], qw, kw, inv, pos, seq, kc_a, vt_a, hq, hkv, eps)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)  # noqa: E731
+    want = ops.bi_attention_bf16(q, kc_a[live].contiguous(), vt_a[live].contiguous(), i32(list(range(len(live)))), i32([1] * len(live)),
+                                 ctx[live].contiguous(), 1, scale)
+    # one launch (the raw entry point takes the shape: the wrapper below did not fall back)
+    kc_b, vt_b = kc0.clone(), vt0.clone()
+    out = torch.full((B, hq, D), 7.0, dtype=torch.bfloat16, device=dev)
+    rc = _lib.lib().bi_attention_decode_qkv_bf16(qkv.data_ptr(), qkv.stride(0), qw.data_ptr(), kw.data_ptr(), inv.data_ptr(),
+                                                 kc_b.data_ptr(), vt_b.data_ptr(), out.data_ptr(), ctx.data_ptr(), B, hq, hkv, D,
+                                                 max_len, scale, eps, torch.cuda.current_stream().cuda_stream)
+    assert rc == _lib.TBIK_OK
+    assert torch.equal(out[live], want)
+    assert torch.equal(kc_b, kc_a) and torch.equal(vt_b, vt_a)
+    for b, c in enumerate(ctxs):
+        if c <= 0:
+            assert (out[b] == 7.0).all()          # nothing written for a sequence without tokens
+    kc_c, vt_c = kc0.clone(), vt0.clone()
+    if len(live) == B:
+        got = ops.bi_attention_decode_qkv(qkv, qw, kw, inv, kc_c, vt_c, ctx, hq, hkv, scale, eps)
+        assert torch.equal(got, want) and torch.equal(kc_c, kc_a) and torch.equal(vt_c, vt_a)
+    # a sequence on its own gives the same bits as in the batch
+    b = live[-1]
+    kc1, vt1 = kc0[b:b + 1].clone(), vt0[b:b + 1].clone()
+    alone = ops.bi_attention_decode_qkv(qkv[b:b + 1], qw, kw, inv, kc1, vt1, ctx[b:b + 1].contiguous(), hq, hkv, scale, eps)
+    assert torch.equal(alone[0], out[b])
+    # a cache length that is not a whole number of tiles: the entry point declines, the wrapper makes the two calls
+    if len(live) == B:
+        L2 = max_len + 4
+        kc2 = torch.zeros((B, hkv, L2, D), dtype=torch.bfloat16, device=dev)
+        vt2 = torch.zeros((B, hkv, D, L2), dtype=torch.bfloat16, device=dev)
+        kc2[:, :, :max_len], vt2[:, :, :, :max_len] = kc0, vt0
+        assert _lib.lib().bi_attention_decode_qkv_bf16(qkv.data_ptr(), qkv.stride(0), qw.data_ptr(), kw.data_ptr(), inv.data_ptr(),
+                                                       kc2.data_ptr(), vt2.data_ptr(), out.data_ptr(), ctx.data_ptr(), B, hq, hkv, D,
+                                                       L2, scale, eps, torch.cuda.current_stream().cuda_stream) == _lib.TBIK_ERR_UNSUPPORTED
+        got2 = ops.bi_attention_decode_qkv(qkv, qw, kw, inv, kc2, vt2, ctx, hq, hkv, scale, eps)
+        assert torch.equal(got2, want) and torch.equal(kc2[:, :, :max_len], kc_a) and torch.equal(vt2[:, :, :, :max_len], vt_a)
+
+
+def test_decoder_with_and_without_the_one_launch_decode_step_gives_the_same_bits(dev):
+    prompts = _prompts(6, seed=11)
+    for tp in (1, 2):
+        a = Qwen3Decoder(SMALL, tp_size=tp, seed=0, device=dev, fused_attention_step=True)
+        b = Qwen3Decoder(SMALL, tp_size=tp, seed=0, device=dev, fused_attention_step=False)
+        for batch in (1, 3, 6):
+            print("case decoder one-launch decode step tp", tp, "batch", batch, flush=True)
+            ia, la = a.generate(prompts[:batch], 8, return_logits=True)
+            ib, lb = b.generate(prompts[:batch], 8, return_logits=True)
+            assert torch.equal(ia, ib) and torch.equal(la, lb), (tp, batch)
+        del a, b
+
+
 def test_graph_replayed_decode_steps_equal_eager_steps(dev):
     """Every replay of the captured decode step must give the eager step's bits (token ids and logits)."""
     prompts = _prompts(5, seed=7)
