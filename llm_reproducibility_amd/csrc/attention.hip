@@ -474,7 +474,34 @@ __global__ __launch_bounds__(512) void attention_decode_kernel(const AttnArgs a,
     }
     const int last_pos = ctx - qlen + min(QMAX - 1, qlen - 1);
     const int ntiles = last_pos / 32 + 1;
-    if (FUSED) __syncthreads();  // the computing waves exchange the heads they formed
+    if (FUSED) {
+      // loaders 0 and 1 form the new key and file the new value while the first tiles are on their way (the computing
+      // waves form the query heads meanwhile); everything they have in flight is drained before the barrier, so the waits
+      // below still count the tile loads alone
+      if (li < 2) {
+        uint16_t* hs = reinterpret_cast<uint16_t*>(lds_dyn + 2 * NS * 8192);
+        const int pos = ctx - 1;
+        const uint16_t* src = f.qkv + (int64_t)b * f.ld + (int64_t)(a.q_heads + (li == 0 ? 0 : a.kv_heads) + kvh) * HD;
+        const uint16_t r1 = src[lane], r2 = src[lane + 64];
+        uint32_t o = (uint32_t)r1 | ((uint32_t)r2 << 16);
+        if (li == 0) o = qk_norm_rope_head(r1, r2, f.kw, pos, f.inv_freq, f.eps, lane);
+        hs[(G + li) * HD + lane] = (uint16_t)(o & 0xffffu);
+        hs[(G + li) * HD + lane + 64] = (uint16_t)(o >> 16);
+        if (pos < a.max_len) {
+          if (li == 0) {
+            uint16_t* dst = f.k_cache + (((int64_t)b * a.kv_heads + kvh) * a.max_len + pos) * HD;
+            dst[lane] = (uint16_t)(o & 0xffffu);
+            dst[lane + 64] = (uint16_t)(o >> 16);
+          } else {
+            uint16_t* dst = f.vt_cache + ((int64_t)b * a.kv_heads + kvh) * (int64_t)HD * a.max_len + pos;
+            dst[(int64_t)lane * a.max_len] = r1;
+            dst[(int64_t)(lane + 64) * a.max_len] = r2;
+          }
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      }
+      __syncthreads();  // the heads are in LDS
+    }
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * PI * (NS - 1)) : "memory");  // K tile 0
     __syncthreads();
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * PI * (NS - 2)) : "memory");  // K tile 1, V^T tile 0
@@ -506,32 +533,19 @@ __global__ __launch_bounds__(512) void attention_decode_kernel(const AttnArgs a,
   const int ntiles = last_pos / 32 + 1;
   const int nfull = (ctx - qlen + 1) / 32;
   bf16x8 qf[4];
-  // FUSED: the G query heads, the key head and the value head of this (sequence, KV head) are formed here, one head per
-  // wave at a time (per-head RMSNorm and rotary embedding as the stand-alone kernel does them), left in LDS for all four
-  // waves and, the key and the value, filed in the caches for the steps to come.  This step takes them from LDS: the tile
+  // FUSED: the G query heads of this (sequence, KV head) are formed here, one head per wave at a time, the key and the
+  // value by two of the loader waves (per-head RMSNorm and rotary embedding as the stand-alone kernel does them); all are
+  // left in LDS for the four computing waves and, the key and the value, filed in the caches for the steps to come.  This step takes them from LDS: the tile
   // that a loader brings in for their position holds whatever the cache held there, and is patched below.
   uint16_t* hs = reinterpret_cast<uint16_t*>(lds_dyn + 2 * NS * 8192);  // [G + 2][128]: q heads, k, v
   const int pos = ctx - 1;
   if (FUSED) {
     const uint16_t* row = f.qkv + (int64_t)b * f.ld;
-    for (int u = wv; u < G + 2; u += 4) {  // wave-uniform
-      const int head = u < G ? kvh * G + u : (u == G ? a.q_heads + kvh : a.q_heads + a.kv_heads + kvh);
-      const uint16_t* src = row + (int64_t)head * HD;
-      const uint16_t r1 = src[lane], r2 = src[lane + 64];
-      uint32_t o = (uint32_t)r1 | ((uint32_t)r2 << 16);
-      if (u <= G) o = qk_norm_rope_head(r1, r2, u < G ? f.qw : f.kw, pos, f.inv_freq, f.eps, lane);
+    for (int u = wv; u < G; u += 4) {  // wave-uniform: the query heads (loaders 0 and 1 take the key and the value)
+      const uint16_t* src = row + (int64_t)(kvh * G + u) * HD;
+      const uint32_t o = qk_norm_rope_head(src[lane], src[lane + 64], f.qw, pos, f.inv_freq, f.eps, lane);
       hs[u * HD + lane] = (uint16_t)(o & 0xffffu);
       hs[u * HD + lane + 64] = (uint16_t)(o >> 16);
-      if (u == G && pos < a.max_len) {
-        uint16_t* dst = f.k_cache + (((int64_t)b * a.kv_heads + kvh) * a.max_len + pos) * HD;
-        dst[lane] = (uint16_t)(o & 0xffffu);
-        dst[lane + 64] = (uint16_t)(o >> 16);
-      }
-      if (u == G + 1 && pos < a.max_len) {
-        uint16_t* dst = f.vt_cache + ((int64_t)b * a.kv_heads + kvh) * (int64_t)HD * a.max_len + pos;
-        dst[(int64_t)lane * a.max_len] = r1;
-        dst[(int64_t)(lane + 64) * a.max_len] = r2;
-      }
     }
     __syncthreads();
 #pragma unroll

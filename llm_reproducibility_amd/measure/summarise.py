@@ -108,19 +108,21 @@ _KINDS = [("gemm_single_acc_stream", "batch-invariant mm (streaming kernels; RMS
           ("gemm_kernel<", "mm / tree GEMM (small-tile kernel)"),
           ("combine_rmsnorm", "shard combine of the K-cut tree GEMM with the add-RMSNorm of the result"),
           ("combine_", "shard combine of the K-cut tree GEMM"),
+          ("attention_decode", "attention (q/k norm + rotary + cache write inside where fused)"),
           ("attention", "attention"), ("rmsnorm", "RMSNorm (+ residual add)"), ("argmax", "token choice (arg-max kernel)"),
           ("silu_mul", "silu_mul"), ("qk_norm_rope", "q/k norm + rotary + cache write")]
 
 
 def decode(args) -> int:
     rows = _trace(args.dir)
-    rope = [i for i, (_, k, _) in enumerate(rows) if "qk_norm_rope" in k]
+    # a layer pass has exactly one attention launch (prefill or decode)
+    att = [i for i, (_, k, _) in enumerate(rows) if "attention" in k]
     need = args.steps * args.layers
-    if len(rope) < need + 1:
-        raise SystemExit(f"only {len(rope)} layer passes in the trace, {need} needed")
-    # the window starts with the kernels in front of the first rotary kernel of its first step (embedding lookup, the
+    if len(att) < need + 1:
+        raise SystemExit(f"only {len(att)} layer passes in the trace, {need} needed")
+    # the window starts with the kernels in front of the first attention launch of its first step (embedding lookup, the
     # first norm / projection): everything after the previous step's token choice
-    first = rope[-need]
+    first = att[-need]
     while first > 0 and "argmax" not in rows[first - 1][1]:
         first -= 1
     win = rows[first:]

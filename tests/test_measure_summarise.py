@@ -48,7 +48,7 @@ def test_counters_scaled_by_the_largest_copy_dispatch(tmp_path, capsys):
     assert "3000  (1 dispatches)" in capsys.readouterr().out
 
 
-def test_decode_breakdown_finds_the_steps_from_the_rotary_kernel(tmp_path, capsys):
+def test_decode_breakdown_finds_the_steps_from_the_attention_launches(tmp_path, capsys):
     t = [0]
 
     def k(name, us):
