@@ -11,7 +11,7 @@ import os
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG_DIR, "libtbik_hip.so")
 
-ABI_VERSION = 16
+ABI_VERSION = 17
 TBIK_OK = 0
 TBIK_ERR_INVALID = 1
 TBIK_ERR_ALIGNMENT = 2
@@ -27,7 +27,7 @@ EXPORTS = (
     "tbik_gemm_f16", "tbik_gemm_f16_workspace_bytes", "tbik_tree_combine_f16", "bi_gemm_f16", "tbik_gemm_f32", "bi_gemm_f32", "bi_rmsnorm_f16", "bi_silu_mul_f16", "bi_qk_norm_rope_cache_bf16", "bi_argmax_bf16",
     "tbik_gemm_bf16_static", "bi_log_softmax", "tbik_gemm_workspace_bytes_rowmajor_b", "tbik_gemm_plan_info",
     "bi_rmsnorm_gemm_bf16", "tbik_gemm_silu_mul_bf16", "bi_argmax_advance_bf16",
-    "tbik_gemm_rmsnorm_bf16", "tbik_tree_combine_rmsnorm_bf16", "bi_attention_decode_qkv_bf16",
+    "tbik_gemm_rmsnorm_bf16", "tbik_tree_combine_rmsnorm_bf16", "bi_attention_decode_qkv_bf16", "bi_gemm_silu_mul_bf16",
 )
 
 _lib = None
@@ -107,6 +107,8 @@ def lib() -> ctypes.CDLL:
     L.bi_argmax_advance_bf16.restype = i32
     L.bi_attention_decode_qkv_bf16.argtypes = [vp, i64, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, f32, f32, vp]
     L.bi_attention_decode_qkv_bf16.restype = i32
+    L.bi_gemm_silu_mul_bf16.argtypes = [vp, i64, vp, i64, vp, i64, i32, i32, i32, vp]
+    L.bi_gemm_silu_mul_bf16.restype = i32
     L.tbik_gemm_rmsnorm_bf16.argtypes = [vp, i64, vp, i64, i64, i32, i32, i32, i32, vp, vp, i64, vp, ctypes.c_float, vp, i64, vp, i64,
                                          vp, ctypes.c_size_t, vp]
     L.tbik_gemm_rmsnorm_bf16.restype = i32

@@ -35,6 +35,8 @@ int rmsnorm_gemm_dispatch(const void* x, int64_t ldx, const void* res, int64_t l
 int attention_decode_qkv_dispatch(const void* qkv, int64_t ld, const void* q_weight, const void* k_weight, const float* inv_freq,
                                   void* k_cache, void* vt_cache, void* out, const int* ctx_len, int batch, int q_heads,
                                   int kv_heads, int head_dim, int max_len, float scale, float eps, hipStream_t stream);
+int gemm_silu_mul_dispatch(const void* x, int64_t ldx, const void* W, int64_t ldw, void* out, int64_t ldo, int M, int inter, int K,
+                           hipStream_t stream);
 int gemm_tree_rmsnorm_dispatch(bool f16, const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, int M, int N,
                                int K, int leaf_k, const void* bias, const void* res, int64_t ldr, const void* norm_w, float eps,
                                void* res_out, int64_t ldro, void* out, int64_t ldo, void* ws, size_t ws_bytes,
@@ -48,7 +50,7 @@ int gemm_tree_gated_dispatch(const void* gate, const void* up, int64_t ld, const
 
 extern "C" {
 
-int tbik_abi_version(void) { return 16; }
+int tbik_abi_version(void) { return 17; }
 
 const char* tbik_error_string(int code) {
   switch (code) {
@@ -133,6 +135,11 @@ int tbik_gemm_silu_mul_bf16(const void* gate, const void* up, int64_t ld, const 
                             int64_t ldc, int M, int N, int K, int leaf_k, const void* bias_or_null, tbik_stream_t stream) {
   return tbik::gemm_tree_gated_dispatch(gate, up, ld, B, ldb_k, ldb_n, C, ldc, M, N, K, leaf_k, bias_or_null,
                                         static_cast<hipStream_t>(stream));
+}
+
+int bi_gemm_silu_mul_bf16(const void* x, int64_t ldx, const void* W, int64_t ldw, void* out, int64_t ldo, int M, int inter, int K,
+                          tbik_stream_t stream) {
+  return tbik::gemm_silu_mul_dispatch(x, ldx, W, ldw, out, ldo, M, inter, K, static_cast<hipStream_t>(stream));
 }
 
 int tbik_gemm_rmsnorm_bf16(const void* A, int64_t lda, const void* B, int64_t ldb_k, int64_t ldb_n, int M, int N, int K,

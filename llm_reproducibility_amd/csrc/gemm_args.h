@@ -68,8 +68,12 @@ struct StreamArgs {
   int64_t ldx, ldw, ldc;
   int M, N, K;
   int vec_store;
+  const uint16_t* W2 = nullptr;  // gated form only: the second weight matrix [N,K] (the `up` half of a merged projection)
 };
 int gemm_single_acc_stream_launch(const StreamArgs& a, bool f16, hipStream_t stream);
+// C[M,N] = silu(X W^T) * (X W2^T), both products rounded to the element type first (the bits of the mm followed by the
+// activation kernel), for the row counts of the windowed kernel; TBIK_ERR_UNSUPPORTED otherwise (nothing launched)
+int gemm_single_acc_stream_gated_launch(const StreamArgs& a, hipStream_t stream);
 // the same product with X = RMSNorm(a.X [+ res]) * w formed while the activations are staged (bf16, a few rows);
 // res_out receives the rounded sum a.X + res when res is given; TBIK_ERR_UNSUPPORTED: run the two launches
 struct StreamNormArgs {

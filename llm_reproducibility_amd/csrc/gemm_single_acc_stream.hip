@@ -15,6 +15,7 @@
 #include "common.h"
 #include "gemm_args.h"
 #include "rmsnorm_row.h"
+#include "silu_mul.h"
 
 namespace tbik {
 
@@ -42,6 +43,33 @@ __device__ __forceinline__ void stream_store(const StreamArgs& p, const f32x4* a
     if (m >= p.M) continue;
     const uint32_t lo = Num::pack(acc[b][0] + bv[0], acc[b][1] + bv[1]);
     const uint32_t hi = Num::pack(acc[b][2] + bv[2], acc[b][3] + bv[3]);
+    uint16_t* dst = p.C + (int64_t)m * p.ldc + n;
+    if (p.vec_store && n + 3 < p.N) {
+      *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);
+    } else {
+      const uint16_t v[4] = {(uint16_t)(lo & 0xffff), (uint16_t)(lo >> 16), (uint16_t)(hi & 0xffff), (uint16_t)(hi >> 16)};
+#pragma unroll
+      for (int e = 0; e < 4; e++)
+        if (n + e < p.N) dst[e] = v[e];
+    }
+  }
+}
+
+// Gated epilogue: gate and up are rounded to the element type exactly as stream_store rounds them (no bias), then
+// silu(gate) * up as the stand-alone activation kernel computes it (silu_mul.h).
+template <int MB, bool F16>
+__device__ __forceinline__ void stream_store_gated(const StreamArgs& p, const f32x4* gate, const f32x4* up, int n0, int r, int g) {
+  using Num = Num16<F16>;
+  const int n = n0 + 4 * g;
+  if (n >= p.N) return;
+  const float z = 0.f;  // the plain epilogue adds a zero bias in fp32: an accumulator of -0 becomes +0 there, so here too
+#pragma unroll
+  for (int b = 0; b < MB; b++) {
+    const int m = b * 16 + r;
+    if (m >= p.M) continue;
+    const uint32_t glo = Num::pack(gate[b][0] + z, gate[b][1] + z), ghi = Num::pack(gate[b][2] + z, gate[b][3] + z);
+    const uint32_t ulo = Num::pack(up[b][0] + z, up[b][1] + z), uhi = Num::pack(up[b][2] + z, up[b][3] + z);
+    const uint32_t lo = silu_mul_pair<F16>(glo, ulo), hi = silu_mul_pair<F16>(ghi, uhi);
     uint16_t* dst = p.C + (int64_t)m * p.ldc + n;
     if (p.vec_store && n + 3 < p.N) {
       *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);
@@ -155,7 +183,10 @@ __global__ __launch_bounds__(NWAVES * 64) void gemm_single_acc_stream_rows_kerne
   stream_store<1, F16>(p, acc, n0, r, g);
 }
 
-template <int MB, int WS, int NWAVES, bool F16>  // MB blocks of 16 activation rows, windows of WS steps (32 k each)
+// GATED: a wave owns strip n0 of BOTH weight matrices (gate and up of a merged projection) and runs the pass over K twice,
+// once per matrix (X is staged again: it comes from the L2), then stores silu(gate) * up: the consumer of the two products
+// inside their producer, one launch and a third of the output bytes.
+template <int MB, int WS, int NWAVES, bool F16, bool GATED = false>  // MB blocks of 16 activation rows, windows of WS steps (32 k each)
 __global__ __launch_bounds__(NWAVES * 64) void gemm_single_acc_stream_kernel(const StreamArgs p) {
   using namespace stream;
   using Num = Num16<F16>;
@@ -176,7 +207,7 @@ __global__ __launch_bounds__(NWAVES * 64) void gemm_single_acc_stream_kernel(con
   const int n0 = (xcd_contiguous_tile(blockIdx.x, gridDim.x) * NW + wave) * 16;
   const int r = lane & 15, g = lane >> 4;
 
-  const uint16_t* wp = p.W + (int64_t)min(n0 + r, p.N - 1) * p.ldw + 8 * g;
+  const uint16_t* wp = p.W + (int64_t)min(n0 + r, p.N - 1) * p.ldw + 8 * g;  // (the second pass of the gated form moves it)
 
   // staging of X: thread t moves 16-byte chunk q % (KW/8) of row q / (KW/8), q = t + NT i, i < XLD
   const uint16_t* xsrc[XLD];
@@ -226,6 +257,7 @@ __global__ __launch_bounds__(NWAVES * 64) void gemm_single_acc_stream_kernel(con
     }
   };
 
+  auto pass = [&]() __attribute__((always_inline)) {
   if (nfull > 0) {
     load_x(0);
     load_w(wa, 0);
@@ -261,16 +293,30 @@ __global__ __launch_bounds__(NWAVES * 64) void gemm_single_acc_stream_kernel(con
       acc[b] = Num::mfma(w, x, acc[b]);
     }
   }
-
-  stream_store<MB, F16>(p, acc, n0, r, g);
+  };
+  pass();
+  if constexpr (GATED) {
+    f32x4 gate[MB];
+#pragma unroll
+    for (int b = 0; b < MB; b++) {
+      gate[b] = acc[b];
+      acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    __syncthreads();  // every wave is through with the last window of X before it is staged again
+    wp = p.W2 + (int64_t)min(n0 + r, p.N - 1) * p.ldw + 8 * g;
+    pass();
+    stream_store_gated<MB, F16>(p, gate, acc, n0, r, g);
+  } else {
+    stream_store<MB, F16>(p, acc, n0, r, g);
+  }
 }
 
-template <int MB, int WS, int NWAVES, bool F16>
+template <int MB, int WS, int NWAVES, bool F16, bool GATED = false>
 static int stream_launch_nw(const StreamArgs& a, hipStream_t stream) {
   const int64_t groups = ((int64_t)a.N + 16 * NWAVES - 1) / (16 * NWAVES);
   if (groups > 0x7fffffff) return TBIK_ERR_INVALID;
   constexpr int smem = 2 * MB * 16 * stream::rowb(WS);
-  auto kern = gemm_single_acc_stream_kernel<MB, WS, NWAVES, F16>;
+  auto kern = gemm_single_acc_stream_kernel<MB, WS, NWAVES, F16, GATED>;
   if (smem > 64 * 1024) {
     static std::atomic<uint64_t> done{0};
     hipError_t e = ensure_dynamic_lds(reinterpret_cast<const void*>(kern), smem, done);
@@ -280,7 +326,7 @@ static int stream_launch_nw(const StreamArgs& a, hipStream_t stream) {
   return hip_code(hipGetLastError());
 }
 
-template <int MB, int WS, bool F16>
+template <int MB, int WS, bool F16, bool GATED = false>
 static int stream_launch(const StreamArgs& a, hipStream_t stream) {
   // Strips per work-group.  More strips share each staged window of X (gate_up of an 8B model at M=64: 80 us with four
   // strips per work-group, 55 us with eight), but HBM bandwidth is shared about equally among the CUs that ask for it,
@@ -291,7 +337,7 @@ static int stream_launch(const StreamArgs& a, hipStream_t stream) {
   // strips, ten rounds of groups of four) is within 2 % for three, four and six.
   const int64_t strips = ((int64_t)a.N + 15) / 16;
   // grids of many rounds do not run in rounds: the last one matters little there, the restaging of X more
-  if (strips > 4 * 1024) return MB >= 3 ? stream_launch_nw<MB, WS, 8, F16>(a, stream) : stream_launch_nw<MB, WS, 4, F16>(a, stream);
+  if (strips > 4 * 1024) return MB >= 3 ? stream_launch_nw<MB, WS, 8, F16, GATED>(a, stream) : stream_launch_nw<MB, WS, 4, F16, GATED>(a, stream);
   static const int cand[5] = {8, 6, 4, 3, 2};
   int best = 4;
   double best_cost = 0.0;
@@ -308,11 +354,11 @@ static int stream_launch(const StreamArgs& a, hipStream_t stream) {
     }
   }
   switch (best) {
-    case 8: return stream_launch_nw<MB, WS, 8, F16>(a, stream);
-    case 6: return stream_launch_nw<MB, WS, 6, F16>(a, stream);
-    case 3: return stream_launch_nw<MB, WS, 3, F16>(a, stream);
-    case 2: return stream_launch_nw<MB, WS, (MB <= 2 ? 2 : 4), F16>(a, stream);
-    default: return stream_launch_nw<MB, WS, 4, F16>(a, stream);
+    case 8: return stream_launch_nw<MB, WS, 8, F16, GATED>(a, stream);
+    case 6: return stream_launch_nw<MB, WS, 6, F16, GATED>(a, stream);
+    case 3: return stream_launch_nw<MB, WS, 3, F16, GATED>(a, stream);
+    case 2: return stream_launch_nw<MB, WS, (MB <= 2 ? 2 : 4), F16, GATED>(a, stream);
+    default: return stream_launch_nw<MB, WS, 4, F16, GATED>(a, stream);
   }
 }
 
@@ -387,6 +433,19 @@ int gemm_single_acc_stream_launch(const StreamArgs& a, bool f16, hipStream_t str
     case 2: return stream_launch<2, 16, false>(a, stream);
     case 3: return stream_launch<3, 16, false>(a, stream);
     default: return stream_launch<4, 16, false>(a, stream);
+  }
+}
+
+// The gated form: only the windowed kernel has it (5 .. 64 rows: fewer rows take the whole-X kernel, whose consumer, the
+// tree matmul of down_proj, forms the activation itself).
+int gemm_single_acc_stream_gated_launch(const StreamArgs& a, hipStream_t stream) {
+  if (a.M <= 0 || a.M > 64 || (a.K & 31) != 0 || a.K < 32 * 16 || !a.W2 || a.bias || (a.N & 15) != 0) return TBIK_ERR_UNSUPPORTED;
+  if (stream_rows_applies(a)) return TBIK_ERR_UNSUPPORTED;
+  switch ((a.M + 15) / 16) {
+    case 1: return stream_launch<1, 16, false, true>(a, stream);
+    case 2: return stream_launch<2, 16, false, true>(a, stream);
+    case 3: return stream_launch<3, 16, false, true>(a, stream);
+    default: return stream_launch<4, 16, false, true>(a, stream);
   }
 }
 

@@ -929,4 +929,21 @@ int gemm_tree_gated_dispatch(const void* gate, const void* up, int64_t ld, const
   return gemm_tree_strip_gated_launch(sa, leaf_k, waves, stream);
 }
 
+// The merged gate/up projection with the activation behind it in the same launch: out[M, inter] = silu(x Wg^T) * (x Wu^T),
+// W = [2*inter, K] (rows 0 .. inter-1 gate, the rest up; the nn.Linear layout), both products rounded to bf16 first.
+// TBIK_ERR_UNSUPPORTED (nothing launched) outside the row counts of the windowed streaming kernel.
+int gemm_silu_mul_dispatch(const void* x, int64_t ldx, const void* W, int64_t ldw, void* out, int64_t ldo, int M, int inter, int K,
+                           hipStream_t stream) {
+  if (M < 0 || inter <= 0 || K <= 0) return TBIK_ERR_INVALID;
+  if (M == 0) return TBIK_ERR_UNSUPPORTED;
+  if (!x || !W || !out) return TBIK_ERR_INVALID;
+  if (ldx < K || ldw < K || ldo < inter) return TBIK_ERR_INVALID;
+  if (!aligned16(x) || !aligned16(W) || (ldx & 7) || (ldw & 7) || (K & 7)) return TBIK_ERR_ALIGNMENT;
+  if (reinterpret_cast<uintptr_t>(out) & 1) return TBIK_ERR_ALIGNMENT;
+  StreamArgs sa{static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(W), static_cast<uint16_t*>(out), nullptr, ldx, ldw, ldo,
+                M, inter, K, ((reinterpret_cast<uintptr_t>(out) & 7) == 0 && (ldo & 3) == 0) ? 1 : 0,
+                static_cast<const uint16_t*>(W) + (int64_t)inter * ldw};
+  return gemm_single_acc_stream_gated_launch(sa, stream);
+}
+
 }  // namespace tbik

@@ -152,7 +152,7 @@ class Qwen3Decoder:
             elif self.fused_consumers:
                 # the add-RMSNorm behind each row-split layer runs in the launch that combines the layer's K shards
                 hp, residual = layer.o_proj.forward_add_norm(attn.reshape(-1, Hq * D), residual, layer.post_norm, cfg.rms_eps)
-                act = ops.bi_silu_mul(matmul_persistent(hp, layer.gate_up_w.t()))
+                act = ops.gemm_silu_mul(hp, layer.gate_up_w)     # the activation inside the projection for 5 .. 64 rows
                 if li + 1 < len(self.layers):
                     h, residual = layer.down_proj.forward_add_norm(act, residual, self.layers[li + 1].input_norm, cfg.rms_eps)
                 else:

@@ -524,6 +524,28 @@ def gemm_tree_silu_mul(gate: torch.Tensor, up: torch.Tensor, B: torch.Tensor, bi
     return gemm_tree(bi_silu_mul(merged), B, bias, leaf_k)
 
 
+def gemm_silu_mul(x: torch.Tensor, W: torch.Tensor) -> torch.Tensor:
+    """bi_silu_mul(bi_gemm(x, W.t())) for the merged gate/up weight W [2*inter, K] (nn.Linear layout): one launch
+    (`bi_gemm_silu_mul_bf16`) for 5 .. 64 bf16 rows, the two calls otherwise.  Same bits either way."""
+    _require_gpu(x, W)
+    M, K = x.shape
+    inter = W.shape[0] // 2
+    fusable = (x.dtype == torch.bfloat16 and W.dtype == torch.bfloat16 and 4 < M <= 64 and W.shape[0] == 2 * inter and inter % 16 == 0
+               and K % 32 == 0 and W.stride(1) == 1 and W.stride(0) % 8 == 0 and _aligned16(W) and not torch.compiler.is_compiling()
+               and ("mm_silu", M, inter, K) not in _declined)
+    if fusable:
+        x2, ldx = _rows16(x)
+        out = torch.empty((M, inter), device=x.device, dtype=x.dtype)
+        rc = _lib.lib().bi_gemm_silu_mul_bf16(x2.data_ptr(), ldx, W.data_ptr(), W.stride(0), out.data_ptr(), out.stride(0), M, inter, K,
+                                              _stream(x))
+        if rc == _lib.TBIK_OK:
+            return out
+        if rc != _lib.TBIK_ERR_UNSUPPORTED:
+            _lib.check(rc, "bi_gemm_silu_mul_bf16")
+        _declined.add(("mm_silu", M, inter, K))
+    return bi_silu_mul(bi_gemm(x, W.t(), None))
+
+
 # --------------------------------------------------------------------------------------------
 # the (add-)RMSNorm behind a row-split layer, inside the launch that combines the layer's K shards
 # --------------------------------------------------------------------------------------------

@@ -1,7 +1,8 @@
 """One-launch compositions for decode-sized batches against the two-launch forms they stand for (bit for bit) and
 against the CPU oracle: RMSNorm inside the batch-invariant mm (`bi_rmsnorm_gemm_bf16`), SiLU * up inside the tree
 matmul of down_proj (`tbik_gemm_silu_mul_bf16`), the add-RMSNorm behind a row-split layer inside the launch that combines
-the layer's K shards (`tbik_gemm_rmsnorm_bf16`, `tbik_tree_combine_rmsnorm_bf16`)."""
+the layer's K shards (`tbik_gemm_rmsnorm_bf16`, `tbik_tree_combine_rmsnorm_bf16`), SiLU * up inside the merged gate/up projection
+(`bi_gemm_silu_mul_bf16`)."""
 import pytest
 import torch
 
@@ -249,3 +250,52 @@ def test_decoder_with_and_without_fused_consumers_gives_the_same_bits(dev):
             b_ids, b_log = plain.generate(prompts[:batch], 6, return_logits=True)
             assert torch.equal(a_ids, b_ids) and torch.equal(a_log, b_log), (tp, batch)
         del fused, plain
+
+
+@pytest.mark.parametrize("M,K,inter", [(5, 4096, 12288), (16, 4096, 12288), (17, 4096, 12288), (32, 4096, 12288), (33, 4096, 12288),
+                                       (64, 4096, 12288), (40, 1024, 4096), (9, 5120, 3200), (48, 2048, 2064), (12, 8192, 1024)])
+def test_silu_mul_inside_the_merged_projection_equals_the_two_calls(dev, M, K, inter):
+    x = O.gaussian_bf16((M, K), 1.0, 80 + M).to(dev)
+    W = O.gaussian_bf16((2 * inter, K), 0.03, 81).to(dev)
+    print("case mm + silu_mul", M, K, inter, flush=True)
+    want = ops.bi_silu_mul(bio.matmul_persistent(x, W.t()))
+    out = torch.empty((M, inter), dtype=torch.bfloat16, device=dev)
+    s = torch.cuda.current_stream().cuda_stream
+    L = _lib.lib()
+    # the raw entry point takes the shape (so the wrapper below did not fall back to the two calls)
+    assert L.bi_gemm_silu_mul_bf16(x.data_ptr(), K, W.data_ptr(), K, out.data_ptr(), inter, M, inter, K, s) == _lib.TBIK_OK
+    assert torch.equal(out, want)
+    assert torch.equal(ops.gemm_silu_mul(x, W), want)
+    # activations and output as views with a row stride of their own
+    xp = torch.zeros((M, K + 64), dtype=torch.bfloat16, device=dev)
+    xp[:, :K] = x
+    op = torch.zeros((M, inter + 8), dtype=torch.bfloat16, device=dev)
+    assert L.bi_gemm_silu_mul_bf16(xp.data_ptr(), K + 64, W.data_ptr(), K, op.data_ptr(), inter + 8, M, inter, K, s) == _lib.TBIK_OK
+    assert torch.equal(op[:, :inter], want) and (op[:, inter:] == 0).all()
+    # every row alone gives the row of the batch (batch invariance of the fused form; a single row takes the two calls)
+    assert torch.equal(ops.gemm_silu_mul(x[M - 1:], W)[0], want[M - 1])
+    # and the oracle's activation of the kernel's own product (the product itself is oracle-checked elsewhere)
+    assert O.bf16_ulp_distance(out.cpu(), O.silu_mul(bio.matmul_persistent(x, W.t()).cpu())).max() <= 1
+
+
+def test_silu_mul_inside_the_merged_projection_declines_other_row_counts(dev):
+    W = O.gaussian_bf16((2 * 4096, 1024), 0.03, 82).to(dev)
+    s = torch.cuda.current_stream().cuda_stream
+    for M, inter in ((4, 4096), (1, 4096), (65, 4096), (300, 4096), (20, 4088)):     # few rows, many rows, a ragged strip
+        x = O.gaussian_bf16((M, 1024), 1.0, 83).to(dev)
+        out = torch.empty((M, inter), dtype=torch.bfloat16, device=dev)
+        assert _lib.lib().bi_gemm_silu_mul_bf16(x.data_ptr(), 1024, W.data_ptr(), 1024, out.data_ptr(), inter, M, inter, 1024, s) \
+            == _lib.TBIK_ERR_UNSUPPORTED, (M, inter)
+        if inter == 4096:
+            assert torch.equal(ops.gemm_silu_mul(x, W), ops.bi_silu_mul(bio.matmul_persistent(x, W.t())))
+
+
+def test_decoder_at_forty_sequences_with_and_without_fused_consumers_gives_the_same_bits(dev):
+    """40 rows per decode step: the add-RMSNorm inside the shard combines and SiLU * up inside the merged projection."""
+    g = torch.Generator().manual_seed(6)
+    prompts = [torch.randint(0, SMALL.vocab_size, (int(n),), generator=g).tolist() for n in torch.randint(3, 20, (40,), generator=g)]
+    fused = Qwen3Decoder(SMALL, tp_size=1, seed=0, device=dev, fused_consumers=True)
+    plain = Qwen3Decoder(SMALL, tp_size=1, seed=0, device=dev, fused_consumers=False, fused_attention_step=False)
+    a_ids, a_log = fused.generate(prompts, 5, return_logits=True)
+    b_ids, b_log = plain.generate(prompts, 5, return_logits=True)
+    assert torch.equal(a_ids, b_ids) and torch.equal(a_log, b_log)
