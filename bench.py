@@ -371,6 +371,13 @@ def table(steps, warmup, hot=False, settle_ms=20.0, full=False, only=None):
         add(f"  the same as separate calls (tree matmul, then add-RMSNorm) M={M}", make_tn,
             lambda x, r, W: bio.rms_norm(matmul_tp_persistent(x, W.t()), w, 1e-6, residual=r), 2.0 * M * 4096 * 12288, by, "hbm",
             short=f"tree, norm dn8B M={M}")
+    # ... and SiLU*up inside the merged gate/up projection (5 .. 64 rows), against the mm followed by the activation kernel
+    def make_gu():
+        return (torch.randn((32, 4096), device=dev).to(torch.bfloat16), (torch.randn((24576, 4096), device=dev) * 0.02).to(torch.bfloat16))
+    add("SiLU*up inside the merged gate/up projection 8B M=32 (one launch)", make_gu, lambda x, W: ops.gemm_silu_mul(x, W),
+        2.0 * 32 * 24576 * 4096, 2.0 * 24576 * 4096, "hbm", short="mm+silu gate_up M=32")
+    add("  the same as two calls (mm, then silu_mul) M=32", make_gu, lambda x, W: ops.bi_silu_mul(bio.matmul_persistent(x, W.t())),
+        2.0 * 32 * 24576 * 4096, 2.0 * 24576 * 4096, "hbm", short="mm, silu gate_up M=32")
     # fixed-order attention (Qwen3-8B heads: 32 query, 8 key/value, head_dim 128)
     Hq, Hkv, D = 32, 8, 128
 
