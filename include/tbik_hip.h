@@ -434,23 +434,6 @@ int tbik_gemm_silu_mul_bf16(const void* gate, const void* up, int64_t ld,
  *   hidden a multiple of 8 and <= 8192, everything 16-byte aligned.
  *   Replaces: tree_all_reduce_sum (src/tbik/tree_based_all_reduce.py:9-37) followed by that add-RMSNorm.
  */
-/*
- * bi_gemm_silu_mul_bf16:  out[M, inter] = bi_silu_mul_bf16( bi_gemm_bf16(x, W) )  for the merged gate/up projection
- *   W = [2*inter, K] K-contiguous (row stride ldw; rows 0 .. inter-1 gate, inter .. 2*inter-1 up), x [M,K] (row stride ldx):
- *   the wave that owns 16 columns of `gate` also owns the same 16 columns of `up`, runs the fixed-order pass over K once per
- *   matrix and stores silu(gate) * up -- the consumer inside the producer again.  Both products are rounded to bf16 before
- *   the activation, so the result is bit-identical to the two calls.  inter a multiple of 16, K a multiple of 32, no bias.
- *   Returns TBIK_ERR_UNSUPPORTED (3), with nothing launched, outside 5 .. 64 rows (fewer rows: the tree matmul of down_proj
- *   forms the activation itself, tbik_gemm_silu_mul_bf16; more: the tile kernels, which have no such epilogue): the caller
- *   then makes the two calls.
- *   Replaces: the merged column-parallel projection through aten::mm (src/bio/batch_invariant_ops.py:442-447) followed by
- *             SiluAndMul, in front of the patched down_proj (src/patch/patch_tp_invariant.py:10-48).
- */
-int bi_gemm_silu_mul_bf16(const void* x, int64_t ldx,
-                          const void* W, int64_t ldw,
-                          void* out, int64_t ldo,
-                          int M, int inter, int K,
-                          tbik_stream_t stream);
 int tbik_gemm_rmsnorm_bf16(const void* A, int64_t lda,
                            const void* B, int64_t ldb_k, int64_t ldb_n,
                            int M, int N, int K, int leaf_k,
@@ -469,6 +452,24 @@ int tbik_tree_combine_rmsnorm_bf16(const void* const* parts, int nparts,
                                    void* residual_out_or_null, int64_t ldro,
                                    void* out, int64_t ldo,
                                    tbik_stream_t stream);
+
+/*
+ * bi_gemm_silu_mul_bf16:  out[M, inter] = bi_silu_mul_bf16( bi_gemm_bf16(x, W) )  for the merged gate/up projection
+ *   W = [2*inter, K] K-contiguous (row stride ldw; rows 0 .. inter-1 gate, inter .. 2*inter-1 up), x [M,K] (row stride ldx):
+ *   the wave that owns 16 columns of `gate` also owns the same 16 columns of `up`, runs the fixed-order pass over K once per
+ *   matrix and stores silu(gate) * up -- the consumer inside the producer again.  Both products are rounded to bf16 before
+ *   the activation, so the result is bit-identical to the two calls.  inter a multiple of 16, K a multiple of 32, no bias.
+ *   Returns TBIK_ERR_UNSUPPORTED (3), with nothing launched, outside 5 .. 64 rows (fewer rows: the tree matmul of down_proj
+ *   forms the activation itself, tbik_gemm_silu_mul_bf16; more: the tile kernels, which have no such epilogue): the caller
+ *   then makes the two calls.
+ *   Replaces: the merged column-parallel projection through aten::mm (src/bio/batch_invariant_ops.py:442-447) followed by
+ *             SiluAndMul, in front of the patched down_proj (src/patch/patch_tp_invariant.py:10-48).
+ */
+int bi_gemm_silu_mul_bf16(const void* x, int64_t ldx,
+                          const void* W, int64_t ldw,
+                          void* out, int64_t ldo,
+                          int M, int inter, int K,
+                          tbik_stream_t stream);
 
 #ifdef __cplusplus
 }
