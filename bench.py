@@ -72,6 +72,36 @@ def hip_time_ms(fn, steps, warmup, settle_ms=0.0):
     return s.elapsed_time(e) / steps, wall_ms / steps
 
 
+def graph_time_ms(fn, calls, replays, settle_ms=0.0):
+    """Average milliseconds per call with the host out of the way: `calls` calls are recorded into one HIP graph and the
+    graph is replayed, so the kernels run back to back however long the Python operator around them takes (a decode
+    kernel of 20 us sits behind 15-40 us of host work per call when launched one by one).  None where the calls cannot
+    be recorded (an operator that synchronises); the caller then keeps its figure from one-by-one launches."""
+    import torch
+    try:
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for _ in range(calls):
+                fn()
+    except Exception:                                   # noqa: BLE001 -- any refusal to record means "measure eagerly"
+        torch.cuda.synchronize()
+        return None
+    t_end = time.perf_counter() + settle_ms * 1e-3
+    g.replay()
+    while time.perf_counter() < t_end:
+        g.replay()
+        torch.cuda.synchronize()
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s.record()
+    for _ in range(replays):
+        g.replay()
+    e.record()
+    torch.cuda.synchronize()
+    ms = s.elapsed_time(e) / (replays * calls)
+    del g
+    return ms
+
+
 class PowerSampler:
     """Board power while a loop runs, read from the driver's hwmon file (microwatts, `power1_input` or `power1_average`
     of the first GPU) every 20 ms on a thread of its own; `mean_w()` drops the first quarter of the samples (ramp-up).
@@ -231,11 +261,16 @@ def ceiling(settle_ms, others=()):
     return res
 
 
-def table(steps, warmup, hot=False, settle_ms=20.0, full=False, only=None):
+GRAPH_BELOW_MS = 0.15
+
+
+def table(steps, warmup, hot=False, settle_ms=20.0, full=False, only=None, graphs=True):
     """Per-shape figures, each after `settle_ms` of the same call run back to back (the settled rate, as for the
     headline).  Unless `hot`, every case cycles through enough distinct input sets (more than 768 MB in all) that
     nothing it reads is still in the 256 MB memory-side cache from the previous call: the GB/s are HBM figures, as in
-    a model whose every layer has its own weights.
+    a model whose every layer has its own weights.  With `graphs`, a case whose call takes less than 150 us is timed as
+    replays of a HIP graph of 32 such calls (`graph_time_ms`): the figure is then the kernels' own back-to-back time, not
+    the Python operator's host time, which is longer than many of these kernels.
 
     Returns a list of rows {case, us, flop, bytes, TFLOPs, GBps, bound, frac}: `flop` and `bytes` are the algorithmic
     work of one call -- 2*M*N*K and 2*(M*K + K*N + M*N) for a matmul, the formulas of the reference's launch metadata
@@ -260,17 +295,24 @@ def table(steps, warmup, hot=False, settle_ms=20.0, full=False, only=None):
             args = sets[state[0] % n]
             state[0] += 1
             return fn(*args)
-        return call
+        return call, n
 
     def add(name, make, fn, flop, nbytes, bound, nsteps=None, short=None):
         """`short`: the key of the row in the JSON line; rows without one appear in the long form only."""
         if (short is None and not full) or (only and only not in name):
             return
-        ms, _ = hip_time_ms(cycling(make, nbytes, fn), nsteps or steps, warmup, settle_ms)
+        call, nsets = cycling(make, nbytes, fn)
+        ms, _ = hip_time_ms(call, nsteps or steps, warmup, settle_ms)
+        how = "eager"
+        if graphs and ms < GRAPH_BELOW_MS:
+            per_graph = nsets * max(1, 32 // nsets)      # whole turns through the input sets: every replay stays cold
+            gms = graph_time_ms(call, per_graph, 3, settle_ms)
+            if gms is not None:
+                ms, how = gms, "graph"
         tf, gbs = flop / ms / 1e9, nbytes / ms / 1e6
         frac = tf / PEAK_BF16_TFLOPS if bound == "mfma" else gbs / PEAK_HBM_GBS
         rows.append({"case": name, "short": short, "us": round(ms * 1e3, 1), "flop": flop, "bytes": nbytes,
-                     "TFLOPs": round(tf, 1), "GBps": round(gbs, 1), "bound": bound, "frac": round(frac, 4)})
+                     "TFLOPs": round(tf, 1), "GBps": round(gbs, 1), "bound": bound, "frac": round(frac, 4), "timed": how})
 
     def operands(M, K, N):
         return lambda: (torch.randn((M, K), device=dev).to(torch.bfloat16), (torch.randn((N, K), device=dev) * 0.02).to(torch.bfloat16))
@@ -346,18 +388,18 @@ def table(steps, warmup, hot=False, settle_ms=20.0, full=False, only=None):
         add(f"  the same as two launches (rms_norm, then mm) M={M}", make_norm,
             lambda x, r, W: bio.matmul_persistent(bio.rms_norm(x, w, 1e-6, residual=r)[0], W.t()), 2.0 * M * 24576 * 4096, by, "hbm",
             short=f"norm, mm gate_up M={M}")
-
-        M = min(M, 3)   # 4 rows of 12288 activations are past what the one-launch kernel forms in every work-group
-
-        def make_gated(M=M):
-            return (torch.randn((M, 2 * 12288), device=dev).to(torch.bfloat16), (torch.randn((4096, 12288), device=dev) * 0.02).to(torch.bfloat16))
-        by = 2.0 * 4096 * 12288
-        add(f"SiLU*up inside the tree matmul, down_proj 8B M={M} (one launch)", make_gated,
-            lambda gu, W: ops.gemm_tree_silu_mul(gu[:, :12288], gu[:, 12288:], W.t(), None, 256), 2.0 * M * 4096 * 12288, by, "hbm",
-            short=f"silu+tree dn8B M={M}")
-        add(f"  the same as two launches (silu_mul, then tree matmul) M={M}", make_gated,
-            lambda gu, W: matmul_tp_persistent(ops.bi_silu_mul(gu), W.t()), 2.0 * M * 4096 * 12288, by, "hbm",
-            short=f"silu, tree dn8B M={M}")
+    # (every work-group of the one-launch kernel forms all M * K activations itself: it takes up to 16384 of them, so one row
+    # of the whole layer or four rows of a TP = 4 shard)
+    for M, K, tag in ((1, 12288, "dn8B"), (4, 3072, "dn8B/TP4")):
+        def make_gated(M=M, K=K):
+            return (torch.randn((M, 2 * K), device=dev).to(torch.bfloat16), (torch.randn((4096, K), device=dev) * 0.02).to(torch.bfloat16))
+        by = 2.0 * 4096 * K
+        add(f"SiLU*up inside the tree matmul, down_proj 8B M={M} K={K} (one launch)", make_gated,
+            lambda gu, W, K=K: ops.gemm_tree_silu_mul(gu[:, :K], gu[:, K:], W.t(), None, 256), 2.0 * M * 4096 * K, by, "hbm",
+            short=f"silu+tree {tag} M={M}")
+        add(f"  the same as two launches (silu_mul, then tree matmul) M={M} K={K}", make_gated,
+            lambda gu, W: matmul_tp_persistent(ops.bi_silu_mul(gu), W.t()), 2.0 * M * 4096 * K, by, "hbm",
+            short=f"silu, tree {tag} M={M}")
     # from five rows on the consumer runs inside the producer: the add-RMSNorm behind a row-split layer in the launch that
     # combines the layer's K shards, against the matmul followed by the norm (same bits)
     for M in (32, 128):
@@ -404,10 +446,10 @@ def table(steps, warmup, hot=False, settle_ms=20.0, full=False, only=None):
 def print_table(rows, hot):
     print("inputs " + ("reused by every call (hot in the memory-side cache)" if hot else
                        "cycled through more than 768 MB of distinct buffers (cold in the 256 MB memory-side cache)"), file=sys.stderr)
-    print(f"{'case':66s} {'us':>10s} {'TFLOP/s':>9s} {'%MFMA':>6s} {'GB/s':>9s} {'%HBM':>6s} {'bound':>6s}", file=sys.stderr)
+    print(f"{'case':66s} {'us':>10s} {'TFLOP/s':>9s} {'%MFMA':>6s} {'GB/s':>9s} {'%HBM':>6s} {'bound':>6s} {'timed':>6s}", file=sys.stderr)
     for r in rows:
         print(f"{r['case']:66s} {r['us']:10.1f} {r['TFLOPs']:9.1f} {100 * r['TFLOPs'] / PEAK_BF16_TFLOPS:6.1f} "
-              f"{r['GBps']:9.1f} {100 * r['GBps'] / PEAK_HBM_GBS:6.1f} {r['bound']:>6s}", file=sys.stderr)
+              f"{r['GBps']:9.1f} {100 * r['GBps'] / PEAK_HBM_GBS:6.1f} {r['bound']:>6s} {r['timed']:>6s}", file=sys.stderr)
 
 
 def decode_step(layers=12, prompt_len=512, batches=(1, 32, 128)):
@@ -451,6 +493,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--table", action="store_true", help="long form of the per-shape table, also printed to stderr")
     ap.add_argument("--table-hot", action="store_true", help="reuse one input set per table case (cache-hot figures)")
+    ap.add_argument("--eager-table", action="store_true",
+                    help="time every table case as one-by-one launches (no HIP-graph replays for the short ones)")
     ap.add_argument("--only", default=None, help="with --table: only the cases whose name contains this (for profiler runs)")
     ap.add_argument("--no-context-table", action="store_true", help="leave the per-shape table out of the JSON line")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -536,14 +580,18 @@ def main():
                                                           ("vendor_gemm_same_operands", lambda: torch.matmul(X, Wt))))
     if args.table or not args.no_context_table:
         t0 = time.perf_counter()
-        rows = table(12, 3, hot=args.table_hot, settle_ms=min(args.settle_ms, 10.0), full=args.table, only=args.only)
+        rows = table(12, 3, hot=args.table_hot, settle_ms=min(args.settle_ms, 10.0), full=args.table, only=args.only,
+                     graphs=not args.eager_table)
         if args.table:
             print_table(rows, args.table_hot)
         # terse in the JSON line: case -> [us per call, algorithmic work of a call (flop when the bound is "m", bytes when
         # it is "h"), achieved share of the bound's peak, bound]
         context["table"] = {r["short"]: [r["us"], int(float(f"{(r['flop'] if r['bound'] == 'mfma' else r['bytes']):.4g}")),
                                          round(r["frac"], 3), r["bound"][0]] for r in rows if r["short"]}
-        context["table_cols"] = ("[us per call (Python operator, HIP events, 12 calls after 10 ms of load, inputs "
+        context["table_cols"] = ("[us per call (HIP events after 10 ms of load; "
+                                 + ("12 calls of the Python operator" if args.eager_table else
+                                    f"calls under {GRAPH_BELOW_MS * 1e3:g} us: 3 replays of a HIP graph of 32 calls of the Python "
+                                    "operator, so no host time; longer ones: 12 calls one by one") + "; inputs "
                                  + ("reused" if args.table_hot else "cycled: cold") + "), algorithmic flop (m) or bytes (h), share of "
                                  f"{PEAK_BF16_TFLOPS:g} TFLOP/s (m) or {PEAK_HBM_GBS:g} GB/s (h), bound]; {time.perf_counter() - t0:.0f} s")
 

@@ -393,7 +393,7 @@ int bi_argmax_advance_bf16(const void* x, int64_t ld, void* next_token, int64_t 
  *   gate, up [M,K] with the same row stride ld (the two halves of the merged gate/up projection: up = gate + inter;
  *   a rank's K shard of both halves in a tensor-parallel run), K = the reduction extent of the row-split projection;
  *   B = [N,K] K-contiguous.  Applies where the one-launch few-rows tree kernel does and forming the activations in
- *   every work-group is cheaper than a launch of its own: M <= 4, M * K <= 40960, N <= 4096 (one work-group per CU).
+ *   every work-group is cheaper than a launch of its own: M <= 4, M * K <= 16384, N <= 4096 (one work-group per CU).
  *   Replaces: SiluAndMul followed by the patched RowParallelLinear forward of down_proj,
  *             src/patch/patch_tp_invariant.py:10-48 (the local matmul of :31).
  */

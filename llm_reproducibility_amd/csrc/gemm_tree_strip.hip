@@ -270,12 +270,13 @@ static int launch_strip_gated_s(const StripArgs& a, hipStream_t stream) {
 // Tree matmul of silu(gate) * up for a.X = gate, a.X2 = up ([M,K] each, row stride a.ldx), bf16: where the one-launch
 // kernel applies, the activations (M rows of 2K + 16 bytes) fit the LDS and forming them in every work-group is cheaper
 // than a launch of its own; 0 otherwise.  Every work-group evaluates all M * K activations, so the price grows with
-// M * K and with the number of work-groups: measured on MI355X against silu_mul + tree matmul, N = 4096 (one work-group
-// per CU), K = 12288: 21.8 / 24.2 / 26.6 / 29.4 us for 1 .. 4 rows against 25.9 / 26.9 / 27.2 / 26.8; K = 3072: 15 us
-// against 26 for 1 .. 4 rows; N = 5120 (320 work-groups), K = 12800: 52 - 53 us against 47.5 at any row count.
+// M * K and with the number of work-groups: measured on MI355X against silu_mul + tree matmul with the launches back to
+// back (replays of a recorded graph, cold weights), N = 4096 (one work-group per CU), K = 12288: 21.5 / 25.3 / 28.2 us
+// for 1 .. 3 rows against 22.6 / 24.3 / 24.9; K = 3072: 15 us against 26 for 1 .. 4 rows; N = 5120 (320 work-groups),
+// K = 12800: 52 - 53 us against 47.5 at any row count.  Hence at most 16384 activations per work-group.
 int gemm_tree_strip_gated_waves(int M, int N, int K, int lb) {
   if (M > 4 || (int64_t)M * (K * 2 + 16) > 128 * 1024) return 0;
-  if ((int64_t)M * K > 40960 || (N + 15) / 16 > 256) return 0;
+  if ((int64_t)M * K > 16384 || (N + 15) / 16 > 256) return 0;
   return gemm_tree_strip_waves(M, N, K, lb);
 }
 
