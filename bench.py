@@ -473,13 +473,19 @@ def decode_step(layers=12, prompt_len=512, batches=(1, 32, 128)):
         torch.cuda.synchronize()
         return time.perf_counter() - t
     for bs in batches:
-        run(bs, short)                                   # warm-up (first use of every kernel at this batch size)
-        a = min(run(bs, short) for _ in range(2))
-        b = min(run(bs, long_) for _ in range(2))
-        step_us = (b - a) / (long_ - short) * 1e6
-        out[f"batch_{bs}"] = {"us_per_step": round(step_us, 1), "us_per_layer": round(step_us / layers, 1)}
+        row = {}
+        for graphs, tag in ((False, ""), (True, "_graph")):
+            model.use_graphs = graphs                    # the step recorded once into a HIP graph and replayed
+            run(bs, short)                               # warm-up (first use of every kernel at this batch size)
+            a = min(run(bs, short) for _ in range(2))
+            b = min(run(bs, long_) for _ in range(2))
+            step_us = (b - a) / (long_ - short) * 1e6
+            row["us_per_step" + tag] = round(step_us, 1)
+            row["us_per_layer" + tag] = round(step_us / layers, 1)
+        out[f"batch_{bs}"] = row
     out["config"] = (f"{layers} layers of the 8B architecture (hidden 4096, 32/8 heads, intermediate 12288, vocabulary 151936), prompts of "
-                     f"{prompt_len} tokens, wall time between the steps {short} and {long_} of greedy decoding, host launches included; "
+                     f"{prompt_len} tokens, wall time between the steps {short} and {long_} of greedy decoding, launched call by call (host launches included) "
+                     f"and, _graph, as replays of the step recorded into one HIP graph; "
                      f"{time.perf_counter() - t0:.0f} s")
     del model
     torch.cuda.empty_cache()
