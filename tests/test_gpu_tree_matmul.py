@@ -636,3 +636,19 @@ def test_invariance_check_module_honours_the_flag(dev, monkeypatch):
     monkeypatch.setenv("TP_INVARIANT_MATMUL", "0")
     name, batch_diff, shard_diff = check_matmul.run(1024, 6144, 2048, 4)
     assert name == "torch.matmul" and batch_diff >= 0.0 and shard_diff >= 0.0
+
+
+def test_a_host_written_in_c_gets_the_same_properties_through_the_c_abi():
+    """tests/c_host/tbik_c_host.c: gcc, the header and the HIP runtime only.  It checks the product against a
+    double-precision one, four K shards + shard tree against the unsharded call and a row alone against the row in its
+    batch, the last two bitwise, and exits with 0 when all hold."""
+    import subprocess
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "c_host")
+    exe = os.path.join(here, "tbik_c_host")
+    if not os.path.exists(exe):
+        subprocess.run(["make", "-C", here], check=True, capture_output=True)
+    print("case C host", exe, flush=True)
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=100)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert r.stdout.strip().endswith("ok"), r.stdout
+    assert "4 K shards + shard tree have the bits of the unsharded call" in r.stdout

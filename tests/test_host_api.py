@@ -33,6 +33,25 @@ def test_library_exports_every_declared_symbol():
     assert b"leaves" in L.tbik_error_string(1)
 
 
+def test_header_is_plain_c_and_a_c_host_links_against_the_library(tmp_path):
+    """The boundary is a C ABI: the header compiles as strict C99 on its own, and a host written in C (tests/c_host) builds
+    with gcc against the library and the HIP runtime -- no C++, no Python in it."""
+    import shutil
+    import subprocess
+    gcc = shutil.which("gcc")
+    if not gcc:
+        pytest.skip("no gcc on this machine")
+    tu = tmp_path / "only_header.c"
+    tu.write_text('#include "tbik_hip.h"\n#include "tbik_measure.h"\nint main(void) { return (int)sizeof(tbik_stream_t) == 0; }\n')
+    r = subprocess.run([gcc, "-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror", "-fsyntax-only", "-I", os.path.join(ROOT, "include"), str(tu)],
+                       capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    _lib.lib()                                          # the library the host links against is built
+    r = subprocess.run(["make", "-B", "-C", os.path.join(ROOT, "tests", "c_host"), f"HOST_OUT={tmp_path / 'host'}"], capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert (tmp_path / "host").exists()
+
+
 def test_tree_params_through_the_c_abi():
     assert _lib.tree_params(12288, 256) == (48, 3, 5)
     assert _lib.tree_params(1536, 256) == (6, 3, 2)
