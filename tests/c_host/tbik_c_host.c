@@ -1,12 +1,13 @@
 /*
  * A host written in plain C against include/tbik_hip.h and the HIP runtime only (no Python, no torch): what a
  * maintainer of a C or cgo/JNI-style binding would write.  It checks, through the C ABI alone,
- *   1. the tree matmul of [M,K] x [K,N] against a double-precision product (within one rounding step of the
- *      output scale),
+ *   1. the tree matmul of [M,K] x [K,N] against a double-precision product (within 2^-6 of the output scale),
  *   2. that four K shards combined by tbik_tree_combine_bf16 give the bits of the unsharded call (the property
  *      simple_matmul.py:23-43 of the reference tests with `== 0.0`),
- *   3. that a row computed alone has the bits it has inside the batch (simple_matmul.py:16-20).
- * Exit status 0 when all three hold.  Built by tests/c_host/Makefile with gcc; run by the GPU test suite.
+ *   3. that a row computed alone has the bits it has inside the batch (simple_matmul.py:16-20),
+ *   4. that the entry point without a workspace (tbik_gemm_bf16_static, for callers that cannot allocate) gives the
+ *      bits of the one with a workspace.
+ * Exit status 0 when all four hold.  Built by tests/c_host/Makefile with gcc; run by the GPU test suite.
  */
 #include <hip/hip_runtime_api.h>
 #include <math.h>
@@ -63,7 +64,8 @@ int main(void) {
   uint16_t* C = (uint16_t*)malloc(c_bytes);
   uint16_t* C_tp = (uint16_t*)malloc(c_bytes);
   uint16_t* C_row = (uint16_t*)malloc((size_t)N * 2);
-  if (!A || !B || !C || !C_tp || !C_row) return 2;
+  uint16_t* C_static = (uint16_t*)malloc(c_bytes);
+  if (!A || !B || !C || !C_tp || !C_row || !C_static) return 2;
   for (size_t i = 0; i < (size_t)M * K; i++) A[i] = bf16_from_float(uniform_pm1());
   for (size_t i = 0; i < (size_t)N * K; i++) B[i] = bf16_from_float(0.05f * uniform_pm1());
 
@@ -101,6 +103,10 @@ int main(void) {
   /* 3. one row alone */
   CHECK_TBIK(tbik_gemm_bf16((const char*)dA + (size_t)ROW * K * 2, K, dB, 1, K, dRow, N, 1, N, K, LEAF, NULL, dWs, ws, stream));
   CHECK_HIP(hipStreamSynchronize(stream));
+  /* 4. the same product through the entry point that allocates nothing and takes no workspace (into shard buffer 1) */
+  CHECK_TBIK(tbik_gemm_bf16_static(dA, K, dB, 1, K, dParts[1], N, M, N, K, LEAF, NULL, stream));
+  CHECK_HIP(hipStreamSynchronize(stream));
+  CHECK_HIP(hipMemcpy(C_static, dParts[1], c_bytes, hipMemcpyDeviceToHost));
   CHECK_HIP(hipMemcpy(C, dC, c_bytes, hipMemcpyDeviceToHost));
   CHECK_HIP(hipMemcpy(C_tp, dParts[0], c_bytes, hipMemcpyDeviceToHost));
   CHECK_HIP(hipMemcpy(C_row, dRow, (size_t)N * 2, hipMemcpyDeviceToHost));
@@ -134,6 +140,9 @@ int main(void) {
   const int row_equal = memcmp(C + (size_t)ROW * N, C_row, (size_t)N * 2) == 0;
   printf("3. row %d alone %s the same row inside the batch of %d\n", ROW, row_equal ? "has the bits of" : "DIFFERS from", M);
   failures += !row_equal;
+  const int static_equal = memcmp(C, C_static, c_bytes) == 0;
+  printf("4. the entry point without a workspace %s the one with a workspace\n", static_equal ? "has the bits of" : "DIFFERS from");
+  failures += !static_equal;
 
   CHECK_HIP(hipStreamDestroy(stream));
   if (dWs) CHECK_HIP(hipFree(dWs));
@@ -143,6 +152,7 @@ int main(void) {
   CHECK_HIP(hipFree(dB));
   CHECK_HIP(hipFree(dA));
   free(exact);
+  free(C_static);
   free(C_row);
   free(C_tp);
   free(C);

@@ -640,8 +640,8 @@ def test_invariance_check_module_honours_the_flag(dev, monkeypatch):
 
 def test_a_host_written_in_c_gets_the_same_properties_through_the_c_abi():
     """tests/c_host/tbik_c_host.c: gcc, the header and the HIP runtime only.  It checks the product against a
-    double-precision one, four K shards + shard tree against the unsharded call and a row alone against the row in its
-    batch, the last two bitwise, and exits with 0 when all hold."""
+    double-precision one, four K shards + shard tree against the unsharded call, a row alone against the row in its
+    batch and the workspace-free entry point against the other, the last three bitwise, and exits with 0 when all hold."""
     import subprocess
     here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "c_host")
     exe = os.path.join(here, "tbik_c_host")
@@ -652,3 +652,4 @@ def test_a_host_written_in_c_gets_the_same_properties_through_the_c_abi():
     assert r.returncode == 0, r.stdout + r.stderr
     assert r.stdout.strip().endswith("ok"), r.stdout
     assert "4 K shards + shard tree have the bits of the unsharded call" in r.stdout
+    assert "without a workspace has the bits of" in r.stdout
