@@ -269,7 +269,7 @@ def table(steps, warmup, hot=False, settle_ms=20.0, full=False, only=None, graph
     headline).  Unless `hot`, every case cycles through enough distinct input sets (more than 768 MB in all) that
     nothing it reads is still in the 256 MB memory-side cache from the previous call: the GB/s are HBM figures, as in
     a model whose every layer has its own weights.  With `graphs`, a case whose call takes less than 150 us is timed as
-    replays of a HIP graph of 32 such calls (`graph_time_ms`): the figure is then the kernels' own back-to-back time, not
+    replays of a HIP graph of about 32 such calls (`graph_time_ms`): the figure is then the kernels' own back-to-back time, not
     the Python operator's host time, which is longer than many of these kernels.
 
     Returns a list of rows {case, us, flop, bytes, TFLOPs, GBps, bound, frac}: `flop` and `bytes` are the algorithmic
@@ -596,7 +596,7 @@ def main():
                                          round(r["frac"], 3), r["bound"][0]] for r in rows if r["short"]}
         context["table_cols"] = ("[us per call (HIP events after 10 ms of load; "
                                  + ("12 calls of the Python operator" if args.eager_table else
-                                    f"calls under {GRAPH_BELOW_MS * 1e3:g} us: 3 replays of a HIP graph of 32 calls of the Python "
+                                    f"calls under {GRAPH_BELOW_MS * 1e3:g} us: 3 replays of a HIP graph of about 32 calls (whole turns through the input sets) of the Python "
                                     "operator, so no host time; longer ones: 12 calls one by one") + "; inputs "
                                  + ("reused" if args.table_hot else "cycled: cold") + "), algorithmic flop (m) or bytes (h), share of "
                                  f"{PEAK_BF16_TFLOPS:g} TFLOP/s (m) or {PEAK_HBM_GBS:g} GB/s (h), bound]; {time.perf_counter() - t0:.0f} s")
