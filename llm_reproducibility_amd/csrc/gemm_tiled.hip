@@ -726,10 +726,19 @@ static int gemm_dispatch_impl(bool tree, bool f16, const void* A, int64_t lda, c
     const int64_t wide_tiles = (int64_t)((M + 127) / 128) * ((N + 255) / 256);
     // 33..128 rows: one row of 128-row tiles whose width balances the grid, when such a grid exists (same MFMA chain
     // per element again; measured faster than the streaming kernel from 33 rows on)
+    const bool narrow_n = N < 4096;   // no one-row grid of at least 128 tiles, whatever their width
     if (!f16 && M > 32 && M <= 128 && (K & 63) == 0 && lda < (1 << 22) && ldb_n < (1 << 22)) {
       QuadArgs qa{a.X, a.W, a.C, a.bias, a.ldx, a.ldw, a.ldc, M, N, K, a.vec_store};
-      const int rc = gemm_single_acc_slab_launch(qa, stream);
-      if (rc != TBIK_ERR_UNSUPPORTED) return rc;
+      if (!narrow_n) {
+        const int rc = gemm_single_acc_slab_launch(qa, stream);
+        if (rc != TBIK_ERR_UNSUPPORTED) return rc;
+      } else {
+        // a narrow weight matrix (a TP shard of a column-split layer): the width chosen by the cost model of the larger
+        // batches beats the streaming kernel (too few strips to fill the chip) and the tiled one from 33 rows on --
+        // [M,4096]x[4096,768] 25 -> 16 us at 33-48 rows, 41 -> 17-22 at 65-128; [M,6144]x[6144,2048] 37 -> 23 and
+        // 59 -> 26-34; [M,12288]x[12288,1536] 70 -> 42 and 115 -> 47-63 (up to 24 rows the streaming kernel still wins)
+        return gemm_single_acc_balanced_launch(qa, stream);
+      }
     }
     // more rows: the same pipeline with the tile width that spreads the grid over the chip (128x256 on large shapes)
     if (!f16 && M > 128 && (K & 63) == 0 && lda < (1 << 22) && ldb_n < (1 << 22)) {

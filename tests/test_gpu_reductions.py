@@ -256,6 +256,24 @@ def test_single_accumulator_mm_large_and_small_kernels_agree_bitwise(dev):
     assert torch.equal(bio.matmul_persistent(ai.to(dev), wi.to(dev).t()).cpu(), O.matmul_single_acc(ai, wi.t()))
 
 
+def test_single_accumulator_mm_on_narrow_weight_matrices_equals_its_small_pieces(dev):
+    """Fewer than 4096 weight rows (a TP shard of a column-split layer) at 33 .. 128 activation rows take the 128-row tiles
+    at the width a cost model picks: same bits as 16 rows at a time through the streaming kernels, ragged widths and a
+    bias included, and within the tolerance of the CPU oracle."""
+    for N, K in ((512, 4096), (768, 1024), (1000, 2048), (2048, 6144), (3072, 1024), (3584, 512)):
+        w = O.gaussian_bf16((N, K), 0.05, N + K).to(dev)
+        bias = O.gaussian_bf16((N,), 1.0, N).to(dev)
+        a = O.gaussian_bf16((128, K), 1.0, K).to(dev)
+        pieces = torch.cat([bio.matmul_persistent(a[r:r + 16], w.t(), bias) for r in range(0, 128, 16)])
+        for m in (33, 48, 64, 65, 100, 128):
+            print("case narrow mm", m, N, K, flush=True)
+            assert torch.equal(bio.matmul_persistent(a[:m], w.t(), bias), pieces[:m]), (m, N, K)
+        assert torch.equal(bio.matmul_persistent(a[:100], w.t()), torch.cat([bio.matmul_persistent(a[r:r + 4], w.t()) for r in range(0, 100, 4)]))
+    a = O.gaussian_bf16((100, 1024), 1.0, 3)
+    w = O.gaussian_bf16((768, 1024), 0.05, 4)
+    assert not O.outside_tolerance(bio.matmul_persistent(a.to(dev), w.to(dev).t()), O.matmul_single_acc(a, w.t())).any()
+
+
 def test_single_accumulator_mm_every_shape_of_a_sweep_equals_its_small_pieces(dev):
     """The mm picks among six kernel families and a dozen tile widths from measured cost models; none of it may change a
     bit.  Over a seeded sweep of shapes (rows 1 .. 4096, the projection widths of the 8B and 32B configurations and ragged
