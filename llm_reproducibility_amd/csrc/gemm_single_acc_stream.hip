@@ -410,10 +410,25 @@ int gemm_single_acc_stream_norm_launch(const StreamArgs& a, const StreamNormArgs
   return stream_rows_launch<4, false, 16>(a, stream, nrm);
 }
 
+// ... and is the faster of the two.  Every work-group of the whole-X kernel stages all of X before it streams, the
+// windowed kernel a window at a time behind its first weights.  Measured on MI355X (cold weights, launches back to back):
+// the whole-X kernel wins on wide weight matrices (gate_up, 24576 rows: 38.4 against 41.4 us at one row of 4096) and
+// while X is small; it loses from a few thousand elements of X on -- [4,4096] x [4096,6144] 16.7 against 13.0 us,
+// [2,8192] x [8192,5120] 29.2 against 22.8, [1,12288] x [12288,4096] 38.3 against 29.9, [8,2048] x [2048,4096] 10.1
+// against 7.2 -- the earlier the more strips there are.
+static bool stream_rows_pays(const StreamArgs& a) {
+#ifdef TBIK_STREAM_ROWS_ALWAYS
+  return true;
+#endif
+  const int64_t xe = (int64_t)a.M * a.K;
+  if (a.K < 512) return true;   // shorter than one window: nothing to stage behind
+  return a.N >= 10240 || xe <= 2048 || (xe <= 4096 && a.N <= 4096) || (xe <= 8192 && a.N <= 3072);
+}
+
 // Requires 0 < M <= 64 and K a multiple of 32 (checked by the dispatcher).
 int gemm_single_acc_stream_launch(const StreamArgs& a, bool f16, hipStream_t stream) {
   if (a.M <= 0 || a.M > 64 || (a.K & 31) != 0) return TBIK_ERR_UNSUPPORTED;
-  if (stream_rows_applies(a)) {
+  if (stream_rows_applies(a) && stream_rows_pays(a)) {
     const int nw = stream_rows_waves(a);
     if (nw == 1) return f16 ? stream_rows_launch<1, true>(a, stream) : stream_rows_launch<1, false>(a, stream);
     if (nw == 3) return f16 ? stream_rows_launch<3, true>(a, stream) : stream_rows_launch<3, false>(a, stream);
