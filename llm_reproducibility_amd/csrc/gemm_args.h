@@ -51,6 +51,7 @@ struct QuadArgs {
   int64_t ldx, ldw, ldc;
   int M, N, K;
   int vec_store;
+  int row_step = 0;    // rows a tile of gemm_single_acc_quad_kernel owns (0 = all 128; 64, 32 or 16: see the kernel)
 };
 int gemm_single_acc_quad_launch(const QuadArgs& a, hipStream_t stream);
 int gemm_single_acc_slab_launch(const QuadArgs& a, hipStream_t stream);  // at most 128 rows; TBIK_ERR_UNSUPPORTED: use another kernel

@@ -36,6 +36,9 @@ struct Shape {
 // NSLOT: slices of the ring.  Three keep a work-group fed when the chip is full of them; a grid of at most one narrow
 // tile per CU (a handful of rows times a moderate N) is a chain of slices, each waiting for loads issued NSLOT - 1
 // slices earlier, so those grids get a ring as deep as the LDS allows (5 or 6 slices).
+// p.row_step < 128: a tile owns only its first row_step rows (it still stages and multiplies 128, the rest clamped to its
+// last row and never stored).  For a grid that would leave most CUs without a tile: a work-group's time is its chain of
+// slices whatever the rows in its tile, so the same rows spread over two to eight times the work-groups finish sooner.
 template <int TN, int NSLOT>
 __global__ __launch_bounds__(quad::NT) void gemm_single_acc_quad_kernel(const QuadArgs p) {
   using namespace quad;
@@ -46,7 +49,8 @@ __global__ __launch_bounds__(quad::NT) void gemm_single_acc_quad_kernel(const Qu
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
 
-  const int tiles_m = (p.M + BM - 1) / BM;
+  const int row_step = p.row_step > 0 ? p.row_step : BM;
+  const int tiles_m = (p.M + row_step - 1) / row_step;
   const int tiles_n = (p.N + BN - 1) / BN;
   int lid = blockIdx.x;
   {
@@ -60,7 +64,8 @@ __global__ __launch_bounds__(quad::NT) void gemm_single_acc_quad_kernel(const Qu
   const int gsz = min(tiles_m - first_m, GROUP);
   const int pid_m = first_m + (lid % per_group) % gsz;
   const int pid_n = (lid % per_group) / gsz;
-  const int m0 = pid_m * BM, n0 = pid_n * BN;
+  const int m0 = pid_m * row_step, n0 = pid_n * BN;
+  const int m_end = min(p.M, m0 + row_step);
 
   const uint8_t* xbase = reinterpret_cast<const uint8_t*>(p.X + (int64_t)m0 * p.ldx);
   const uint8_t* wbase = reinterpret_cast<const uint8_t*>(p.W + (int64_t)n0 * p.ldw);
@@ -70,7 +75,7 @@ __global__ __launch_bounds__(quad::NT) void gemm_single_acc_quad_kernel(const Qu
 #pragma unroll
     for (int i = 0; i < NDMA; i++) {
       const int row = (i * NWAVE + wave) * 8 + r;  // 0..383: X rows, then W rows; rows past the edge are clamped
-      if (i < XDMA) voff[i] = (uint32_t)(((min(m0 + row, p.M - 1) - m0) * p.ldx + c * 8) * 2);
+      if (i < XDMA) voff[i] = (uint32_t)(((min(m0 + row, m_end - 1) - m0) * p.ldx + c * 8) * 2);
       else voff[i] = (uint32_t)(((min(n0 + row - BM, p.N - 1) - n0) * p.ldw + c * 8) * 2);
     }
   }
@@ -166,7 +171,7 @@ __global__ __launch_bounds__(quad::NT) void gemm_single_acc_quad_kernel(const Qu
 #pragma unroll
     for (int b = 0; b < TN; b++) {
       const int n = n0 + (wn * TN + b) * 16 + fchk * 4;
-      if (m >= p.M || n >= p.N) continue;
+      if (m >= m_end || n >= p.N) continue;
       float bv[4] = {0.f, 0.f, 0.f, 0.f};
       if (p.bias) {
 #pragma unroll
@@ -194,7 +199,9 @@ static int quad_launch(const QuadArgs& a, hipStream_t stream) {
   constexpr int BN = Shape<TN>::BN;
   constexpr size_t smem = (size_t)NSLOT * Shape<TN>::STAGE_BYTES;  // 144 KiB for the 256-wide tile
   static_assert(smem <= 160 * 1024 && (NSLOT - 1) * Shape<TN>::NDMA < 64, "ring does not fit the LDS or the wait counter");
-  const int64_t tiles = (int64_t)((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN);
+  const int row_step = a.row_step > 0 ? a.row_step : BM;
+  if (row_step > BM || (row_step & 15)) return TBIK_ERR_INVALID;
+  const int64_t tiles = (int64_t)((a.M + row_step - 1) / row_step) * ((a.N + BN - 1) / BN);
   if (tiles <= 0 || tiles > 0x7fffffff || a.K < BK || (a.K % BK) != 0) return TBIK_ERR_UNSUPPORTED;
   if (a.ldx >= (1 << 22) || a.ldw >= (1 << 22)) return TBIK_ERR_UNSUPPORTED;  // 32-bit in-tile byte offsets
   static std::atomic<uint64_t> done{0};
@@ -205,6 +212,21 @@ static int quad_launch(const QuadArgs& a, hipStream_t stream) {
 }
 
 int gemm_single_acc_quad_launch(const QuadArgs& a, hipStream_t stream) { return quad_launch<8>(a, stream); }
+
+// Rows per tile for a grid of one row of tiles that leaves CUs idle: the smallest step, down to 32 rows, that still fits
+// the grid into one work-group per CU (see the kernel); 0 = no split.  Measured on MI355X (cold weights, launches back to
+// back): [128,4096] x [4096,4096] 22.6 -> 17.8 us, [128,8192] x [8192,2048] 38.1 -> 29.6, [96,12288] x [12288,3072]
+// 60.2 -> 44.1, [64,12288] x [12288,2048] 47.3 -> 42.3.  Below 64 rows the second tile re-reads the weights for a
+// handful of rows and the split loses (33 rows: 30.3 -> 32.9), and steps of 16 are no better than 32.
+static int quad_row_step(int M, int64_t tiles_n) {
+  if (M < 64) return 0;
+  int best = 0;
+  for (int step = quad::BM / 2; step >= 32; step /= 2) {
+    const int64_t tm = ((int64_t)M + step - 1) / step;
+    if (tm >= 2 && tiles_n * tm <= 256) best = step;
+  }
+  return best;
+}
 
 // 33..128 rows: one row of tiles, so the call is one pass over the weights.  A work-group's time is set by the
 // length of K (the ring is a chain of slices, each about a memory round trip), not by the width of its tile, so the
@@ -230,11 +252,13 @@ int gemm_single_acc_slab_launch(const QuadArgs& a, hipStream_t stream) {
   // at most one work-group per CU: the deep ring (see the kernel); qkv [M,4096]x[4096,6144] at M=40 27 -> 18 us, at
   // M=128 28 -> 24; [M,12288]x[12288,4096] at M=64 72 -> 49 (an eight-slice ring was measured too: no further gain)
   const bool deep = (((int64_t)a.N + 32 * best - 1) / (32 * (best ? best : 1))) <= 256;
+  QuadArgs b = a;
+  if (best) b.row_step = quad_row_step(a.M, ((int64_t)a.N + 32 * best - 1) / (32 * best));
   switch (best) {
-    case 4: return deep ? quad_launch<4, 5>(a, stream) : quad_launch<4>(a, stream);
-    case 3: return deep ? quad_launch<3, 5>(a, stream) : quad_launch<3>(a, stream);
-    case 2: return deep ? quad_launch<2, 6>(a, stream) : quad_launch<2>(a, stream);
-    case 1: return deep ? quad_launch<1, 6>(a, stream) : quad_launch<1>(a, stream);
+    case 4: return deep ? quad_launch<4, 5>(b, stream) : quad_launch<4>(b, stream);
+    case 3: return deep ? quad_launch<3, 5>(b, stream) : quad_launch<3>(b, stream);
+    case 2: return deep ? quad_launch<2, 6>(b, stream) : quad_launch<2>(b, stream);
+    case 1: return deep ? quad_launch<1, 6>(b, stream) : quad_launch<1>(b, stream);
     default: return TBIK_ERR_UNSUPPORTED;
   }
 }
@@ -321,6 +345,16 @@ int gemm_single_acc_balanced_launch(const QuadArgs& a, hipStream_t stream) {
   // at most one narrow tile per CU: the deep ring (see the kernel); qkv at M=160 31 -> 25 us, [M,12288]x[12288,4096]
   // at M=192 73 -> 51
   const bool deep = tm * (((int64_t)a.N + 32 * best - 1) / (32 * best)) <= 256;
+  if (tm == 1 && best <= 4) {
+    QuadArgs b = a;
+    b.row_step = quad_row_step(a.M, ((int64_t)a.N + 32 * best - 1) / (32 * best));
+    switch (best) {
+      case 4: return quad_launch<4, 5>(b, stream);
+      case 3: return quad_launch<3, 5>(b, stream);
+      case 2: return quad_launch<2, 6>(b, stream);
+      default: return quad_launch<1, 6>(b, stream);
+    }
+  }
   switch (best) {
     case 8: return quad_launch<8>(a, stream);
     case 6: return quad_launch<6>(a, stream);

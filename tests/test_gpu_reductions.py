@@ -258,9 +258,10 @@ def test_single_accumulator_mm_large_and_small_kernels_agree_bitwise(dev):
 
 def test_single_accumulator_mm_on_narrow_weight_matrices_equals_its_small_pieces(dev):
     """Fewer than 4096 weight rows (a TP shard of a column-split layer) at 33 .. 128 activation rows take the 128-row tiles
-    at the width a cost model picks: same bits as 16 rows at a time through the streaming kernels, ragged widths and a
-    bias included, and within the tolerance of the CPU oracle."""
-    for N, K in ((512, 4096), (768, 1024), (1000, 2048), (2048, 6144), (3072, 1024), (3584, 512)):
+    at the width a cost model picks, and from 64 rows on a grid of at most 128 such tiles (4096 weight rows included) is
+    cut into tiles that own 64 or 32 of their rows: same bits as 16 rows at a time through the streaming kernels, ragged
+    widths and a bias included, and within the tolerance of the CPU oracle."""
+    for N, K in ((512, 4096), (768, 1024), (1000, 2048), (2048, 6144), (3072, 1024), (3584, 512), (4096, 1024)):
         w = O.gaussian_bf16((N, K), 0.05, N + K).to(dev)
         bias = O.gaussian_bf16((N,), 1.0, N).to(dev)
         a = O.gaussian_bf16((128, K), 1.0, K).to(dev)
