@@ -488,7 +488,10 @@ static bool make_plan(int M, int N, int K, int leaf_k, bool f16, Plan* pl, bool 
   bool wide = false;
   if (M >= 64 && !rowmajor_b) {  // the wide kernels exist for [N,K] weights only
     wide_cost_us(M, N, K, leaf_k, f16, flb, lb, &split);
-    wide = wide_tiles * split >= 64;
+    // exactly 64 rows fit one 64-row tile of the tiled kernel, which half-empty 128-row tiles only beat on a grid that
+    // fills most of the chip: [64,25600] x [25600,4096] 66 us on 128 work-groups of the wide kernel, 51 on the tiled one;
+    // [64,16384] x [16384,8192] 75 on 256 against 97
+    wide = wide_tiles * split >= (M == 64 ? 160 : 64);
   }
   if (!wide) {
     const int bm = M <= 16 ? 16 : ((M <= 64 || rowmajor_b) ? 64 : 128), bn = M <= 16 ? 64 : 128;
@@ -528,6 +531,10 @@ struct NarrowPlan {
 static bool narrow_plan(int M, int N, int K, int leaf_k, bool f16, NarrowPlan* np) {
   int T, flb, level_k;
   if (f16 || leaf_k != 256 || M < 64 || M > 512 || tbik_tree_params(K, leaf_k, &T, &flb, &level_k) != TBIK_OK) return false;
+  // exactly 64 rows: the 64-row tiles of the tiled kernel cut K at most eightfold, which fills the chip from 32 column
+  // tiles on and then beats 128-row tiles that are half empty ([64,8192] x [8192,4096] 25.6 -> 21.1 us, [64,4096] x
+  // [4096,4096] 14.7 -> 13.5); narrower matrices need the deeper cut of this plan (N = 2048: 15.5 against 16.8)
+  if (M == 64 && N >= 4096) return false;
   const int lb = level_k - 1;
   const int64_t tiles = (((int64_t)N + 127) / 128) * ((M + 127) / 128);
   int best = 0, best_ls = 0;
