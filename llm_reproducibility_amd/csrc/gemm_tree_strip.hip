@@ -235,6 +235,10 @@ int gemm_tree_strip_waves(int M, int N, int K, int lb) {
   if ((int64_t)N * K > 150000000) return 0;
   const int64_t strips = ((int64_t)N + 15) / 16;
   if (strips < 64) return 0;
+  // half the chip or less, and a long K: the K-cut grid of the tiled kernel spreads the same weights over all CUs
+  // ([1,8192] x [8192,1024] 13.1 us here, 9.4 there; [4,25600] x [25600,2048] 38.8 against 31.8; up to K = 3072 this
+  // kernel is still ahead, 6.5 against 7.5 at N = 2048)
+  if (strips <= 128 && K >= 4096) return 0;
   const int64_t rounds = (strips + 255) / 256;
   if (strips > 256 && rounds * 256 * 100 > strips * 115) return 0;
   if (lb == 1) return 2;
